@@ -1,0 +1,258 @@
+"""Pins the float half of the CPU oracle (KDE, basis projection, their
+gradients, sampling, pooling, layer composition) against library routines,
+closed forms, autograd of float64 restatements and known-answer tests.  No GPU."""
+import numpy as np
+import pytest
+import torch
+from sklearn.neighbors import KernelDensity
+
+
+def _grid_nbh(oracle, rng, batch, n, d, cell, centres=None):
+    pts = rng.random((n, d)).astype(np.float32)
+    bids = np.repeat(np.arange(batch), n // batch).astype(np.int32)
+    g = oracle.Grid(pts, bids, batch, cell)
+    if centres is None:
+        return g, oracle.Neighborhood(g, cell)
+    return g, oracle.Neighborhood(g, cell, *centres)
+
+
+@pytest.mark.parametrize("d,cell", [(2, 0.7), (2, 1.5), (3, 0.7), (3, 1.8), (4, 2.0)])
+def test_pdf_matches_sklearn_kde(oracle, d, cell):
+    """compute_pdf_test.py:76-108: pdf / N equals sklearn's Gaussian KDE of the
+    cloud scaled by 1/cell (bandwidth 0.1 makes the truncation at the radius
+    immaterial: the dropped tail is below exp(-50))."""
+    rng = np.random.default_rng(20 + d)
+    batch, n, bw = 4, 400, 0.1
+    g, nbh = _grid_nbh(oracle, rng, batch, n, d, cell)
+    inv_bw = np.full(d, 1.0 / np.float32(bw), dtype=np.float32)
+    pdf = oracle.compute_pdf(g.sorted_points, nbh.neighbors, nbh.ranges, inv_bw,
+                             nbh.inv_radii, 0)
+    for b in range(batch):
+        sel = g.sorted_batch_ids == b
+        x = g.sorted_points[sel].astype(np.float64) / cell
+        kde = KernelDensity(bandwidth=bw).fit(x)
+        expect = np.exp(kde.score_samples(x))
+        np.testing.assert_allclose(pdf[sel] / sel.sum(), expect, rtol=2e-5)
+
+
+def test_pdf_two_point_closed_form(oracle):
+    pts = np.array([[0.0, 0.0, 0.0], [0.03, -0.04, 0.12]], dtype=np.float32)
+    nbrs = np.array([[0, 0], [1, 0], [0, 1], [1, 1]], dtype=np.int32)
+    ranges = np.array([2, 4], dtype=np.int32)
+    bw, r = np.float32(0.25), np.float32(0.2)
+    pdf = oracle.compute_pdf(pts, nbrs, ranges, [1 / bw] * 3, [1 / r] * 3, 0)
+    u = (pts[1].astype(np.float64) - pts[0]) / (float(bw) * float(r))
+    one = (1 / float(bw) / np.sqrt(2 * np.pi)) ** 3
+    expect = one * (1 + np.exp(-0.5 * (u ** 2).sum()))
+    np.testing.assert_allclose(pdf, [expect, expect], rtol=1e-6)
+
+
+def _kde_torch(pts, nbrs, n, inv_bw, inv_r):
+    scale = torch.tensor(inv_bw.astype(np.float64) * inv_r.astype(np.float64))
+    bwt = torch.tensor(inv_bw.astype(np.float64))
+    u = (pts[nbrs[:, 0]] - pts[nbrs[:, 1]]) * scale
+    val = torch.prod(bwt * torch.exp(-0.5 * u * u) / np.sqrt(2 * np.pi), dim=1)
+    return torch.zeros(n, dtype=torch.float64).index_add(0, torch.tensor(nbrs[:, 1]).long(), val)
+
+
+@pytest.mark.parametrize("d", [2, 3, 4])
+def test_pdf_grads_match_autograd_and_differences(oracle, d):
+    rng = np.random.default_rng(40 + d)
+    g, nbh = _grid_nbh(oracle, rng, 2, 300, d, 0.4)
+    inv_bw = np.full(d, 1 / np.float32(0.3), dtype=np.float32)
+    up = rng.standard_normal(len(g.sorted_points)).astype(np.float32)
+    got = oracle.compute_pdf_pt_grads(g.sorted_points, nbh.neighbors, nbh.ranges, inv_bw,
+                                      nbh.inv_radii, up, 0)
+    pts = torch.tensor(g.sorted_points.astype(np.float64), requires_grad=True)
+    pdf = _kde_torch(pts, nbh.neighbors, len(pts), inv_bw, nbh.inv_radii)
+    (pdf * torch.tensor(up.astype(np.float64))).sum().backward()
+    np.testing.assert_allclose(got, pts.grad.numpy(), rtol=1e-9, atol=1e-9)
+    # central difference on a few coordinates (neighbour lists held fixed)
+    base = g.sorted_points.astype(np.float64)
+    for (i, k) in [(0, 0), (17, d - 1), (123, 1)]:
+        h = 1e-4
+        vals = []
+        for s in (+1, -1):
+            p = base.copy()
+            p[i, k] += s * h
+            with torch.no_grad():
+                v = _kde_torch(torch.tensor(p), nbh.neighbors, len(p), inv_bw, nbh.inv_radii)
+            vals.append(float((v * torch.tensor(up.astype(np.float64))).sum()))
+        np.testing.assert_allclose(got[i, k], (vals[0] - vals[1]) / (2 * h), rtol=1e-4,
+                                   atol=1e-5)
+
+
+def test_pdf_mode1_uses_sqrt_of_point_count(oracle):
+    """compute_pdf_kernels.cu.cc:56,102: mode 1 replaces the inverse bandwidth by
+    sqrt(number of points)."""
+    rng = np.random.default_rng(2)
+    g, nbh = _grid_nbh(oracle, rng, 1, 100, 3, 0.5)
+    a = oracle.compute_pdf(g.sorted_points, nbh.neighbors, nbh.ranges, [123.0] * 3,
+                           nbh.inv_radii, 1)
+    b = oracle.compute_pdf(g.sorted_points, nbh.neighbors, nbh.ranges, [10.0] * 3,
+                           nbh.inv_radii, 0)
+    np.testing.assert_allclose(a, b, rtol=1e-12)
+
+
+@pytest.mark.parametrize("c,k", [(1, 8), (3, 16), (8, 8), (16, 32), (24, 64)])
+def test_basis_proj_matches_segment_sum(oracle, c, k):
+    """basis_proj_test.py:88-111: per centre the sum over its neighbours of
+    feature (outer) basis."""
+    rng = np.random.default_rng(60 + c + k)
+    g, nbh = _grid_nbh(oracle, rng, 2, 400, 3, 0.25,
+                       centres=(rng.random((90, 3)).astype(np.float32),
+                                np.repeat([0, 1], 45).astype(np.int32)))
+    m = len(nbh.neighbors)
+    basis = rng.random((m, k)).astype(np.float32)
+    feat = rng.standard_normal((400, c)).astype(np.float32)
+    ids = nbh.original_neigh_ids
+    out, mag = oracle.basis_proj(basis, feat, ids, nbh.ranges, with_magnitude=True)
+    per_pair = feat[ids[:, 0]].astype(np.float64)[:, :, None] * \
+        basis.astype(np.float64)[:, None, :]
+    expect = np.zeros((90, c, k))
+    np.add.at(expect, ids[:, 1], per_pair)
+    np.testing.assert_allclose(out, expect, rtol=1e-12, atol=1e-12)
+    emag = np.zeros((90, c, k))
+    np.add.at(emag, ids[:, 1], np.abs(per_pair))
+    np.testing.assert_allclose(mag, emag, rtol=1e-12, atol=1e-12)
+    f32 = oracle.basis_proj_f32(basis, feat, ids, nbh.ranges)
+    assert np.all(np.abs(f32 - expect) <= 1e-5 * emag + 1e-30)
+
+
+@pytest.mark.parametrize("c,k", [(3, 8), (16, 16), (8, 32)])
+def test_basis_proj_grads_match_autograd(oracle, c, k):
+    rng = np.random.default_rng(80 + c + k)
+    g, nbh = _grid_nbh(oracle, rng, 2, 300, 3, 0.3)
+    ids = nbh.original_neigh_ids
+    m = len(ids)
+    basis = rng.random((m, k)).astype(np.float32)
+    feat = rng.standard_normal((300, c)).astype(np.float32)
+    up = rng.standard_normal((300, c, k)).astype(np.float32)
+    db, df = oracle.basis_proj_grads(basis, feat, ids, nbh.ranges, up)
+    tb = torch.tensor(basis.astype(np.float64), requires_grad=True)
+    tf_ = torch.tensor(feat.astype(np.float64), requires_grad=True)
+    per_pair = tf_[torch.tensor(ids[:, 0]).long()][:, :, None] * tb[:, None, :]
+    out = torch.zeros(300, c, k, dtype=torch.float64).index_add(
+        0, torch.tensor(ids[:, 1]).long(), per_pair)
+    (out * torch.tensor(up.astype(np.float64))).sum().backward()
+    np.testing.assert_allclose(db, tb.grad.numpy(), rtol=1e-10, atol=1e-10)
+    np.testing.assert_allclose(df, tf_.grad.numpy(), rtol=1e-10, atol=1e-10)
+    # adjoint identity <up, proj(basis, feat)> == <dbasis, basis> == <dfeat, feat>
+    fwd = oracle.basis_proj(basis, feat, ids, nbh.ranges)
+    lhs = float((fwd * up).sum())
+    np.testing.assert_allclose(float((db * basis).sum()), lhs, rtol=1e-9)
+    np.testing.assert_allclose(float((df * feat).sum()), lhs, rtol=1e-9)
+    db32, df32 = oracle.basis_proj_grads_f32(basis, feat, ids, nbh.ranges, up)
+    np.testing.assert_allclose(db32, db, rtol=1e-4, atol=1e-4)
+    np.testing.assert_allclose(df32, df, rtol=1e-4, atol=1e-3)
+
+
+@pytest.mark.parametrize("n_sqrt,scale", [(6, 1), (100, 5)])
+def test_poisson_collinear_known_answer(oracle, n_sqrt, scale):
+    """sample_test.py:61-78: the reference passes an [n, n, 2] array, i.e. n clouds
+    of n collinear points each (spacing scale/(n-1)); with radius 2*scale/n only
+    adjacent points are neighbours, so every second point of each line survives:
+    n*n // 2 in total."""
+    t = np.linspace(0, scale, num=n_sqrt)
+    pts = np.array(np.meshgrid(t, t)).T.reshape(-1, 2).astype(np.float32)
+    bids = np.repeat(np.arange(n_sqrt), n_sqrt).astype(np.int32)
+    cell = (scale * np.array([2, 2], dtype=np.float32) / n_sqrt).astype(np.float32)
+    g = oracle.Grid(pts, bids, n_sqrt, cell)
+    nbh = oracle.Neighborhood(g, cell)
+    spts, sb, sidx = oracle.sampling(g.sorted_points, g.sorted_batch_ids, g.sorted_keys,
+                                     g.num_cells, nbh.neighbors, nbh.ranges, 0)
+    assert len(spts) == n_sqrt ** 2 // 2
+    assert np.array_equal(spts, g.sorted_points[sidx])
+
+
+@pytest.mark.parametrize("d,batch", [(2, 1), (3, 4), (4, 3)])
+def test_poisson_invariants(oracle, d, batch):
+    rng = np.random.default_rng(30 + d)
+    cell = {2: 0.05, 3: 0.12, 4: 0.25}[d]
+    g, nbh = _grid_nbh(oracle, rng, batch, 600 * batch, d, cell)
+    spts, sb, sidx = oracle.sampling(g.sorted_points, g.sorted_batch_ids, g.sorted_keys,
+                                     g.num_cells, nbh.neighbors, nbh.ranges, 0)
+    assert np.all(np.diff(sidx) > 0)
+    chosen = np.zeros(len(g.sorted_points), bool)
+    chosen[sidx] = True
+    starts = oracle.segment_starts(nbh.ranges)
+    for i in range(len(chosen)):
+        others = nbh.neighbors[starts[i]:nbh.ranges[i], 0]
+        others = others[others != i]
+        if chosen[i]:
+            assert not chosen[others].any()          # separation
+        else:
+            assert chosen[others].any()              # maximality
+
+
+@pytest.mark.parametrize("cell", [0.1, 0.7, np.sqrt(3)])
+def test_cell_average_matches_numpy_loop(oracle, cell):
+    """sample_test.py:101-125."""
+    rng = np.random.default_rng(12)
+    g, nbh = _grid_nbh(oracle, rng, 2, 200, 3, np.float32(cell))
+    spts, sb, first = oracle.sampling(g.sorted_points, g.sorted_batch_ids, g.sorted_keys,
+                                      g.num_cells, nbh.neighbors, nbh.ranges, 1)
+    uk, start, cnt = np.unique(-g.sorted_keys, return_index=True, return_counts=True)
+    assert np.array_equal(first, start)
+    for u in range(len(uk)):
+        seg = g.sorted_points[start[u]:start[u] + cnt[u]].astype(np.float64)
+        np.testing.assert_allclose(spts[u], seg.mean(axis=0), rtol=1e-5, atol=1e-7)
+        assert sb[u] == g.sorted_batch_ids[start[u]]
+
+
+def test_sampling_rejects_bad_mode(oracle):
+    with pytest.raises(ValueError):
+        oracle.sampling(np.zeros((1, 3)), [0], [0], [1, 1, 1], np.zeros((1, 2)), [1], 2)
+
+
+def test_mcconv_forward_matches_per_centre_loop(oracle):
+    """monte_carlo_conv_test.py:66-108: out[i] = sum_j feat_j (x) relu(W d_ij / r + b)
+    / pdf_j, flattened and multiplied by the output weights."""
+    from tensorflow_graphics_point_clouds_amd import synthetic
+    cfg = synthetic.config1()
+    pts, bids = cfg["points"][:600], np.repeat([0, 1], 300).astype(np.int32)
+    feat = cfg["features"][:600]
+    r = np.float32(0.25)
+    g = oracle.Grid(pts, bids, 2, r)
+    nbh = oracle.Neighborhood(g, r, pts, bids)
+    pdf = nbh.pdf_per_pair(0.2)
+    out, basis, proj = oracle.mc_conv_forward(feat, pts, pts, nbh, pdf, cfg["weights"],
+                                              cfg["biases"], cfg["final_weights"], r)
+    w = cfg["weights"][0].astype(np.float64)
+    b = cfg["biases"][0, 0].astype(np.float64)
+    starts = oracle.segment_starts(nbh.ranges)
+    ids = nbh.original_neigh_ids
+    for i in [0, 7, 311, 599]:
+        acc = np.zeros((8, 16))
+        for m in range(starts[i], nbh.ranges[i]):
+            j = ids[m, 0]
+            delta = ((pts[j] - pts[i]) / np.full(3, r, np.float32)).astype(np.float64)
+            h = np.maximum(delta @ w + b, 0.0) / pdf[m]
+            acc += np.outer(feat[j].astype(np.float64), np.float32(h).astype(np.float64))
+        expect = acc.reshape(-1) @ cfg["final_weights"][0].astype(np.float64)
+        np.testing.assert_allclose(out[i], expect, rtol=1e-9, atol=1e-9)
+
+
+def test_pooling_matches_loops(oracle):
+    """pooling_layers_test.py:53-69, 112-135."""
+    rng = np.random.default_rng(4)
+    g, nbh = _grid_nbh(oracle, rng, 2, 300, 3, 0.2,
+                       centres=(rng.random((40, 3)).astype(np.float32),
+                                np.repeat([0, 1], 20).astype(np.int32)))
+    feat = rng.standard_normal((300, 5)).astype(np.float32)
+    ids = nbh.original_neigh_ids
+    mx = oracle.local_pool(feat, ids, 40, "max")
+    av = oracle.local_pool(feat, ids, 40, "avg")
+    starts = oracle.segment_starts(nbh.ranges)
+    for i in range(40):
+        rows = feat[ids[starts[i]:nbh.ranges[i], 0]].astype(np.float64)
+        if len(rows):
+            np.testing.assert_allclose(mx[i], rows.max(axis=0))
+            np.testing.assert_allclose(av[i], rows.mean(axis=0))
+        else:
+            assert np.all(av[i] == 0)
+    gm = oracle.global_pool(feat, g.batch_ids, 2, "max")
+    ga = oracle.global_pool(feat, g.batch_ids, 2, "avg")
+    for b in range(2):
+        np.testing.assert_allclose(gm[b], feat[g.batch_ids == b].max(axis=0))
+        np.testing.assert_allclose(ga[b], feat[g.batch_ids == b].astype(np.float64).mean(axis=0))
