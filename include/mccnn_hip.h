@@ -1,0 +1,328 @@
+/*
+ * mccnn_hip.h - C ABI of libmccnn_hip.so, the gfx950 implementation of the
+ * Monte-Carlo point-cloud convolution ops.
+ *
+ * Each entry point replaces one registered op of the reference's native package
+ * (custom_ops/tfg_custom_ops) or one piece of caller glue around it; the
+ * reference interface it stands for is cited above each declaration.
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer unless its name ends in _host;
+ *     tensors are row-major and contiguous; float = fp32, keys = int64,
+ *     indices = int32.  The small per-dimension vectors (num_cells,
+ *     inv_cell_sizes, inv_radii, inv_bandwidth) are device tensors as they are
+ *     in the reference ops.
+ *   - every tensor argument is preceded by the extents the reference op
+ *     validates, so the same shape errors can be reported.
+ *   - all work is enqueued on `stream` (a hipStream_t).  Only the *_count entry
+ *     points, which return a size the caller must allocate, synchronise the
+ *     stream (once); nothing else blocks.
+ *   - the library never allocates device memory: ops that need scratch take a
+ *     caller-owned workspace whose size the matching *_workspace_bytes function
+ *     returns.  Workspace contents are private to the library between a
+ *     *_count call and the *_fill call that follows it.
+ *   - "ranges" are inclusive end offsets: the pairs of centre i are rows
+ *     [ranges[i-1], ranges[i]) of the neighbour table, ranges[-1] == 0.
+ *   - return value: MCCNN_OK, MCCNN_INVALID_ARGUMENT (shape / attribute
+ *     violation; the reference raises errors::InvalidArgument) or
+ *     MCCNN_HIP_ERROR (the reference prints and exits,
+ *     shared/cc/kernels/tf_gpu_device.cpp:89-100).  mccnn_last_error() returns
+ *     the message of the calling thread's last failure.
+ *   - re-entrant: no mutable global state; calls on different streams may
+ *     overlap.
+ */
+#ifndef MCCNN_HIP_H_
+#define MCCNN_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void *mccnn_stream_t; /* hipStream_t */
+
+#define MCCNN_OK 0
+#define MCCNN_INVALID_ARGUMENT 1
+#define MCCNN_HIP_ERROR 2
+
+#define MCCNN_MIN_DIMENSIONS 2 /* shared/cc/kernels/defines.hpp:25 */
+#define MCCNN_MAX_DIMENSIONS 6 /* shared/cc/kernels/defines.hpp:26 */
+
+const char *mccnn_last_error(void);
+int mccnn_abi_version(void);
+
+/* ---------------------------------------------------------------- grid ---- */
+
+/* ComputeKeys: compute_keys/cc/ops/compute_keys_ops.cpp:29-121.
+ * keys_out[i] = batch_id * prod(num_cells) + row-major index of
+ * clamp(floor(p * inv_cell_sizes - scaled_aabb_min[batch_id]), 0, num_cells-1). */
+int mccnn_compute_keys(mccnn_stream_t stream, int64_t num_pts, int num_dims,
+                       const float *points, int64_t batch_ids_len,
+                       const int32_t *batch_ids, int64_t aabb_rows, int aabb_dims,
+                       const float *scaled_aabb_min, int num_cells_len,
+                       const int32_t *num_cells, int inv_cell_sizes_len,
+                       const float *inv_cell_sizes, int64_t *keys_out);
+
+/* The sort step of pylib/pc/Grid.py:56-64 (tf.argsort(keys, 'DESCENDING') and
+ * the gathers): stable descending sort, equal keys keep ascending original
+ * index.  key_bits = number of significant key bits (keys < 2^key_bits),
+ * 1..64.  sorted_keys_out / sorted_indices_out must not alias the inputs. */
+size_t mccnn_sort_keys_workspace_bytes(int64_t num_pts);
+int mccnn_sort_keys_descending(mccnn_stream_t stream, int64_t num_pts,
+                               int key_bits, const int64_t *keys,
+                               int64_t *sorted_keys_out,
+                               int32_t *sorted_indices_out, void *workspace,
+                               size_t workspace_bytes);
+int mccnn_gather_points(mccnn_stream_t stream, int64_t num_pts, int num_dims,
+                        const float *points, const int32_t *batch_ids,
+                        const int32_t *indices, float *points_out,
+                        int32_t *batch_ids_out);
+
+/* Per-cloud bounding box, grid shape and op inputs derived from them, the
+ * caller glue of pylib/pc/PointCloud.py:38-43, pylib/pc/Grid.py:44-48 and
+ * pylib/pc/custom_ops/custom_ops_wrapper.py:37-43:
+ *   aabb_min/max_out [B,D] = segment min/max -/+ 1e-9f
+ *   num_cells_out [D]      = max(1, max_b ceil((max-min)/cell_sizes))
+ *   scaled_aabb_min_out    = aabb_min / cell_sizes
+ *   inv_cell_sizes_out     = 1 / cell_sizes
+ * cell_sizes is a device vector [D]. */
+int mccnn_grid_setup(mccnn_stream_t stream, int64_t num_pts, int num_dims,
+                     const float *points, const int32_t *batch_ids,
+                     int batch_size, const float *cell_sizes,
+                     float *aabb_min_out, float *aabb_max_out,
+                     int32_t *num_cells_out, float *scaled_aabb_min_out,
+                     float *inv_cell_sizes_out);
+
+/* Small gathers of the caller glue:
+ *   original ids  out[m] = (sorted_indices[neighbors[m,0]], neighbors[m,1])
+ *                 pylib/pc/Neighborhood.py:246-250
+ *   pdf per pair  out[m] = pdf[neighbors[m,0]]   pylib/pc/Neighborhood.py:287
+ *   int32 gather  out[i] = src[indices[i]]       pylib/pc/sampling.py:142-146 */
+int mccnn_original_neighbor_ids(mccnn_stream_t stream, int64_t num_neighbors,
+                                const int32_t *neighbors,
+                                const int32_t *sorted_indices,
+                                int32_t *original_neighbors_out);
+int mccnn_gather_pdf(mccnn_stream_t stream, int64_t num_neighbors,
+                     const int32_t *neighbors, const float *pdf,
+                     float *pdf_per_pair_out);
+int mccnn_gather_i32(mccnn_stream_t stream, int64_t count, const int32_t *src,
+                     const int32_t *indices, int32_t *out);
+
+/* BuildGridDs: build_grid_ds/cc/ops/build_grid_ds_ops.cpp:27-115.
+ * ds_out is int32 [batch_size, num_cells[0], num_cells[1], 2]: (first, last+1)
+ * index of each column in the sorted arrays, (0,0) when empty.  num_cells is
+ * passed twice as in the reference: device copy and host copy. */
+int mccnn_build_grid_ds(mccnn_stream_t stream, int64_t num_pts,
+                        const int64_t *sorted_keys, int num_cells_len,
+                        const int32_t *num_cells, int num_cells_host_len,
+                        const int32_t *num_cells_host, int batch_size,
+                        int32_t *ds_out);
+
+/* ----------------------------------------------------------- neighbours --- */
+
+/* FindNeighbors: find_neighbors/cc/ops/find_neighbors_ops.cpp:42-259, split
+ * where the reference synchronises to size its second output
+ * (find_neighbors/cc/kernels/scan_alg_kernels.cu.cc:259-265).
+ *
+ * _count writes ranges_out [num_samples] (inclusive end offsets), stores
+ * the total pair count in *num_neighbors_out_host and synchronises `stream`.
+ * _fill writes neighbors_out [M,2] rows (sorted point index, centre index),
+ * grouped by centre, ascending point index inside a centre.
+ * max_neighs > 0 keeps the first max_neighs pairs of each centre in that order
+ * (the reference picks a wall-clock-seeded random subset,
+ * store_neighbors_kernels.cu.cc:216). */
+size_t mccnn_find_neighbors_workspace_bytes(int num_dims, int64_t num_samples);
+int mccnn_find_neighbors_count(
+    mccnn_stream_t stream, int64_t num_samples, int num_dims,
+    const float *samples, int64_t sample_batch_ids_len,
+    const int32_t *sample_batch_ids, int64_t num_pts, int pts_dims,
+    const float *points, int64_t point_keys_len, const int64_t *point_keys,
+    int ds_rank, int ds_batch, int ds_nx, int ds_ny, int ds_last,
+    const int32_t *grid_ds, int num_cells_len, const int32_t *num_cells,
+    int aabb_dims, const float *scaled_aabb_min, int inv_cell_sizes_len,
+    const float *inv_cell_sizes, int inv_radii_len, const float *inv_radii,
+    int max_neighs, void *workspace, size_t workspace_bytes,
+    int32_t *ranges_out, int64_t *num_neighbors_out_host);
+int mccnn_find_neighbors_fill(
+    mccnn_stream_t stream, int64_t num_samples, int num_dims,
+    const float *samples, const int32_t *sample_batch_ids, int64_t num_pts,
+    const float *points, const int64_t *point_keys, const int32_t *grid_ds,
+    const int32_t *num_cells, const float *scaled_aabb_min,
+    const float *inv_cell_sizes, const float *inv_radii, int max_neighs,
+    void *workspace, size_t workspace_bytes, const int32_t *ranges,
+    int64_t num_neighbors, int32_t *neighbors_out);
+
+/* ------------------------------------------------------------------ pdf --- */
+
+/* ComputePdf / ComputePdfWithPtGrads: compute_pdf/cc/ops/compute_pdf_ops.cpp:28-161.
+ * pdf_out[i] = sum over the pairs of centre i of
+ *   prod_d bw_d * exp(-0.5 * ((p_j - p_i)_d * bw_d * inv_radii_d)^2) * 0.39894228
+ * with bw = inv_bandwidth (mode 0) or sqrt(num_pts) (mode 1, as the reference
+ * computes it).  Centres are the points themselves: num_samples == num_pts. */
+int mccnn_compute_pdf(mccnn_stream_t stream, int64_t num_pts, int num_dims,
+                      const float *points, int64_t num_neighbors,
+                      int neighbors_rank, int neighbors_cols,
+                      const int32_t *neighbors, int64_t num_samples,
+                      const int32_t *ranges, int inv_bandwidth_len,
+                      const float *inv_bandwidth, int inv_radii_len,
+                      const float *inv_radii, int mode, float *pdf_out);
+
+/* ComputePdfPtGrads: compute_pdf/cc/ops/compute_pdf_ops.cpp:163-259.
+ * pt_grads_out [num_pts, D] = d(sum_i pdf_grads_i * pdf_i) / d(points). */
+int mccnn_compute_pdf_pt_grads(mccnn_stream_t stream, int64_t num_pts,
+                               int num_dims, const float *points,
+                               int64_t num_neighbors, int neighbors_rank,
+                               int neighbors_cols, const int32_t *neighbors,
+                               int64_t num_samples, const int32_t *ranges,
+                               int inv_bandwidth_len, const float *inv_bandwidth,
+                               int inv_radii_len, const float *inv_radii,
+                               int64_t pdf_grads_len, const float *pdf_grads,
+                               int mode, float *pt_grads_out);
+
+/* ----------------------------------------------------------- basis_proj --- */
+
+/* BasisProj: basis_proj/cc/ops/basis_proj_ops.cpp:25-131.
+ * out [num_samples, C, K]: out[i,c,k] = sum_m features[neighbors[m,0], c] *
+ * basis[m,k] over the pairs m of centre i.  K in {8,16,32,64}; C < 8 or a
+ * multiple of 8.  neighbors[:,0] indexes `features` (original point ids). */
+int mccnn_basis_proj(mccnn_stream_t stream, int64_t basis_rows, int num_basis,
+                     const float *basis, int64_t num_pts, int num_features,
+                     const float *features, int64_t num_neighbors,
+                     int neighbors_rank, int neighbors_cols,
+                     const int32_t *neighbors, int64_t num_samples,
+                     const int32_t *ranges, float *out);
+
+/* BasisProjGrads: basis_proj/cc/ops/basis_proj_ops.cpp:133-227.
+ * basis_grads_out [M,K], feature_grads_out [num_pts, C] for upstream gradient
+ * in_grads [num_samples, C, K] (its three extents are validated). */
+int mccnn_basis_proj_grads(mccnn_stream_t stream, int64_t basis_rows,
+                           int num_basis, const float *basis, int64_t num_pts,
+                           int num_features, const float *features,
+                           int64_t num_neighbors, int neighbors_rank,
+                           int neighbors_cols, const int32_t *neighbors,
+                           int64_t num_samples, const int32_t *ranges,
+                           int in_grads_rank, int64_t in_grads_dim0,
+                           int64_t in_grads_dim1, int64_t in_grads_dim2,
+                           const float *in_grads, float *basis_grads_out,
+                           float *feature_grads_out);
+
+/* ------------------------------------------------------------- sampling --- */
+
+/* Sampling: sampling/cc/ops/sampling_ops.cpp:33-204, split at the host
+ * synchronisation that sizes the outputs.  mode 0 = Poisson disk (2^D cell
+ * parity passes, count_sampling_pd_kernels.cu.cc:156-181), mode 1 = cell average.
+ * Inputs are the SORTED points / batch ids / keys and the self-neighbourhood.
+ * _count stores S in *num_sampled_out_host and synchronises; _fill writes
+ * sample_pts_out [S,D], sample_batch_ids_out [S], sample_indices_out [S]
+ * (mode 0: selected sorted indices, ascending; mode 1: first sorted index of
+ * each occupied cell, cells in sorted-key order). */
+size_t mccnn_sampling_workspace_bytes(int64_t num_pts);
+int mccnn_sampling_count(mccnn_stream_t stream, int mode, int64_t num_pts,
+                         int num_dims, const float *points,
+                         int64_t batch_ids_len, const int32_t *batch_ids,
+                         int64_t point_keys_len, const int64_t *point_keys,
+                         int num_cells_len, const int32_t *num_cells,
+                         int64_t num_neighbors, int neighbors_rank,
+                         int neighbors_cols, const int32_t *neighbors,
+                         int64_t ranges_len, const int32_t *ranges,
+                         void *workspace, size_t workspace_bytes,
+                         int64_t *num_sampled_out_host);
+int mccnn_sampling_fill(mccnn_stream_t stream, int mode, int64_t num_pts,
+                        int num_dims, const float *points,
+                        const int32_t *batch_ids, const int64_t *point_keys,
+                        const int32_t *num_cells, void *workspace,
+                        size_t workspace_bytes, int64_t num_sampled,
+                        float *sample_pts_out, int32_t *sample_batch_ids_out,
+                        int32_t *sample_indices_out);
+
+/* -------------------------------------------------------------- pooling --- */
+
+/* Local pooling over neighbourhoods, pylib/pc/layers/Pooling.py:107-166
+ * (tf.math.unsorted_segment_max / _mean over the pairs).  kind 0 = max,
+ * 1 = average.  out [num_samples, C]; a centre without pairs gets -FLT_MAX
+ * (max) or 0 (average), as the TensorFlow segment ops give.  neighbors holds
+ * ORIGINAL point ids in column 0. */
+int mccnn_local_pool(mccnn_stream_t stream, int kind, int64_t num_pts,
+                     int num_features, const float *features,
+                     int64_t num_neighbors, const int32_t *neighbors,
+                     int64_t num_samples, const int32_t *ranges, float *out);
+
+/* Gradient of the above.  Max: every pair whose feature equals the pooled value
+ * receives out_grads / (number of such pairs), the rule of TensorFlow's
+ * unsorted_segment_max gradient; average: out_grads / (pairs of the centre).
+ * `out` is the forward result.  feature_grads_out [num_pts, C] is overwritten. */
+int mccnn_local_pool_grads(mccnn_stream_t stream, int kind, int64_t num_pts,
+                           int num_features, const float *features,
+                           int64_t num_neighbors, const int32_t *neighbors,
+                           int64_t num_samples, const int32_t *ranges,
+                           const float *out, const float *out_grads,
+                           float *feature_grads_out);
+
+/* Global pooling per cloud, pylib/pc/layers/Pooling.py:25-104.  out [B, C];
+ * counts_out [B] (int32) receives the number of points of each cloud. */
+int mccnn_global_pool(mccnn_stream_t stream, int kind, int64_t num_pts,
+                      int num_features, const float *features,
+                      const int32_t *batch_ids, int batch_size, float *out,
+                      int32_t *counts_out);
+/* Gradient of the above with the tie rule of mccnn_local_pool_grads.
+ * tie_workspace is [B, C] floats of scratch (kind 0 only, may be NULL for 1). */
+int mccnn_global_pool_grads(mccnn_stream_t stream, int kind, int64_t num_pts,
+                            int num_features, const float *features,
+                            const int32_t *batch_ids, int batch_size,
+                            const float *out, const int32_t *counts,
+                            const float *out_grads, float *tie_workspace,
+                            float *feature_grads_out);
+
+/* --------------------------------------------------- layer composition --- */
+
+#define MCCNN_ACT_RELU 0
+#define MCCNN_ACT_LEAKY_RELU 1 /* slope 0.2 */
+#define MCCNN_ACT_ELU 2
+
+/* Per-pair basis of the Monte-Carlo convolution,
+ * pylib/pc/layers/MCConv.py:163-171 and :264-269 for a one-hidden-layer kernel:
+ *   delta_m = (points_in[nbr_m] - points_out[ctr_m]) * inv_radius     (fp32)
+ *   basis[m, l*H + h] = act(delta_m . W[l,:,h] + b[l,h]) / pdf[m]
+ * neighbors holds ORIGINAL ids (point, centre).  weights [L, D, H], biases
+ * [L, H] with L*H = num_basis. */
+int mccnn_mc_basis(mccnn_stream_t stream, int64_t num_neighbors, int num_dims,
+                   int num_basis, int activation, const float *points_in,
+                   const float *points_out, const int32_t *neighbors,
+                   const float *inv_radii, const float *weights,
+                   const float *biases, int num_mlps, const float *pdf,
+                   float *basis_out);
+
+/* Gradient of the above w.r.t. weights and biases (accumulated over all pairs)
+ * for upstream basis_grads [M, num_basis].  weight_grads_out [L,D,H] and
+ * bias_grads_out [L,H] are overwritten.  partials is a workspace of
+ * mccnn_mc_basis_grads_workspace_bytes() bytes. */
+size_t mccnn_mc_basis_grads_workspace_bytes(int num_dims, int num_basis);
+int mccnn_mc_basis_grads(mccnn_stream_t stream, int64_t num_neighbors,
+                         int num_dims, int num_basis, int activation,
+                         const float *points_in, const float *points_out,
+                         const int32_t *neighbors, const float *inv_radii,
+                         const float *weights, const float *biases,
+                         int num_mlps, const float *pdf,
+                         const float *basis_grads, void *workspace,
+                         size_t workspace_bytes, float *weight_grads_out,
+                         float *bias_grads_out);
+
+/* Per-pair kernel-point weights, pylib/pc/layers/KPConv.py:29-57,193-213:
+ *   d[m,k] = || delta_m - (kernel_points[k] + offsets[ctr_m,k]) ||
+ *   kind 0: max(1 - d/sigma, 0);  kind 1: exp(-(d/(sigma/3))^2)
+ * written to basis_out [M, num_basis] with columns >= num_kernel_points zero.
+ * offsets [num_samples, num_kernel_points, D] may be NULL (rigid).  dist_out
+ * [M, num_kernel_points] may be NULL. */
+int mccnn_kp_basis(mccnn_stream_t stream, int64_t num_neighbors, int num_dims,
+                   int num_kernel_points, int num_basis, int kind, float sigma,
+                   const float *points_in, const float *points_out,
+                   const int32_t *neighbors, const float *inv_radii,
+                   const float *kernel_points, const float *offsets,
+                   float *basis_out, float *dist_out);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MCCNN_HIP_H_ */

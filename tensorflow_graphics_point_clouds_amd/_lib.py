@@ -1,0 +1,82 @@
+"""ctypes loader for libmccnn_hip.so and helpers to pass torch tensors through
+its C ABI (include/mccnn_hip.h).  There is no fallback: if the library is not
+built, or a tensor is not a contiguous GPU tensor of the right dtype, the call
+raises."""
+import ctypes
+import os
+import subprocess
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libmccnn_hip.so")
+CSRC_DIR = os.path.join(_HERE, "csrc")
+
+_lib = None
+
+i64 = ctypes.c_int64
+cint = ctypes.c_int
+cfloat = ctypes.c_float
+csize = ctypes.c_size_t
+vptr = ctypes.c_void_p
+
+
+class InvalidArgumentError(ValueError):
+    """Shape or attribute violation reported by an op (the reference raises
+    tf.errors.InvalidArgumentError for the same conditions)."""
+
+
+def build(jobs=8):
+    """Compile every HIP source for gfx950 into libmccnn_hip.so (in-tree)."""
+    subprocess.run(["make", "-C", CSRC_DIR, "-B", "-j%d" % jobs], check=True,
+                   stdout=subprocess.DEVNULL)
+    global _lib
+    _lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                "libmccnn_hip.so is not built (expected at %s); run "
+                "`make -C %s` or __graft_entry__.build()" % (LIB_PATH, CSRC_DIR))
+        handle = ctypes.CDLL(LIB_PATH)
+        handle.mccnn_last_error.restype = ctypes.c_char_p
+        for name in ("mccnn_sort_keys_workspace_bytes",
+                     "mccnn_find_neighbors_workspace_bytes",
+                     "mccnn_sampling_workspace_bytes",
+                     "mccnn_mc_basis_grads_workspace_bytes"):
+            getattr(handle, name).restype = csize
+        _lib = handle
+    return _lib
+
+
+def check(rc):
+    if rc == 0:
+        return
+    msg = lib().mccnn_last_error().decode("utf-8", "replace")
+    if rc == 1:
+        raise InvalidArgumentError(msg)
+    raise RuntimeError("HIP error in libmccnn_hip: " + msg)
+
+
+def stream():
+    import torch
+    return vptr(torch.cuda.current_stream().cuda_stream)
+
+
+def ptr(t, dtype=None):
+    """Device pointer of a contiguous GPU tensor (None -> NULL)."""
+    if t is None:
+        return vptr(0)
+    if not t.is_cuda:
+        raise TypeError("expected a GPU tensor, got one on %s" % t.device)
+    if dtype is not None and t.dtype != dtype:
+        raise TypeError("expected dtype %s, got %s" % (dtype, t.dtype))
+    if not t.is_contiguous():
+        raise TypeError("expected a contiguous tensor")
+    return vptr(t.data_ptr())
+
+
+def workspace(nbytes, device):
+    import torch
+    return torch.empty(max(int(nbytes), 1), dtype=torch.uint8, device=device)

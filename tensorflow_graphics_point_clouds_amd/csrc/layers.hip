@@ -1,0 +1,272 @@
+// Per-pair basis functions of the convolution layers, evaluated in registers
+// from the two point coordinates of a pair:
+//   Monte-Carlo convolution  pylib/pc/layers/MCConv.py:163-171, 264-269
+//   kernel-point convolution pylib/pc/layers/KPConv.py:29-57, 193-213
+// One lane per (pair, basis column): the K lanes of a pair read the same two
+// points (broadcast loads) and write one contiguous basis row.
+#include "common.h"
+#include "fill.h"
+
+namespace mccnn {
+
+__device__ __forceinline__ float act_fwd(int act, float z) {
+  if (act == MCCNN_ACT_RELU) return z > 0.0f ? z : 0.0f;
+  if (act == MCCNN_ACT_LEAKY_RELU) return z > 0.0f ? z : 0.2f * z;
+  return z > 0.0f ? z : expm1f(z);
+}
+
+__device__ __forceinline__ float act_bwd(int act, float z) {
+  if (act == MCCNN_ACT_RELU) return z > 0.0f ? 1.0f : 0.0f;
+  if (act == MCCNN_ACT_LEAKY_RELU) return z > 0.0f ? 1.0f : 0.2f;
+  return z > 0.0f ? 1.0f : expf(z);
+}
+
+// delta = (p_in[nbr] - p_out[ctr]) * inv_radii
+template <int D>
+__device__ __forceinline__ void pair_delta(const float *__restrict__ pin,
+                                           const float *__restrict__ pout, int2 pr,
+                                           const float *ir, float *delta) {
+#pragma unroll
+  for (int d = 0; d < D; ++d)
+    delta[d] = (pin[(int64_t)pr.x * D + d] - pout[(int64_t)pr.y * D + d]) * ir[d];
+}
+
+// weights [L, D, H]: column j = l*H + h reads weights[(l*D + d)*H + h].
+template <int D>
+__global__ void __launch_bounds__(256) mc_basis_kernel(
+    int64_t m_total, int K, int H, int act, const float *__restrict__ pin,
+    const float *__restrict__ pout, const int2 *__restrict__ nbrs,
+    const float *__restrict__ inv_radii, const float *__restrict__ weights,
+    const float *__restrict__ biases, const float *__restrict__ pdf, float *__restrict__ basis) {
+  float ir[D];
+#pragma unroll
+  for (int d = 0; d < D; ++d) ir[d] = inv_radii[d];
+  const int64_t total = m_total * K;
+  for (int64_t t = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; t < total;
+       t += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t m = t / K;
+    const int j = (int)(t - m * K);
+    const int l = j / H, h = j - l * H;
+    float delta[D];
+    pair_delta<D>(pin, pout, nbrs[m], ir, delta);
+    float z = biases[j];
+#pragma unroll
+    for (int d = 0; d < D; ++d) z += delta[d] * weights[(l * D + d) * H + h];
+    basis[t] = act_fwd(act, z) / pdf[m];
+  }
+}
+
+constexpr int kGradBlocks = 1024;
+
+// Each block walks a strided share of the pairs; thread (row r, column j) keeps
+// D weight partials and one bias partial, reduced over the rows in LDS and
+// written to partials[block][(D+1)*K].
+template <int D>
+__global__ void __launch_bounds__(256) mc_basis_grads_kernel(
+    int64_t m_total, int K, int H, int act, const float *__restrict__ pin,
+    const float *__restrict__ pout, const int2 *__restrict__ nbrs,
+    const float *__restrict__ inv_radii, const float *__restrict__ weights,
+    const float *__restrict__ biases, const float *__restrict__ pdf,
+    const float *__restrict__ dbasis, float *__restrict__ partials) {
+  __shared__ float red[256 * (D + 1)];
+  float ir[D];
+#pragma unroll
+  for (int d = 0; d < D; ++d) ir[d] = inv_radii[d];
+  const int rows = 256 / K;                 // pairs handled per step by this block
+  const int j = threadIdx.x % K, r = threadIdx.x / K;
+  const int l = j / H, h = j - l * H;
+  float w[D], dw[D], db = 0.0f;
+#pragma unroll
+  for (int d = 0; d < D; ++d) {
+    w[d] = weights[(l * D + d) * H + h];
+    dw[d] = 0.0f;
+  }
+  const float bj = biases[j];
+  for (int64_t m = (int64_t)blockIdx.x * rows + r; m < m_total; m += (int64_t)gridDim.x * rows) {
+    float delta[D];
+    pair_delta<D>(pin, pout, nbrs[m], ir, delta);
+    float z = bj;
+#pragma unroll
+    for (int d = 0; d < D; ++d) z += delta[d] * w[d];
+    const float dz = dbasis[m * K + j] * act_bwd(act, z) / pdf[m];
+    db += dz;
+#pragma unroll
+    for (int d = 0; d < D; ++d) dw[d] += delta[d] * dz;
+  }
+#pragma unroll
+  for (int d = 0; d < D; ++d) red[d * 256 + threadIdx.x] = dw[d];
+  red[D * 256 + threadIdx.x] = db;
+  __syncthreads();
+  if (r == 0) {
+    for (int q = 0; q <= D; ++q) {
+      float s = 0.0f;
+      for (int rr = 0; rr < rows; ++rr) s += red[q * 256 + rr * K + j];
+      partials[((int64_t)blockIdx.x * (D + 1) + q) * K + j] = s;
+    }
+  }
+}
+
+// weight_grads [L, D, H], bias_grads [L, H] from partials [blocks][(D+1)][K].
+__global__ void mc_basis_grads_reduce_kernel(int blocks, int D, int K, int H,
+                                             const float *__restrict__ partials,
+                                             float *__restrict__ dweights,
+                                             float *__restrict__ dbiases) {
+  const int t = blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= (D + 1) * K) return;
+  const int q = t / K, j = t - q * K;
+  float s = 0.0f;
+  for (int b = 0; b < blocks; ++b) s += partials[((int64_t)b * (D + 1) + q) * K + j];
+  const int l = j / H, h = j - l * H;
+  if (q < D) dweights[(l * D + q) * H + h] = s;
+  else dbiases[j] = s;
+}
+
+template <int D>
+__global__ void __launch_bounds__(256) kp_basis_kernel(
+    int64_t m_total, int KP, int K, int kind, float sigma, const float *__restrict__ pin,
+    const float *__restrict__ pout, const int2 *__restrict__ nbrs,
+    const float *__restrict__ inv_radii, const float *__restrict__ kpts,
+    const float *__restrict__ offsets, float *__restrict__ basis, float *__restrict__ dist_out) {
+  float ir[D];
+#pragma unroll
+  for (int d = 0; d < D; ++d) ir[d] = inv_radii[d];
+  const int64_t total = m_total * K;
+  for (int64_t t = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; t < total;
+       t += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t m = t / K;
+    const int k = (int)(t - m * K);
+    float wgt = 0.0f;
+    if (k < KP) {
+      const int2 pr = nbrs[m];
+      float delta[D];
+      pair_delta<D>(pin, pout, pr, ir, delta);
+      float sq = 0.0f;
+#pragma unroll
+      for (int d = 0; d < D; ++d) {
+        float kp = kpts[k * D + d];
+        if (offsets) kp += offsets[((int64_t)pr.y * KP + k) * D + d];
+        const float diff = delta[d] - kp;
+        sq += diff * diff;
+      }
+      const float dist = sqrtf(sq);
+      if (dist_out) dist_out[m * KP + k] = dist;
+      if (kind == 0) {
+        const float v = 1.0f - dist / sigma;
+        wgt = v > 0.0f ? v : 0.0f;
+      } else {
+        const float q = dist / (sigma / 3.0f);
+        wgt = expf(-(q * q));
+      }
+    }
+    basis[t] = wgt;
+  }
+}
+
+static bool valid_basis_count(int k) { return k == 8 || k == 16 || k == 32 || k == 64; }
+
+}  // namespace mccnn
+
+using namespace mccnn;
+
+extern "C" int mccnn_mc_basis(mccnn_stream_t stream, int64_t num_neighbors, int num_dims,
+                              int num_basis, int activation, const float *points_in,
+                              const float *points_out, const int32_t *neighbors,
+                              const float *inv_radii, const float *weights, const float *biases,
+                              int num_mlps, const float *pdf, float *basis_out) {
+  MCCNN_REQUIRE(valid_dims(num_dims), "mc_basis expects a valid number of dimensions");
+  MCCNN_REQUIRE(valid_basis_count(num_basis), "mc_basis expects 8, 16, 32 or 64 basis functions");
+  MCCNN_REQUIRE(num_mlps > 0 && num_basis % num_mlps == 0,
+                "mc_basis expects the number of basis functions to be divisible by the number of "
+                "kernel MLPs");
+  MCCNN_REQUIRE(activation >= 0 && activation <= 2, "mc_basis expects a known activation");
+  MCCNN_REQUIRE(num_neighbors >= 0, "mc_basis expects a non-negative size");
+  if (num_neighbors == 0) return MCCNN_OK;
+  MCCNN_REQUIRE(points_in && points_out && neighbors && inv_radii && weights && biases && pdf &&
+                    basis_out,
+                "mc_basis received a null tensor");
+  int64_t work = num_neighbors * num_basis;
+  if (work > (int64_t)1 << 26) work = (int64_t)1 << 26;
+  MCCNN_DIM_SWITCH(num_dims, hipLaunchKernelGGL(mc_basis_kernel<D>, dim3(blocks_for(work, 256)),
+                                                dim3(256), 0, as_stream(stream), num_neighbors,
+                                                num_basis, num_basis / num_mlps, activation,
+                                                points_in, points_out, (const int2 *)neighbors,
+                                                inv_radii, weights, biases, pdf, basis_out));
+  MCCNN_LAUNCH_CHECK();
+  return MCCNN_OK;
+}
+
+extern "C" size_t mccnn_mc_basis_grads_workspace_bytes(int num_dims, int num_basis) {
+  if (!valid_dims(num_dims) || num_basis <= 0) return 0;
+  return align256(sizeof(float) * (size_t)kGradBlocks * (num_dims + 1) * num_basis);
+}
+
+extern "C" int mccnn_mc_basis_grads(mccnn_stream_t stream, int64_t num_neighbors, int num_dims,
+                                    int num_basis, int activation, const float *points_in,
+                                    const float *points_out, const int32_t *neighbors,
+                                    const float *inv_radii, const float *weights,
+                                    const float *biases, int num_mlps, const float *pdf,
+                                    const float *basis_grads, void *workspace,
+                                    size_t workspace_bytes, float *weight_grads_out,
+                                    float *bias_grads_out) {
+  MCCNN_REQUIRE(valid_dims(num_dims), "mc_basis_grads expects a valid number of dimensions");
+  MCCNN_REQUIRE(valid_basis_count(num_basis),
+                "mc_basis_grads expects 8, 16, 32 or 64 basis functions");
+  MCCNN_REQUIRE(num_mlps > 0 && num_basis % num_mlps == 0,
+                "mc_basis_grads expects the number of basis functions to be divisible by the "
+                "number of kernel MLPs");
+  MCCNN_REQUIRE(activation >= 0 && activation <= 2, "mc_basis_grads expects a known activation");
+  MCCNN_REQUIRE(num_neighbors >= 0, "mc_basis_grads expects a non-negative size");
+  MCCNN_REQUIRE(weight_grads_out && bias_grads_out && workspace,
+                "mc_basis_grads received a null tensor");
+  MCCNN_REQUIRE(workspace_bytes >= mccnn_mc_basis_grads_workspace_bytes(num_dims, num_basis),
+                "mc_basis_grads workspace too small");
+  MCCNN_REQUIRE(num_neighbors == 0 || (points_in && points_out && neighbors && inv_radii &&
+                                       weights && biases && pdf && basis_grads),
+                "mc_basis_grads received a null tensor");
+  hipStream_t s = as_stream(stream);
+  const int rows = 256 / num_basis;
+  int blocks = (int)((num_neighbors + rows - 1) / rows);
+  if (blocks > kGradBlocks) blocks = kGradBlocks;
+  if (blocks < 1) blocks = 1;
+  MCCNN_DIM_SWITCH(num_dims, hipLaunchKernelGGL(mc_basis_grads_kernel<D>, dim3(blocks), dim3(256),
+                                                0, s, num_neighbors, num_basis,
+                                                num_basis / num_mlps, activation, points_in,
+                                                points_out, (const int2 *)neighbors, inv_radii,
+                                                weights, biases, pdf, basis_grads,
+                                                (float *)workspace));
+  MCCNN_LAUNCH_CHECK();
+  const int outs = (num_dims + 1) * num_basis;
+  hipLaunchKernelGGL(mc_basis_grads_reduce_kernel, dim3(blocks_for(outs, 64)), dim3(64), 0, s,
+                     blocks, num_dims, num_basis, num_basis / num_mlps,
+                     (const float *)workspace, weight_grads_out, bias_grads_out);
+  MCCNN_LAUNCH_CHECK();
+  return MCCNN_OK;
+}
+
+extern "C" int mccnn_kp_basis(mccnn_stream_t stream, int64_t num_neighbors, int num_dims,
+                              int num_kernel_points, int num_basis, int kind, float sigma,
+                              const float *points_in, const float *points_out,
+                              const int32_t *neighbors, const float *inv_radii,
+                              const float *kernel_points, const float *offsets, float *basis_out,
+                              float *dist_out) {
+  MCCNN_REQUIRE(valid_dims(num_dims), "kp_basis expects a valid number of dimensions");
+  MCCNN_REQUIRE(valid_basis_count(num_basis), "kp_basis expects 8, 16, 32 or 64 basis columns");
+  MCCNN_REQUIRE(num_kernel_points > 0 && num_kernel_points <= num_basis,
+                "kp_basis expects 1 <= kernel points <= basis columns");
+  MCCNN_REQUIRE(kind == 0 || kind == 1, "kp_basis expects kind 0 (linear) or 1 (gaussian)");
+  MCCNN_REQUIRE(sigma > 0.0f, "kp_basis expects a positive sigma");
+  MCCNN_REQUIRE(num_neighbors >= 0, "kp_basis expects a non-negative size");
+  if (num_neighbors == 0) return MCCNN_OK;
+  MCCNN_REQUIRE(points_in && points_out && neighbors && inv_radii && kernel_points && basis_out,
+                "kp_basis received a null tensor");
+  int64_t work = num_neighbors * num_basis;
+  if (work > (int64_t)1 << 26) work = (int64_t)1 << 26;
+  MCCNN_DIM_SWITCH(num_dims, hipLaunchKernelGGL(kp_basis_kernel<D>, dim3(blocks_for(work, 256)),
+                                                dim3(256), 0, as_stream(stream), num_neighbors,
+                                                num_kernel_points, num_basis, kind, sigma,
+                                                points_in, points_out, (const int2 *)neighbors,
+                                                inv_radii, kernel_points, offsets, basis_out,
+                                                dist_out));
+  MCCNN_LAUNCH_CHECK();
+  return MCCNN_OK;
+}

@@ -1,0 +1,296 @@
+// Radius neighbour search on the sorted regular grid
+// (custom_ops/tfg_custom_ops/find_neighbors/cc/ops/find_neighbors_ops.cpp:86-250).
+//
+// Three stages, all deterministic:
+//   ranges  one lane per (centre, cell offset): the column of the 2-D table and
+//           a binary search over the descending keys give the contiguous slice
+//           of sorted points that lies in the offset cell row
+//           (find_ranges_grid_ds_kernels.cu.cc:48-235);
+//   count   16 lanes per centre stride over the slices and test
+//           |(s - p) * inv_radii| < 1 (count_neighbors_kernels.cu.cc:83-86);
+//   fill    same traversal; the slot of a hit is the centre's start offset plus
+//           a ballot prefix inside the 16-lane group, so the pairs of a centre
+//           come out in ascending sorted-point index without atomics or a sort.
+// Offsets are enumerated so that the slices of a centre ascend in index.
+// Compiled with -ffp-contract=off (the distance test decides integer output).
+#include "common.h"
+#include "fill.h"
+
+namespace mccnn {
+
+constexpr int kGroup = 16;                 // lanes per centre
+constexpr int kNbrThreads = 256;
+constexpr int kCentresPerBlock = kNbrThreads / kGroup;
+
+// Offsets act on dims 0..max(D-2,1); the last dim is covered by the key search.
+template <int D>
+struct OffsetInfo {
+  static constexpr int kDims = (D - 2 > 1 ? D - 2 : 1) + 1;
+  static constexpr int count() {
+    int c = 1;
+    for (int i = 0; i < kDims; ++i) c *= 3;
+    return c;
+  }
+};
+
+template <int D>
+__global__ void __launch_bounds__(256) nbr_ranges_kernel(
+    int64_t ns, const float *__restrict__ samples, const int *__restrict__ sbids,
+    const int64_t *__restrict__ keys, const int2 *__restrict__ ds,
+    const int *__restrict__ num_cells, const float *__restrict__ smin,
+    const float *__restrict__ inv_cell, int2 *__restrict__ ranges) {
+  constexpr int R = OffsetInfo<D>::count();
+  constexpr int OD = OffsetInfo<D>::kDims;
+  const GridShape<D> g = load_shape<D>(num_cells);
+  float ic[D];
+#pragma unroll
+  for (int d = 0; d < D; ++d) ic[d] = inv_cell[d];
+  const int64_t total = ns * R;
+  for (int64_t t = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; t < total;
+       t += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t c = t / R;
+    int r = (int)(t - c * R);
+    const int b = sbids[c];
+    float p[D], m[D];
+#pragma unroll
+    for (int d = 0; d < D; ++d) {
+      p[d] = samples[c * D + d];
+      m[d] = smin[(int64_t)b * D + d];
+    }
+    int cell[D];
+    cell_of_point<D>(p, m, ic, g, cell);
+    // offset digits, most significant = dim 0, value 1 - digit (descending)
+    bool inside = true;
+#pragma unroll
+    for (int d = OD - 1; d >= 0; --d) {
+      cell[d] += 1 - (r % 3);
+      r /= 3;
+      inside = inside && cell[d] >= 0 && cell[d] < g.n[d];
+    }
+    int2 out = make_int2(0, 0);
+    if (inside) {
+      const int64_t col = ((int64_t)b * g.n[0] + cell[0]) * g.n[1] + cell[1];
+      const int2 span = ds[col];
+      if (span.y > span.x) {
+        if (D == 2) {
+          out = span;
+        } else {
+          const int64_t aux = key_of_cell<D>(cell, g, b);
+          const int w = cell[D - 1];
+          const int64_t maxk = aux + (w < g.n[D - 1] - 1 ? 1 : 0);
+          const int64_t mink = aux - (w > 0 ? 1 : 0);
+          int lo = span.x, hi = span.y;
+          while (lo < hi) {                       // first index with key <= maxk
+            const int mid = lo + ((hi - lo) >> 1);
+            if (keys[mid] > maxk) lo = mid + 1; else hi = mid;
+          }
+          const int first = lo;
+          hi = span.y;
+          while (lo < hi) {                       // first index with key < mink
+            const int mid = lo + ((hi - lo) >> 1);
+            if (keys[mid] >= mink) lo = mid + 1; else hi = mid;
+          }
+          if (lo > first) out = make_int2(first, lo);
+        }
+      }
+    }
+    ranges[t] = out;
+  }
+}
+
+template <int D>
+__device__ __forceinline__ bool within_radius(const float *s, const float *__restrict__ pts,
+                                              int64_t j, const float *ir) {
+  float acc = 0.0f;
+#pragma unroll
+  for (int d = 0; d < D; ++d) {
+    const float diff = s[d] - pts[j * D + d];
+    const float sc = diff * ir[d];
+    const float sq = sc * sc;
+    acc = acc + sq;
+  }
+  return sqrtf(acc) < 1.0f;
+}
+
+// kFill == false: counts[c] = number of hits (clamped to max_neighs when > 0).
+// kFill == true : writes the pairs of centre c starting at its start offset.
+template <int D, bool kFill>
+__global__ void __launch_bounds__(kNbrThreads) nbr_visit_kernel(
+    int64_t ns, const float *__restrict__ samples, const float *__restrict__ pts,
+    const int2 *__restrict__ ranges, const float *__restrict__ inv_radii, int max_neighs,
+    int *__restrict__ counts, const int *__restrict__ ends, int2 *__restrict__ nbrs) {
+  constexpr int R = OffsetInfo<D>::count();
+  const int sub = threadIdx.x & (kGroup - 1);
+  const int lane = lane_id();
+  const uint64_t group_mask = ((1ull << kGroup) - 1ull) << (lane & ~(kGroup - 1));
+  const uint64_t below_mask = group_mask & ((1ull << lane) - 1ull);
+  float ir[D];
+#pragma unroll
+  for (int d = 0; d < D; ++d) ir[d] = inv_radii[d];
+  const int64_t c = (int64_t)blockIdx.x * kCentresPerBlock + threadIdx.x / kGroup;
+  if (c >= ns) return;
+  float s[D];
+#pragma unroll
+  for (int d = 0; d < D; ++d) s[d] = samples[c * D + d];
+  const int limit = max_neighs > 0 ? max_neighs : 0x7fffffff;
+  int found = 0;                                   // kFill: slots used so far
+  int64_t start = 0;
+  if (kFill) start = c > 0 ? ends[c - 1] : 0;
+  for (int r = 0; r < R; ++r) {
+    const int2 span = ranges[c * R + r];
+    for (int j0 = span.x; j0 < span.y; j0 += kGroup) {
+      const int j = j0 + sub;
+      const bool hit = j < span.y && within_radius<D>(s, pts, j, ir);
+      if (kFill) {
+        const uint64_t hits = __ballot(hit) & group_mask;
+        const int slot = found + __popcll(hits & below_mask);
+        if (hit && slot < limit) nbrs[start + slot] = make_int2(j, (int)c);
+        found += __popcll(hits);
+      } else {
+        found += hit ? 1 : 0;
+      }
+    }
+  }
+  if (!kFill) {
+#pragma unroll
+    for (int off = kGroup / 2; off > 0; off >>= 1) found += __shfl_xor(found, off, kWave);
+    if (sub == 0) counts[c] = found < limit ? found : limit;
+  }
+}
+
+struct NbrWorkspace {
+  int2 *ranges;
+  int *scan_scratch;
+  int64_t *total;
+  size_t bytes;
+};
+
+static int offsets_for(int d) {
+  int od = (d - 2 > 1 ? d - 2 : 1) + 1, c = 1;
+  for (int i = 0; i < od; ++i) c *= 3;
+  return c;
+}
+
+static NbrWorkspace carve_nbr_workspace(void *ws, int d, int64_t ns) {
+  char *p = (char *)ws;
+  NbrWorkspace w;
+  size_t off = 0;
+  w.ranges = (int2 *)(p + off);
+  off += align256(sizeof(int2) * (size_t)ns * offsets_for(d));
+  w.scan_scratch = (int *)(p + off);
+  off += align256(sizeof(int) * scan_scratch_ints(ns));
+  w.total = (int64_t *)(p + off);
+  off += 256;
+  w.bytes = off;
+  return w;
+}
+
+}  // namespace mccnn
+
+using namespace mccnn;
+
+extern "C" size_t mccnn_find_neighbors_workspace_bytes(int num_dims, int64_t num_samples) {
+  if (!valid_dims(num_dims) || num_samples < 0) return 0;
+  return carve_nbr_workspace(nullptr, num_dims, num_samples).bytes;
+}
+
+extern "C" int mccnn_find_neighbors_count(
+    mccnn_stream_t stream, int64_t num_samples, int num_dims, const float *samples,
+    int64_t sample_batch_ids_len, const int32_t *sample_batch_ids, int64_t num_pts, int pts_dims,
+    const float *points, int64_t point_keys_len, const int64_t *point_keys, int ds_rank,
+    int ds_batch, int ds_nx, int ds_ny, int ds_last, const int32_t *grid_ds, int num_cells_len,
+    const int32_t *num_cells, int aabb_dims, const float *scaled_aabb_min, int inv_cell_sizes_len,
+    const float *inv_cell_sizes, int inv_radii_len, const float *inv_radii, int max_neighs,
+    void *workspace, size_t workspace_bytes, int32_t *ranges_out,
+    int64_t *num_neighbors_out_host) {
+  MCCNN_REQUIRE(valid_dims(num_dims), "FindNeighbors expects a valid number of dimensions");
+  MCCNN_REQUIRE(num_cells_len == num_dims,
+                "FindNeighbors expects a number of dimensions in num_cells equal to the number of "
+                "dimensions in the input points");
+  MCCNN_REQUIRE(pts_dims == num_dims,
+                "FindNeighbors expects a number of dimensions in points equal to the number of "
+                "dimensions in the samples");
+  MCCNN_REQUIRE(aabb_dims == num_dims,
+                "FindNeighbors expects a number of dimensions in scaled_aabb_min equal to the "
+                "number of dimensions in the input points");
+  MCCNN_REQUIRE(inv_cell_sizes_len == num_dims,
+                "FindNeighbors expects a number of dimensions in inv_cell_sizes equal to the "
+                "number of dimensions in the input points");
+  MCCNN_REQUIRE(inv_radii_len == num_dims,
+                "FindNeighbors expects a number of dimensions in inv_radii equal to the number of "
+                "dimensions in the input points");
+  MCCNN_REQUIRE(sample_batch_ids_len == num_samples,
+                "FindNeighbors expects the same number of batch ids as samples");
+  MCCNN_REQUIRE(point_keys_len == num_pts,
+                "FindNeighbors expects the same number of keys as points");
+  MCCNN_REQUIRE(ds_rank == 4 && ds_last == 2,
+                "FindNeighbors expects a grid acceleration data structure with the right format "
+                "(B, X, Y, 2)");
+  MCCNN_REQUIRE(ds_batch > 0 && ds_nx > 0 && ds_ny > 0,
+                "FindNeighbors expects a non-empty grid acceleration data structure");
+  MCCNN_REQUIRE(num_samples >= 0 && num_pts >= 0 && num_samples < ((int64_t)1 << 31) &&
+                    num_pts < ((int64_t)1 << 31),
+                "FindNeighbors expects sizes in [0, 2^31)");
+  MCCNN_REQUIRE(num_neighbors_out_host, "FindNeighbors received a null output");
+  *num_neighbors_out_host = 0;
+  if (num_samples == 0) return MCCNN_OK;
+  MCCNN_REQUIRE(samples && sample_batch_ids && grid_ds && num_cells && scaled_aabb_min &&
+                    inv_cell_sizes && inv_radii && ranges_out && workspace,
+                "FindNeighbors received a null tensor");
+  MCCNN_REQUIRE(num_pts == 0 || (points && point_keys), "FindNeighbors received a null tensor");
+  const NbrWorkspace w = carve_nbr_workspace(workspace, num_dims, num_samples);
+  MCCNN_REQUIRE(workspace_bytes >= w.bytes, "FindNeighbors workspace too small (%zu < %zu)",
+                workspace_bytes, w.bytes);
+  hipStream_t s = as_stream(stream);
+  const int64_t work = num_samples * offsets_for(num_dims);
+  MCCNN_DIM_SWITCH(num_dims,
+                   hipLaunchKernelGGL(nbr_ranges_kernel<D>, dim3(blocks_for(work, 256)), dim3(256),
+                                      0, s, num_samples, samples, sample_batch_ids,
+                                      (const int64_t *)point_keys, (const int2 *)grid_ds,
+                                      num_cells, scaled_aabb_min, inv_cell_sizes, w.ranges));
+  MCCNN_LAUNCH_CHECK();
+  const unsigned grid = blocks_for(num_samples, kCentresPerBlock);
+  MCCNN_DIM_SWITCH(num_dims, hipLaunchKernelGGL((nbr_visit_kernel<D, false>), dim3(grid),
+                                                dim3(kNbrThreads), 0, s, num_samples, samples,
+                                                points, (const int2 *)w.ranges, inv_radii,
+                                                max_neighs, ranges_out, (const int *)nullptr,
+                                                (int2 *)nullptr));
+  MCCNN_LAUNCH_CHECK();
+  int rc = inclusive_scan_i32(s, num_samples, ranges_out, w.scan_scratch, w.total);
+  if (rc != MCCNN_OK) return rc;
+  MCCNN_HIP_CHECK(hipMemcpyAsync(num_neighbors_out_host, w.total, sizeof(int64_t),
+                                 hipMemcpyDeviceToHost, s));
+  MCCNN_HIP_CHECK(hipStreamSynchronize(s));
+  MCCNN_REQUIRE(*num_neighbors_out_host < ((int64_t)1 << 31),
+                "FindNeighbors found %lld pairs; the int32 offsets of the op contract hold fewer "
+                "than 2^31",
+                (long long)*num_neighbors_out_host);
+  return MCCNN_OK;
+}
+
+extern "C" int mccnn_find_neighbors_fill(
+    mccnn_stream_t stream, int64_t num_samples, int num_dims, const float *samples,
+    const int32_t *sample_batch_ids, int64_t num_pts, const float *points,
+    const int64_t *point_keys, const int32_t *grid_ds, const int32_t *num_cells,
+    const float *scaled_aabb_min, const float *inv_cell_sizes, const float *inv_radii,
+    int max_neighs, void *workspace, size_t workspace_bytes, const int32_t *ranges,
+    int64_t num_neighbors, int32_t *neighbors_out) {
+  (void)sample_batch_ids; (void)point_keys; (void)grid_ds; (void)num_cells;
+  (void)scaled_aabb_min; (void)inv_cell_sizes; (void)num_pts;
+  MCCNN_REQUIRE(valid_dims(num_dims), "FindNeighbors expects a valid number of dimensions");
+  MCCNN_REQUIRE(num_samples >= 0 && num_neighbors >= 0, "FindNeighbors expects non-negative sizes");
+  if (num_samples == 0 || num_neighbors == 0) return MCCNN_OK;
+  MCCNN_REQUIRE(samples && points && inv_radii && ranges && neighbors_out && workspace,
+                "FindNeighbors received a null tensor");
+  const NbrWorkspace w = carve_nbr_workspace(workspace, num_dims, num_samples);
+  MCCNN_REQUIRE(workspace_bytes >= w.bytes, "FindNeighbors workspace too small (%zu < %zu)",
+                workspace_bytes, w.bytes);
+  const unsigned grid = blocks_for(num_samples, kCentresPerBlock);
+  MCCNN_DIM_SWITCH(num_dims, hipLaunchKernelGGL((nbr_visit_kernel<D, true>), dim3(grid),
+                                                dim3(kNbrThreads), 0, as_stream(stream),
+                                                num_samples, samples, points,
+                                                (const int2 *)w.ranges, inv_radii, max_neighs,
+                                                (int *)nullptr, ranges, (int2 *)neighbors_out));
+  MCCNN_LAUNCH_CHECK();
+  return MCCNN_OK;
+}

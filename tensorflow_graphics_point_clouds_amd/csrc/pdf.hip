@@ -1,0 +1,190 @@
+// Gaussian kernel density per point over its neighbour list and the gradient
+// with respect to the point coordinates
+// (custom_ops/tfg_custom_ops/compute_pdf/cc/kernels/compute_pdf_kernels.cu.cc:72-215).
+//
+// 16 lanes share a centre and stride over its pairs; the pair table is read
+// coalesced, neighbour coordinates are gathered (they sit close together in the
+// sorted array, so the gathers hit L2).  The product over dimensions of
+// exp(-u_d^2/2) is evaluated as one exponential of the summed exponent.
+#include "common.h"
+#include "fill.h"
+
+namespace mccnn {
+
+constexpr int kPdfGroup = 16;
+constexpr int kPdfThreads = 256;
+constexpr int kPdfCentresPerBlock = kPdfThreads / kPdfGroup;
+constexpr float kInvSqrt2Pi = 0.39894228f;
+
+template <int D>
+struct PdfScale {
+  float s[D];     // bw_d * inv_radii_d
+  float norm;     // prod_d bw_d * 0.39894228
+};
+
+template <int D>
+__device__ __forceinline__ PdfScale<D> load_pdf_scale(const float *__restrict__ inv_bw,
+                                                      const float *__restrict__ inv_r, int mode,
+                                                      int64_t n) {
+  PdfScale<D> sc;
+  sc.norm = 1.0f;
+#pragma unroll
+  for (int d = 0; d < D; ++d) {
+    const float bw = mode == 0 ? inv_bw[d] : sqrtf((float)n);
+    sc.s[d] = bw * inv_r[d];
+    sc.norm *= bw * kInvSqrt2Pi;
+  }
+  return sc;
+}
+
+template <int D>
+__global__ void __launch_bounds__(kPdfThreads) compute_pdf_kernel(
+    int64_t n, const float *__restrict__ pts, const int2 *__restrict__ nbrs,
+    const int *__restrict__ ranges, const float *__restrict__ inv_bw,
+    const float *__restrict__ inv_r, int mode, float *__restrict__ pdf) {
+  const PdfScale<D> sc = load_pdf_scale<D>(inv_bw, inv_r, mode, n);
+  const int sub = threadIdx.x & (kPdfGroup - 1);
+  const int64_t c = (int64_t)blockIdx.x * kPdfCentresPerBlock + threadIdx.x / kPdfGroup;
+  if (c >= n) return;
+  float p[D];
+#pragma unroll
+  for (int d = 0; d < D; ++d) p[d] = pts[c * D + d];
+  const int64_t a = c > 0 ? ranges[c - 1] : 0, b = ranges[c];
+  float acc = 0.0f;
+  for (int64_t m = a + sub; m < b; m += kPdfGroup) {
+    const int64_t j = nbrs[m].x;
+    float e = 0.0f;
+#pragma unroll
+    for (int d = 0; d < D; ++d) {
+      const float u = (pts[j * D + d] - p[d]) * sc.s[d];
+      e += u * u;
+    }
+    acc += expf(-0.5f * e);
+  }
+#pragma unroll
+  for (int off = kPdfGroup / 2; off > 0; off >>= 1) acc += __shfl_xor(acc, off, kWave);
+  if (sub == 0) pdf[c] = acc * sc.norm;
+}
+
+// grad[i] += g, grad[j] -= g with g_d = pdf_grad_i * pdf_ij * u_d * s_d.  The
+// centre's own sum is reduced in registers and added once; the neighbour side is
+// one atomic per pair and dimension.
+template <int D>
+__global__ void __launch_bounds__(kPdfThreads) compute_pdf_grads_kernel(
+    int64_t n, const float *__restrict__ pts, const int2 *__restrict__ nbrs,
+    const int *__restrict__ ranges, const float *__restrict__ inv_bw,
+    const float *__restrict__ inv_r, const float *__restrict__ pdf_grads, int mode,
+    float *__restrict__ grads) {
+  const PdfScale<D> sc = load_pdf_scale<D>(inv_bw, inv_r, mode, n);
+  const int sub = threadIdx.x & (kPdfGroup - 1);
+  const int64_t c = (int64_t)blockIdx.x * kPdfCentresPerBlock + threadIdx.x / kPdfGroup;
+  if (c >= n) return;
+  float p[D], own[D];
+#pragma unroll
+  for (int d = 0; d < D; ++d) {
+    p[d] = pts[c * D + d];
+    own[d] = 0.0f;
+  }
+  const float up = pdf_grads[c] * sc.norm;
+  const int64_t a = c > 0 ? ranges[c - 1] : 0, b = ranges[c];
+  for (int64_t m = a + sub; m < b; m += kPdfGroup) {
+    const int64_t j = nbrs[m].x;
+    float u[D], e = 0.0f;
+#pragma unroll
+    for (int d = 0; d < D; ++d) {
+      u[d] = (pts[j * D + d] - p[d]) * sc.s[d];
+      e += u[d] * u[d];
+    }
+    const float local = up * expf(-0.5f * e);
+#pragma unroll
+    for (int d = 0; d < D; ++d) {
+      const float gd = u[d] * sc.s[d] * local;
+      own[d] += gd;
+      if (j != c) unsafeAtomicAdd(&grads[j * D + d], -gd);
+    }
+  }
+#pragma unroll
+  for (int d = 0; d < D; ++d) {
+    float v = own[d];
+#pragma unroll
+    for (int off = kPdfGroup / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+    if (sub == 0) unsafeAtomicAdd(&grads[c * D + d], v);
+  }
+}
+
+static int check_pdf_args(const char *op, int64_t num_pts, int num_dims, int neighbors_rank,
+                          int neighbors_cols, int64_t num_samples, int inv_bandwidth_len,
+                          int inv_radii_len, int mode) {
+  MCCNN_REQUIRE(mode >= 0 && mode < 2, "%s requires a mode between 0 and 1", op);
+  MCCNN_REQUIRE(num_samples == num_pts, "%s expects the same points as samples", op);
+  MCCNN_REQUIRE(valid_dims(num_dims), "%s expects a valid number of dimensions", op);
+  MCCNN_REQUIRE(inv_bandwidth_len == num_dims,
+                "%s expects a number of dimensions in inv_bandwidth equal to the number of "
+                "dimensions in the input points", op);
+  MCCNN_REQUIRE(inv_radii_len == num_dims,
+                "%s expects a number of dimensions in inv_radii equal to the number of dimensions "
+                "in the input points", op);
+  MCCNN_REQUIRE(neighbors_rank == 2 && neighbors_cols == 2,
+                "%s expects a neighbor tensor with 2 dimensions and 2 indices per neighbor", op);
+  return MCCNN_OK;
+}
+
+}  // namespace mccnn
+
+using namespace mccnn;
+
+extern "C" int mccnn_compute_pdf(mccnn_stream_t stream, int64_t num_pts, int num_dims,
+                                 const float *points, int64_t num_neighbors, int neighbors_rank,
+                                 int neighbors_cols, const int32_t *neighbors,
+                                 int64_t num_samples, const int32_t *ranges,
+                                 int inv_bandwidth_len, const float *inv_bandwidth,
+                                 int inv_radii_len, const float *inv_radii, int mode,
+                                 float *pdf_out) {
+  int rc = check_pdf_args("ComputePdf", num_pts, num_dims, neighbors_rank, neighbors_cols,
+                          num_samples, inv_bandwidth_len, inv_radii_len, mode);
+  if (rc != MCCNN_OK) return rc;
+  MCCNN_REQUIRE(num_pts >= 0 && num_neighbors >= 0, "ComputePdf expects non-negative sizes");
+  if (num_pts == 0) return MCCNN_OK;
+  MCCNN_REQUIRE(points && ranges && inv_bandwidth && inv_radii && pdf_out &&
+                    (neighbors || num_neighbors == 0),
+                "ComputePdf received a null tensor");
+  const unsigned grid = blocks_for(num_pts, kPdfCentresPerBlock);
+  MCCNN_DIM_SWITCH(num_dims, hipLaunchKernelGGL(compute_pdf_kernel<D>, dim3(grid),
+                                                dim3(kPdfThreads), 0, as_stream(stream), num_pts,
+                                                points, (const int2 *)neighbors, ranges,
+                                                inv_bandwidth, inv_radii, mode, pdf_out));
+  MCCNN_LAUNCH_CHECK();
+  return MCCNN_OK;
+}
+
+extern "C" int mccnn_compute_pdf_pt_grads(mccnn_stream_t stream, int64_t num_pts, int num_dims,
+                                          const float *points, int64_t num_neighbors,
+                                          int neighbors_rank, int neighbors_cols,
+                                          const int32_t *neighbors, int64_t num_samples,
+                                          const int32_t *ranges, int inv_bandwidth_len,
+                                          const float *inv_bandwidth, int inv_radii_len,
+                                          const float *inv_radii, int64_t pdf_grads_len,
+                                          const float *pdf_grads, int mode,
+                                          float *pt_grads_out) {
+  int rc = check_pdf_args("ComputePdfPtGrads", num_pts, num_dims, neighbors_rank, neighbors_cols,
+                          num_samples, inv_bandwidth_len, inv_radii_len, mode);
+  if (rc != MCCNN_OK) return rc;
+  MCCNN_REQUIRE(pdf_grads_len == num_samples,
+                "ComputePdfPtGrads expects a number of pdf gradients equal to the number of "
+                "samples");
+  MCCNN_REQUIRE(num_pts >= 0 && num_neighbors >= 0, "ComputePdfPtGrads expects non-negative sizes");
+  if (num_pts == 0) return MCCNN_OK;
+  MCCNN_REQUIRE(points && ranges && inv_bandwidth && inv_radii && pdf_grads && pt_grads_out &&
+                    (neighbors || num_neighbors == 0),
+                "ComputePdfPtGrads received a null tensor");
+  hipStream_t s = as_stream(stream);
+  rc = fill_zero(s, pt_grads_out, sizeof(float) * (size_t)num_pts * num_dims);
+  if (rc != MCCNN_OK) return rc;
+  const unsigned grid = blocks_for(num_pts, kPdfCentresPerBlock);
+  MCCNN_DIM_SWITCH(num_dims, hipLaunchKernelGGL(compute_pdf_grads_kernel<D>, dim3(grid),
+                                                dim3(kPdfThreads), 0, s, num_pts, points,
+                                                (const int2 *)neighbors, ranges, inv_bandwidth,
+                                                inv_radii, pdf_grads, mode, pt_grads_out));
+  MCCNN_LAUNCH_CHECK();
+  return MCCNN_OK;
+}

@@ -1,0 +1,206 @@
+// Stable descending radix sort of (cell key, point index) pairs: the sort step
+// of the reference's grid construction (pylib/pc/Grid.py:56-64,
+// tf.argsort(keys, 'DESCENDING'): equal keys keep ascending original index).
+//
+// LSD radix sort, 8-bit digits, on the complemented digit so that ascending
+// digit order is descending key order while stability keeps equal keys in input
+// order.  Per pass: (1) per-tile digit histogram in LDS, written digit-major,
+// (2) prefix sum over [256 digits x tiles], (3) stable scatter: ranks inside a
+// tile come from wavefront ballots (matching lanes with the same digit) plus
+// per-wave LDS counters, never from atomics, so the order is deterministic.
+#include "common.h"
+#include "fill.h"
+
+namespace mccnn {
+
+constexpr int kSortThreads = 256;
+constexpr int kSortItems = 8;
+constexpr int kSortTile = kSortThreads * kSortItems;
+constexpr int kSortWaves = kSortThreads / kWave;
+constexpr int kRadix = 256;
+
+__device__ __forceinline__ int digit_of(int64_t key, int shift) {
+  return (int)((~(uint64_t)key >> shift) & (kRadix - 1));
+}
+
+__global__ void __launch_bounds__(kSortThreads) sort_hist_kernel(
+    int64_t n, int shift, int nb, const int64_t *__restrict__ keys, int *__restrict__ hist) {
+  __shared__ int bins[kRadix];
+  bins[threadIdx.x] = 0;
+  __syncthreads();
+  const int64_t base = (int64_t)blockIdx.x * kSortTile;
+#pragma unroll
+  for (int k = 0; k < kSortItems; ++k) {
+    const int64_t i = base + k * kSortThreads + threadIdx.x;
+    if (i < n) atomicAdd(&bins[digit_of(keys[i], shift)], 1);
+  }
+  __syncthreads();
+  hist[(int64_t)threadIdx.x * nb + blockIdx.x] = bins[threadIdx.x];
+}
+
+// hist holds the INCLUSIVE prefix sums of the digit-major histogram.
+template <bool kFirstPass>
+__global__ void __launch_bounds__(kSortThreads) sort_scatter_kernel(
+    int64_t n, int shift, int nb, const int64_t *__restrict__ keys_in,
+    const int *__restrict__ idx_in, const int *__restrict__ hist,
+    int64_t *__restrict__ keys_out, int *__restrict__ idx_out) {
+  __shared__ int running[kRadix];              // items of each digit seen in earlier rounds
+  __shared__ int wcount[kSortWaves][kRadix];   // per wave, this round
+  const int lane = lane_id(), wave = threadIdx.x / kWave;
+  running[threadIdx.x] = 0;
+#pragma unroll
+  for (int w = 0; w < kSortWaves; ++w) wcount[w][threadIdx.x] = 0;
+  __syncthreads();
+
+  const int64_t base = (int64_t)blockIdx.x * kSortTile;
+  int64_t key[kSortItems];
+  int rank[kSortItems];
+#pragma unroll
+  for (int k = 0; k < kSortItems; ++k) {
+    const int64_t i = base + k * kSortThreads + threadIdx.x;
+    const bool live = i < n;
+    key[k] = live ? keys_in[i] : 0;
+    const int d = digit_of(key[k], shift);
+    // lanes of this wave holding the same digit (dead lanes match nothing)
+    uint64_t same = __ballot(live);
+#pragma unroll
+    for (int bit = 0; bit < 8; ++bit) {
+      const uint64_t b = __ballot((d >> bit) & 1);
+      same &= ((d >> bit) & 1) ? b : ~b;
+    }
+    const int below = __popcll(same & ((1ull << lane) - 1ull));
+    if (live && below == 0) wcount[wave][d] = __popcll(same);
+    __syncthreads();
+    int r = running[d] + below;
+#pragma unroll
+    for (int w = 0; w < kSortWaves; ++w)
+      if (w < wave) r += wcount[w][d];
+    rank[k] = r;
+    __syncthreads();
+    {
+      int add = 0;
+#pragma unroll
+      for (int w = 0; w < kSortWaves; ++w) {
+        add += wcount[w][threadIdx.x];
+        wcount[w][threadIdx.x] = 0;
+      }
+      running[threadIdx.x] += add;
+    }
+    __syncthreads();
+  }
+  // running[d] is now this tile's count of digit d: global start of the tile's
+  // run of digit d = inclusive prefix - count.
+  const int start = hist[(int64_t)threadIdx.x * nb + blockIdx.x] - running[threadIdx.x];
+  __syncthreads();
+  running[threadIdx.x] = start;
+  __syncthreads();
+#pragma unroll
+  for (int k = 0; k < kSortItems; ++k) {
+    const int64_t i = base + k * kSortThreads + threadIdx.x;
+    if (i < n) {
+      const int d = digit_of(key[k], shift);
+      const int64_t dst = (int64_t)running[d] + rank[k];
+      keys_out[dst] = key[k];
+      idx_out[dst] = kFirstPass ? (int)i : idx_in[i];
+    }
+  }
+}
+
+__global__ void __launch_bounds__(256) sort_copy_kernel(int64_t n, const int64_t *__restrict__ keys,
+                                                        int64_t *__restrict__ keys_out,
+                                                        int *__restrict__ idx_out) {
+  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n;
+       i += (int64_t)gridDim.x * blockDim.x) {
+    keys_out[i] = keys[i];
+    idx_out[i] = (int)i;
+  }
+}
+
+struct SortWorkspace {
+  int64_t *keys_tmp;
+  int *idx_tmp;
+  int *hist;
+  int *scan_scratch;
+  int64_t *total;
+  size_t bytes;
+};
+
+static SortWorkspace carve_sort_workspace(void *ws, int64_t n) {
+  const int64_t nb = (n + kSortTile - 1) / kSortTile;
+  char *p = (char *)ws;
+  SortWorkspace w;
+  size_t off = 0;
+  w.keys_tmp = (int64_t *)(p + off);
+  off += align256(sizeof(int64_t) * (size_t)n);
+  w.idx_tmp = (int *)(p + off);
+  off += align256(sizeof(int) * (size_t)n);
+  w.hist = (int *)(p + off);
+  off += align256(sizeof(int) * (size_t)(kRadix * nb));
+  w.scan_scratch = (int *)(p + off);
+  off += align256(sizeof(int) * scan_scratch_ints(kRadix * nb));
+  w.total = (int64_t *)(p + off);
+  off += 256;
+  w.bytes = off;
+  return w;
+}
+
+}  // namespace mccnn
+
+using namespace mccnn;
+
+extern "C" size_t mccnn_sort_keys_workspace_bytes(int64_t num_pts) {
+  if (num_pts < 0) num_pts = 0;
+  return carve_sort_workspace(nullptr, num_pts).bytes;
+}
+
+extern "C" int mccnn_sort_keys_descending(mccnn_stream_t stream, int64_t num_pts, int key_bits,
+                                          const int64_t *keys, int64_t *sorted_keys_out,
+                                          int32_t *sorted_indices_out, void *workspace,
+                                          size_t workspace_bytes) {
+  MCCNN_REQUIRE(num_pts >= 0 && num_pts < ((int64_t)1 << 31),
+                "sort_keys expects 0 <= num_pts < 2^31");
+  MCCNN_REQUIRE(key_bits >= 1 && key_bits <= 64, "sort_keys expects key_bits in [1, 64]");
+  if (num_pts == 0) return MCCNN_OK;
+  MCCNN_REQUIRE(keys && sorted_keys_out && sorted_indices_out && workspace,
+                "sort_keys received a null tensor");
+  MCCNN_REQUIRE((const void *)keys != (const void *)sorted_keys_out,
+                "sort_keys output must not alias the input");
+  const SortWorkspace w = carve_sort_workspace(workspace, num_pts);
+  MCCNN_REQUIRE(workspace_bytes >= w.bytes, "sort_keys workspace too small (%zu < %zu)",
+                workspace_bytes, w.bytes);
+  hipStream_t s = as_stream(stream);
+  const int passes = (key_bits + 7) / 8;
+  const int nb = (int)((num_pts + kSortTile - 1) / kSortTile);
+  // Ping-pong so that the last pass lands in the caller's buffers.
+  int64_t *kbuf[2];
+  int *ibuf[2];
+  if (passes % 2 == 1) {
+    kbuf[0] = (int64_t *)sorted_keys_out; ibuf[0] = sorted_indices_out;
+    kbuf[1] = w.keys_tmp;                 ibuf[1] = w.idx_tmp;
+  } else {
+    kbuf[0] = w.keys_tmp;                 ibuf[0] = w.idx_tmp;
+    kbuf[1] = (int64_t *)sorted_keys_out; ibuf[1] = sorted_indices_out;
+  }
+  const int64_t *kin = (const int64_t *)keys;
+  const int *iin = nullptr;
+  for (int p = 0; p < passes; ++p) {
+    const int shift = 8 * p;
+    int64_t *kout = kbuf[p & 1];
+    int *iout = ibuf[p & 1];
+    hipLaunchKernelGGL(sort_hist_kernel, dim3(nb), dim3(kSortThreads), 0, s, num_pts, shift, nb,
+                       kin, w.hist);
+    MCCNN_LAUNCH_CHECK();
+    int rc = inclusive_scan_i32(s, (int64_t)kRadix * nb, w.hist, w.scan_scratch, w.total);
+    if (rc != MCCNN_OK) return rc;
+    if (p == 0)
+      hipLaunchKernelGGL(sort_scatter_kernel<true>, dim3(nb), dim3(kSortThreads), 0, s, num_pts,
+                         shift, nb, kin, iin, w.hist, kout, iout);
+    else
+      hipLaunchKernelGGL(sort_scatter_kernel<false>, dim3(nb), dim3(kSortThreads), 0, s, num_pts,
+                         shift, nb, kin, iin, w.hist, kout, iout);
+    MCCNN_LAUNCH_CHECK();
+    kin = kout;
+    iin = iout;
+  }
+  return MCCNN_OK;
+}

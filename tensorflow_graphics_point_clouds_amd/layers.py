@@ -1,0 +1,260 @@
+"""Convolution and pooling layers composed from the HIP ops, with the call
+signatures of the reference's layers (pylib/pc/layers/MCConv.py, KPConv.py,
+Pooling.py).  Per-pair basis evaluation, basis projection, pooling and all
+their gradients are kernels of libmccnn_hip.so; the dense
+[N, C*K] x [C*K, C_out] product is a plain library GEMM (torch.matmul)."""
+import math
+
+import torch
+
+from . import _lib, pc, tfg_custom_ops
+from ._lib import cfloat, cint, i64, ptr, stream
+
+_F32, _I32 = torch.float32, torch.int32
+
+_ACTIVATIONS = {"relu": 0, "lrelu": 1, "leakyrelu": 1, "leaky_relu": 1, "elu": 2}
+
+
+class _MCBasis(torch.autograd.Function):
+    """basis[m, l*H + h] = act(delta_m . W[l,:,h] + b[l,h]) / pdf[m]
+    (MCConv.py:163-171); differentiable in the kernel weights and biases."""
+
+    @staticmethod
+    def forward(ctx, weights, biases, points_in, points_out, neighbors, inv_radii, pdf, act):
+        num_mlps, dims, hidden = weights.shape
+        k = num_mlps * hidden
+        basis = torch.empty((neighbors.shape[0], k), dtype=_F32, device=weights.device)
+        _lib.check(_lib.lib().mccnn_mc_basis(
+            stream(), i64(neighbors.shape[0]), cint(dims), cint(k), cint(act),
+            ptr(points_in, _F32), ptr(points_out, _F32), ptr(neighbors, _I32),
+            ptr(inv_radii, _F32), ptr(weights, _F32), ptr(biases, _F32), cint(num_mlps),
+            ptr(pdf, _F32), ptr(basis)))
+        ctx.save_for_backward(weights, biases, points_in, points_out, neighbors, inv_radii, pdf)
+        ctx.act = act
+        return basis
+
+    @staticmethod
+    def backward(ctx, grad):
+        weights, biases, points_in, points_out, neighbors, inv_radii, pdf = ctx.saved_tensors
+        num_mlps, dims, hidden = weights.shape
+        k = num_mlps * hidden
+        L = _lib.lib()
+        ws = _lib.workspace(L.mccnn_mc_basis_grads_workspace_bytes(cint(dims), cint(k)),
+                            weights.device)
+        dw, db = torch.empty_like(weights), torch.empty_like(biases)
+        _lib.check(L.mccnn_mc_basis_grads(
+            stream(), i64(neighbors.shape[0]), cint(dims), cint(k), cint(ctx.act),
+            ptr(points_in, _F32), ptr(points_out, _F32), ptr(neighbors, _I32),
+            ptr(inv_radii, _F32), ptr(weights, _F32), ptr(biases, _F32), cint(num_mlps),
+            ptr(pdf, _F32), ptr(grad.contiguous(), _F32), ptr(ws), _lib.csize(ws.numel()),
+            ptr(dw), ptr(db)))
+        return dw, db, None, None, None, None, None, None
+
+
+def _truncated_normal(shape, std, generator, device):
+    t = torch.empty(shape, dtype=_F32)
+    torch.nn.init.trunc_normal_(t, mean=0.0, std=std, a=-2 * std, b=2 * std,
+                                generator=generator)
+    return t.to(device)
+
+
+class MCConv(torch.nn.Module):
+    """Monte-Carlo convolution (pylib/pc/layers/MCConv.py:35-278) with a
+    one-hidden-layer kernel MLP per output group."""
+
+    def __init__(self, num_features_in, num_features_out, num_dims, num_mlps=4, mlp_size=(8,),
+                 non_linearity_type="leaky_relu", weights=None, biases=None,
+                 final_weights=None, device="cuda", seed=0):
+        super().__init__()
+        if num_features_out % num_mlps != 0:
+            raise ValueError("The number of output features must be divisible by the number"
+                             " of kernel MLPs")
+        if len(mlp_size) != 1:
+            raise NotImplementedError("only one hidden layer is evaluated by the HIP kernel")
+        hidden = int(mlp_size[0])
+        self._num_features_in, self._num_features_out = num_features_in, num_features_out
+        self._num_dims, self._num_mlps, self._hidden = num_dims, num_mlps, hidden
+        self._act = _ACTIVATIONS[non_linearity_type.lower()]
+        gen = torch.Generator().manual_seed(seed)
+        if weights is None:      # MCConv.py:100-135: truncated normal, He scale
+            weights = _truncated_normal((num_mlps, num_dims, hidden),
+                                        math.sqrt(2.0 / num_dims), gen, device)
+        if biases is None:
+            biases = torch.zeros((num_mlps, 1, hidden), dtype=_F32, device=device)
+        if final_weights is None:
+            final_weights = _truncated_normal(
+                (num_mlps, hidden * num_features_in, num_features_out // num_mlps),
+                math.sqrt(2.0 / (hidden * num_features_in)), gen, device)
+        self.weights = torch.nn.Parameter(weights.to(_F32).contiguous())
+        self.biases = torch.nn.Parameter(biases.to(_F32).contiguous())
+        self.final_weights = torch.nn.Parameter(final_weights.to(_F32).contiguous())
+        self.last_neighborhood = None
+
+    def forward(self, features, point_cloud_in, point_cloud_out, radius, neighborhood=None,
+                bandwidth=0.2):
+        d = self._num_dims
+        dev = features.device
+        radii = pc._as_vector(radius, d, dev)
+        if neighborhood is None:
+            grid = pc.Grid(point_cloud_in, radii)
+            neighborhood = pc.Neighborhood(grid, radii, point_cloud_out)
+        self.last_neighborhood = neighborhood
+        pdf = neighborhood.get_pdf(bandwidth=bandwidth, mode=pc.KDEMode.constant)
+        basis = _MCBasis.apply(self.weights, self.biases.reshape(self._num_mlps, self._hidden),
+                               point_cloud_in._points, point_cloud_out._points,
+                               neighborhood._original_neigh_ids, torch.reciprocal(radii), pdf,
+                               self._act)
+        proj = tfg_custom_ops.basis_proj(basis, features.contiguous(),
+                                         neighborhood._original_neigh_ids,
+                                         neighborhood._samples_neigh_ranges)
+        n, c, l, h = proj.shape[0], self._num_features_in, self._num_mlps, self._hidden
+        if l == 1:
+            return proj.reshape(n, c * h) @ self.final_weights[0]
+        p = proj.reshape(n, c, l, h).permute(2, 0, 1, 3).reshape(l, n, c * h)
+        return torch.bmm(p, self.final_weights).permute(1, 0, 2).reshape(n, -1)
+
+
+def _padded_basis_count(num_kernel_points):
+    for k in (8, 16, 32, 64):
+        if num_kernel_points <= k:
+            return k
+    raise ValueError("at most 64 kernel points are supported")
+
+
+class KPConv(torch.nn.Module):
+    """Rigid kernel-point convolution (pylib/pc/layers/KPConv.py:60-315).  The
+    kernel points are scaled by 0.75 as in the reference (:131); `kernel_points`
+    is [K, D] in units of the convolution radius."""
+
+    def __init__(self, num_features_in, num_features_out, kernel_points, num_dims=3,
+                 kernel_weighting="linear", weights=None, device="cuda", seed=0):
+        super().__init__()
+        kp = torch.as_tensor(kernel_points, dtype=_F32).to(device) * 0.75
+        self._kernel_points = kp.contiguous()
+        self._num_kernel_points = kp.shape[0]
+        self._num_basis = _padded_basis_count(kp.shape[0])
+        self._kind = {"linear": 0, "gaussian": 1}[kernel_weighting]
+        self._num_features_in, self._num_features_out = num_features_in, num_features_out
+        self._num_dims = num_dims
+        if weights is None:      # Glorot normal as KPConv.py:133-160
+            gen = torch.Generator().manual_seed(seed)
+            fan_in, fan_out = self._num_kernel_points * num_features_in, num_features_out
+            weights = (torch.randn((fan_in, fan_out), generator=gen) *
+                       math.sqrt(2.0 / (fan_in + fan_out))).to(device)
+        self.weights = torch.nn.Parameter(weights.to(_F32).contiguous())
+        self.last_neighborhood = None
+
+    def forward(self, features, point_cloud_in, point_cloud_out, conv_radius, neighborhood=None,
+                kernel_influence_dist=None):
+        d, dev = self._num_dims, features.device
+        sigma = 1.0 if kernel_influence_dist is None else float(kernel_influence_dist) / float(
+            conv_radius)
+        radii = pc._as_vector(conv_radius, d, dev)
+        if neighborhood is None:
+            grid = pc.Grid(point_cloud_in, radii)
+            neighborhood = pc.Neighborhood(grid, radii, point_cloud_out)
+        self.last_neighborhood = neighborhood
+        ids = neighborhood._original_neigh_ids
+        kp, k = self._num_kernel_points, self._num_basis
+        basis = torch.empty((ids.shape[0], k), dtype=_F32, device=dev)
+        _lib.check(_lib.lib().mccnn_kp_basis(
+            stream(), i64(ids.shape[0]), cint(d), cint(kp), cint(k), cint(self._kind),
+            cfloat(sigma), ptr(point_cloud_in._points, _F32), ptr(point_cloud_out._points, _F32),
+            ptr(ids, _I32), ptr(torch.reciprocal(radii), _F32), ptr(self._kernel_points, _F32),
+            ptr(None), ptr(basis), ptr(None)))
+        proj = tfg_custom_ops.basis_proj(basis, features.contiguous(), ids,
+                                         neighborhood._samples_neigh_ranges)
+        c = self._num_features_in
+        if k == kp:
+            return proj.reshape(-1, c * k) @ self.weights
+        # zero rows for the padded basis columns instead of slicing the projection
+        w = torch.nn.functional.pad(self.weights.reshape(c, kp, -1), (0, 0, 0, k - kp))
+        return proj.reshape(-1, c * k) @ w.reshape(c * k, -1)
+
+
+class _LocalPool(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, features, neighbors, ranges, kind):
+        out = torch.empty((ranges.shape[0], features.shape[1]), dtype=_F32,
+                          device=features.device)
+        _lib.check(_lib.lib().mccnn_local_pool(
+            stream(), cint(kind), i64(features.shape[0]), cint(features.shape[1]),
+            ptr(features, _F32), i64(neighbors.shape[0]), ptr(neighbors, _I32),
+            i64(ranges.shape[0]), ptr(ranges, _I32), ptr(out)))
+        ctx.save_for_backward(features, neighbors, ranges, out)
+        ctx.kind = kind
+        return out
+
+    @staticmethod
+    def backward(ctx, grad):
+        features, neighbors, ranges, out = ctx.saved_tensors
+        dfeat = torch.empty_like(features)
+        _lib.check(_lib.lib().mccnn_local_pool_grads(
+            stream(), cint(ctx.kind), i64(features.shape[0]), cint(features.shape[1]),
+            ptr(features, _F32), i64(neighbors.shape[0]), ptr(neighbors, _I32),
+            i64(ranges.shape[0]), ptr(ranges, _I32), ptr(out, _F32),
+            ptr(grad.contiguous(), _F32), ptr(dfeat)))
+        return dfeat, None, None, None
+
+
+class _LocalPointPooling:
+    kind = 0
+
+    def __call__(self, features, point_cloud_in, point_cloud_out, pooling_radius,
+                 neighborhood=None):
+        if neighborhood is None:
+            radii = pc._as_vector(pooling_radius, point_cloud_in._dimension, features.device)
+            grid = pc.Grid(point_cloud_in, radii)
+            neighborhood = pc.Neighborhood(grid, radii, point_cloud_out)
+        return _LocalPool.apply(features.contiguous(), neighborhood._original_neigh_ids,
+                                neighborhood._samples_neigh_ranges, self.kind)
+
+
+class MaxPooling(_LocalPointPooling):
+    """pylib/pc/layers/Pooling.py:169-206."""
+    kind = 0
+
+
+class AveragePooling(_LocalPointPooling):
+    """pylib/pc/layers/Pooling.py:209-246."""
+    kind = 1
+
+
+class _GlobalPool(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, features, batch_ids, batch_size, kind):
+        out = torch.empty((batch_size, features.shape[1]), dtype=_F32, device=features.device)
+        counts = torch.empty(batch_size, dtype=_I32, device=features.device)
+        _lib.check(_lib.lib().mccnn_global_pool(
+            stream(), cint(kind), i64(features.shape[0]), cint(features.shape[1]),
+            ptr(features, _F32), ptr(batch_ids, _I32), cint(batch_size), ptr(out), ptr(counts)))
+        ctx.save_for_backward(features, batch_ids, out, counts)
+        ctx.kind, ctx.batch_size = kind, batch_size
+        return out
+
+    @staticmethod
+    def backward(ctx, grad):
+        features, batch_ids, out, counts = ctx.saved_tensors
+        dfeat = torch.empty_like(features)
+        tie = torch.empty_like(out) if ctx.kind == 0 else None
+        _lib.check(_lib.lib().mccnn_global_pool_grads(
+            stream(), cint(ctx.kind), i64(features.shape[0]), cint(features.shape[1]),
+            ptr(features, _F32), ptr(batch_ids, _I32), cint(ctx.batch_size), ptr(out, _F32),
+            ptr(counts, _I32), ptr(grad.contiguous(), _F32), ptr(tie), ptr(dfeat)))
+        return dfeat, None, None, None
+
+
+class GlobalMaxPooling:
+    """pylib/pc/layers/Pooling.py:25-61."""
+
+    def __call__(self, features, point_cloud):
+        return _GlobalPool.apply(features.contiguous(), point_cloud._batch_ids,
+                                 point_cloud._batch_size, 0)
+
+
+class GlobalAveragePooling:
+    """pylib/pc/layers/Pooling.py:64-104."""
+
+    def __call__(self, features, point_cloud):
+        return _GlobalPool.apply(features.contiguous(), point_cloud._batch_ids,
+                                 point_cloud._batch_size, 1)

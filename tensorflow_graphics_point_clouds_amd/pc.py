@@ -1,0 +1,190 @@
+"""Thin counterparts of the reference's callers of the op path, on torch GPU
+tensors: `PointCloud` (segmented form only), `Grid`, `Neighborhood`, `sample`
+and `PointHierarchy` (pylib/pc/PointCloud.py, Grid.py, Neighborhood.py,
+sampling.py, PointHierarchy.py).  They only arrange arguments: bounding boxes,
+grid shape, sort and gathers are kernels of libmccnn_hip.so as well.
+"""
+import ctypes
+import enum
+
+import torch
+
+from . import _lib, tfg_custom_ops
+from ._lib import cint, i64, ptr, stream
+
+_F32, _I32, _I64 = torch.float32, torch.int32, torch.int64
+
+
+class KDEMode(enum.Enum):
+    """pylib/pc/Neighborhood.py: constant bandwidth, bandwidth from the number of
+    points, or no density estimate."""
+    constant = 0
+    num_points = 1
+    no_pdf = 2
+
+
+def _as_vector(value, dims, device):
+    t = torch.as_tensor(value, dtype=_F32).reshape(-1)
+    if t.numel() == 1:
+        t = t.repeat(dims)
+    return t.to(device).contiguous()
+
+
+class PointCloud:
+    """Points [N, D] with a batch id per point (pylib/pc/PointCloud.py:68-134,
+    segmented input)."""
+
+    def __init__(self, points, batch_ids, batch_size=None):
+        self._points = torch.as_tensor(points, dtype=_F32).contiguous()
+        self._batch_ids = torch.as_tensor(batch_ids, dtype=_I32,
+                                          device=self._points.device).contiguous()
+        if self._points.dim() != 2 or self._batch_ids.shape[0] != self._points.shape[0]:
+            raise ValueError("expected points [N, D] and batch_ids [N]")
+        if batch_size is None:
+            batch_size = int(self._batch_ids.max().item()) + 1
+        self._batch_size = int(batch_size)
+        self._dimension = self._points.shape[1]
+
+
+class Grid:
+    """Regular grid over a point cloud (pylib/pc/Grid.py:32-84): grid shape from
+    the per-cloud bounding boxes, cell keys, stable descending sort, gathers."""
+
+    def __init__(self, point_cloud, cell_sizes):
+        L = _lib.lib()
+        pc = point_cloud
+        dev, n, d, b = pc._points.device, pc._points.shape[0], pc._dimension, pc._batch_size
+        self._point_cloud = pc
+        self._batch_size = b
+        self._cell_sizes = _as_vector(cell_sizes, d, dev)
+        self._aabb_min = torch.empty((b, d), dtype=_F32, device=dev)
+        self._aabb_max = torch.empty((b, d), dtype=_F32, device=dev)
+        self._num_cells = torch.empty(d, dtype=_I32, device=dev)
+        self._scaled_aabb_min = torch.empty((b, d), dtype=_F32, device=dev)
+        self._inv_cell_sizes = torch.empty(d, dtype=_F32, device=dev)
+        _lib.check(L.mccnn_grid_setup(
+            stream(), i64(n), cint(d), ptr(pc._points, _F32), ptr(pc._batch_ids, _I32), cint(b),
+            ptr(self._cell_sizes), ptr(self._aabb_min), ptr(self._aabb_max),
+            ptr(self._num_cells), ptr(self._scaled_aabb_min), ptr(self._inv_cell_sizes)))
+        self._cur_keys = tfg_custom_ops.compute_keys(
+            pc._points, pc._batch_ids, self._scaled_aabb_min, self._num_cells,
+            self._inv_cell_sizes)
+        # host copy of the grid shape: sizes the key width and the column table
+        self._num_cells_host = [int(v) for v in self._num_cells.tolist()]
+        total = b
+        for v in self._num_cells_host:
+            total *= v
+        key_bits = max(1, (total - 1).bit_length())
+        self._sorted_keys = torch.empty(n, dtype=_I64, device=dev)
+        self._sorted_indices = torch.empty(n, dtype=_I32, device=dev)
+        ws = _lib.workspace(L.mccnn_sort_keys_workspace_bytes(i64(n)), dev)
+        _lib.check(L.mccnn_sort_keys_descending(
+            stream(), i64(n), cint(key_bits), ptr(self._cur_keys), ptr(self._sorted_keys),
+            ptr(self._sorted_indices), ptr(ws), _lib.csize(ws.numel())))
+        self._sorted_points = torch.empty_like(pc._points)
+        self._sorted_batch_ids = torch.empty_like(pc._batch_ids)
+        _lib.check(L.mccnn_gather_points(
+            stream(), i64(n), cint(d), ptr(pc._points), ptr(pc._batch_ids),
+            ptr(self._sorted_indices), ptr(self._sorted_points), ptr(self._sorted_batch_ids)))
+        self._fast_DS = None
+
+    def get_DS(self):
+        if self._fast_DS is None:
+            self._fast_DS = tfg_custom_ops.build_grid_ds(
+                self._sorted_keys, self._num_cells, self._num_cells_host, self._batch_size)
+        return self._fast_DS
+
+
+class Neighborhood:
+    """Neighbour pairs of the centres `point_cloud_sample` (default: the grid's
+    own sorted points) inside `grid` (pylib/pc/Neighborhood.py:218-311)."""
+
+    def __init__(self, grid, radius, point_cloud_sample=None, max_neighbors=0):
+        d = grid._point_cloud._dimension
+        dev = grid._sorted_points.device
+        self._radii = _as_vector(radius, d, dev)
+        self._grid = grid
+        if point_cloud_sample is None:
+            self._equal_samples = True
+            self._point_cloud_sampled = PointCloud(grid._sorted_points, grid._sorted_batch_ids,
+                                                   grid._batch_size)
+        else:
+            self._equal_samples = False
+            self._point_cloud_sampled = point_cloud_sample
+        self.max_neighbors = max_neighbors
+        self._inv_radii = torch.reciprocal(self._radii)
+        s = self._point_cloud_sampled
+        self._samples_neigh_ranges, self._neighbors = tfg_custom_ops.find_neighbors(
+            s._points, s._batch_ids, grid._sorted_points, grid._sorted_keys, grid.get_DS(),
+            grid._num_cells, grid._scaled_aabb_min, grid._inv_cell_sizes, self._inv_radii,
+            max_neighbors)
+        # pairs addressed by original point ids (Neighborhood.py:246-250)
+        self._original_neigh_ids = torch.empty_like(self._neighbors)
+        _lib.check(_lib.lib().mccnn_original_neighbor_ids(
+            stream(), i64(self._neighbors.shape[0]), ptr(self._neighbors, _I32),
+            ptr(grid._sorted_indices, _I32), ptr(self._original_neigh_ids)))
+        self._pdf = None
+        self._pdf_per_point = None
+
+    def compute_pdf(self, bandwidth=0.2, mode=KDEMode.constant, normalize=False):
+        d = self._grid._point_cloud._dimension
+        dev = self._neighbors.device
+        if mode == KDEMode.no_pdf:
+            self._pdf = torch.ones(self._neighbors.shape[0], dtype=_F32, device=dev)
+        else:
+            nbh = self if self._equal_samples else Neighborhood(self._grid, self._radii, None)
+            bw = _as_vector(bandwidth, d, dev)
+            self._pdf_per_point = tfg_custom_ops.compute_pdf_with_pt_grads(
+                self._grid._sorted_points, nbh._neighbors, nbh._samples_neigh_ranges,
+                torch.reciprocal(bw), nbh._inv_radii, mode.value)
+            self._pdf = torch.empty(self._neighbors.shape[0], dtype=_F32, device=dev)
+            _lib.check(_lib.lib().mccnn_gather_pdf(
+                stream(), i64(self._neighbors.shape[0]), ptr(self._neighbors, _I32),
+                ptr(self._pdf_per_point.detach(), _F32), ptr(self._pdf)))
+        if normalize:
+            raise NotImplementedError("normalised densities are not part of the op path")
+
+    def get_pdf(self, **kwargs):
+        if self._pdf is None:
+            self.compute_pdf(**kwargs)
+        return self._pdf
+
+
+_SAMPLE_MODES = {"average": 1, "cell average": 1, "cell_average": 1,
+                 "poisson": 0, "poisson disk": 0, "poisson_disk": 0}
+
+
+def sample(neighborhood, sample_mode="poisson"):
+    """pylib/pc/sampling.py:123-150 -> (PointCloud, original indices or None)."""
+    mode = _SAMPLE_MODES[sample_mode.lower()]
+    g = neighborhood._grid
+    pts, bids, idx = tfg_custom_ops.sampling(
+        g._sorted_points, g._sorted_batch_ids, g._sorted_keys, g._num_cells,
+        neighborhood._neighbors, neighborhood._samples_neigh_ranges, mode)
+    original = None
+    if mode == 0:
+        original = torch.empty_like(idx)
+        _lib.check(_lib.lib().mccnn_gather_i32(
+            stream(), i64(idx.shape[0]), ptr(g._sorted_indices, _I32), ptr(idx, _I32),
+            ptr(original)))
+    return PointCloud(pts, bids, g._batch_size), original
+
+
+class PointHierarchy:
+    """Successively sampled point clouds (pylib/pc/PointHierarchy.py:40-98)."""
+
+    def __init__(self, point_cloud, cell_sizes, sample_mode="poisson"):
+        self._point_clouds = [point_cloud]
+        self._cell_sizes = []
+        self._neighborhoods = []
+        self._sample_indices = []
+        cur = point_cloud
+        for cs in cell_sizes:
+            cs = _as_vector(cs, point_cloud._dimension, point_cloud._points.device)
+            self._cell_sizes.append(cs)
+            grid = Grid(cur, cs)
+            nbh = Neighborhood(grid, cs)
+            cur, idx = sample(nbh, sample_mode)
+            self._neighborhoods.append(nbh)
+            self._point_clouds.append(cur)
+            self._sample_indices.append(idx)

@@ -1,0 +1,211 @@
+"""The eight entry points of the reference's native op package
+(custom_ops/tfg_custom_ops/__init__.py:16-26), on torch GPU tensors, with the
+positional argument order of the reference's REGISTER_OP declarations.  Each
+function forwards to one or two C-ABI calls of libmccnn_hip.so on torch's
+current stream; nothing is computed in Python or torch.
+
+Gradients mirror custom_ops_wrapper.py:159-169 and :192-198: `basis_proj` and
+`compute_pdf_with_pt_grads` are differentiable (basis and features / points),
+the other ops are not.
+"""
+import torch
+
+from .. import _lib
+from .._lib import InvalidArgumentError, cint, i64, ptr, stream, vptr
+
+__all__ = ["compute_keys", "build_grid_ds", "find_neighbors", "sampling",
+           "compute_pdf_with_pt_grads", "compute_pdf_pt_grads", "basis_proj",
+           "basis_proj_grads", "InvalidArgumentError"]
+
+_F32, _I32, _I64 = torch.float32, torch.int32, torch.int64
+
+
+def _dim(t, axis, default=-1):
+    return t.shape[axis] if t.dim() > axis else default
+
+
+def compute_keys(points, batch_ids, scaled_aabb_min, num_cells, inv_cell_sizes):
+    """ComputeKeys (compute_keys_ops.cpp:29-41): int64 cell key per point."""
+    keys = torch.empty(points.shape[0], dtype=_I64, device=points.device)
+    _lib.check(_lib.lib().mccnn_compute_keys(
+        stream(), i64(points.shape[0]), cint(_dim(points, 1)), ptr(points, _F32),
+        i64(batch_ids.shape[0]), ptr(batch_ids, _I32),
+        i64(scaled_aabb_min.shape[0]), cint(_dim(scaled_aabb_min, 1)),
+        ptr(scaled_aabb_min, _F32), cint(num_cells.shape[0]), ptr(num_cells, _I32),
+        cint(inv_cell_sizes.shape[0]), ptr(inv_cell_sizes, _F32), ptr(keys)))
+    return keys
+
+
+def build_grid_ds(sorted_keys, num_cells, num_cells_host, batch_size):
+    """BuildGridDs (build_grid_ds_ops.cpp:27-40): [B, n0, n1, 2] column table.
+    `num_cells_host` is the host copy (list / CPU tensor / numpy) that sizes it."""
+    host = [int(v) for v in (num_cells_host.tolist() if hasattr(num_cells_host, "tolist")
+                             else num_cells_host)]
+    if batch_size <= 0:
+        raise InvalidArgumentError("BuildGridDs requires a positive batch size")
+    if len(host) < 2:
+        raise InvalidArgumentError("BuildGridDs expects a valid number of dimensions")
+    import ctypes
+    host_arr = (ctypes.c_int32 * len(host))(*host)
+    ds = torch.empty((batch_size, host[0], host[1], 2), dtype=_I32, device=sorted_keys.device)
+    _lib.check(_lib.lib().mccnn_build_grid_ds(
+        stream(), i64(sorted_keys.shape[0]), ptr(sorted_keys, _I64), cint(num_cells.shape[0]),
+        ptr(num_cells, _I32), cint(len(host)), host_arr, cint(batch_size), ptr(ds)))
+    return ds
+
+
+def find_neighbors(samples, samples_batch_ids, points, point_keys, grid_acc_ds, num_cells,
+                   scaled_aabb_min, inv_cell_sizes, inv_radii, max_neighs=0):
+    """FindNeighbors (find_neighbors_ops.cpp:42-61) -> (ranges [N_out] inclusive
+    end offsets, neighbors [M, 2] rows (sorted point index, centre index))."""
+    import ctypes
+    L = _lib.lib()
+    ns, nd = samples.shape[0], _dim(samples, 1)
+    dev = samples.device
+    ws_bytes = L.mccnn_find_neighbors_workspace_bytes(cint(nd), i64(ns))
+    ws = _lib.workspace(ws_bytes, dev)
+    ranges = torch.empty(ns, dtype=_I32, device=dev)
+    total = ctypes.c_int64(0)
+    dsr = grid_acc_ds.dim()
+    _lib.check(L.mccnn_find_neighbors_count(
+        stream(), i64(ns), cint(nd), ptr(samples, _F32), i64(samples_batch_ids.shape[0]),
+        ptr(samples_batch_ids, _I32), i64(points.shape[0]), cint(_dim(points, 1)),
+        ptr(points, _F32), i64(point_keys.shape[0]), ptr(point_keys, _I64), cint(dsr),
+        cint(_dim(grid_acc_ds, 0)), cint(_dim(grid_acc_ds, 1)), cint(_dim(grid_acc_ds, 2)),
+        cint(_dim(grid_acc_ds, 3)), ptr(grid_acc_ds, _I32), cint(num_cells.shape[0]),
+        ptr(num_cells, _I32), cint(_dim(scaled_aabb_min, 1)), ptr(scaled_aabb_min, _F32),
+        cint(inv_cell_sizes.shape[0]), ptr(inv_cell_sizes, _F32), cint(inv_radii.shape[0]),
+        ptr(inv_radii, _F32), cint(max_neighs), ptr(ws), _lib.csize(ws.numel()), ptr(ranges),
+        ctypes.byref(total)))
+    m = int(total.value)
+    neighbors = torch.empty((m, 2), dtype=_I32, device=dev)
+    _lib.check(L.mccnn_find_neighbors_fill(
+        stream(), i64(ns), cint(nd), ptr(samples, _F32), ptr(samples_batch_ids, _I32),
+        i64(points.shape[0]), ptr(points, _F32), ptr(point_keys, _I64), ptr(grid_acc_ds, _I32),
+        ptr(num_cells, _I32), ptr(scaled_aabb_min, _F32), ptr(inv_cell_sizes, _F32),
+        ptr(inv_radii, _F32), cint(max_neighs), ptr(ws), _lib.csize(ws.numel()), ptr(ranges),
+        i64(m), ptr(neighbors)))
+    return ranges, neighbors
+
+
+def sampling(points, batch_ids, point_keys, num_cells, neighbors, sample_neigh_indices, mode):
+    """Sampling (sampling_ops.cpp:33-53): mode 0 Poisson disk, mode 1 cell average.
+    -> (sample_pts [S, D], sample_batch_ids [S], sample_indices [S])."""
+    import ctypes
+    L = _lib.lib()
+    n, nd = points.shape[0], _dim(points, 1)
+    dev = points.device
+    ws = _lib.workspace(L.mccnn_sampling_workspace_bytes(i64(n)), dev)
+    total = ctypes.c_int64(0)
+    _lib.check(L.mccnn_sampling_count(
+        stream(), cint(mode), i64(n), cint(nd), ptr(points, _F32), i64(batch_ids.shape[0]),
+        ptr(batch_ids, _I32), i64(point_keys.shape[0]), ptr(point_keys, _I64),
+        cint(num_cells.shape[0]), ptr(num_cells, _I32), i64(neighbors.shape[0]),
+        cint(neighbors.dim()), cint(_dim(neighbors, 1)), ptr(neighbors, _I32),
+        i64(sample_neigh_indices.shape[0]), ptr(sample_neigh_indices, _I32), ptr(ws),
+        _lib.csize(ws.numel()), ctypes.byref(total)))
+    s = int(total.value)
+    out_pts = torch.empty((s, nd), dtype=_F32, device=dev)
+    out_bids = torch.empty(s, dtype=_I32, device=dev)
+    out_idx = torch.empty(s, dtype=_I32, device=dev)
+    _lib.check(L.mccnn_sampling_fill(
+        stream(), cint(mode), i64(n), cint(nd), ptr(points, _F32), ptr(batch_ids, _I32),
+        ptr(point_keys, _I64), ptr(num_cells, _I32), ptr(ws), _lib.csize(ws.numel()), i64(s),
+        ptr(out_pts), ptr(out_bids), ptr(out_idx)))
+    return out_pts, out_bids, out_idx
+
+
+def _compute_pdf_raw(points, neighbors, ranges, inv_bandwidth, inv_radii, mode):
+    pdf = torch.empty(ranges.shape[0], dtype=_F32, device=points.device)
+    _lib.check(_lib.lib().mccnn_compute_pdf(
+        stream(), i64(points.shape[0]), cint(_dim(points, 1)), ptr(points, _F32),
+        i64(neighbors.shape[0]), cint(neighbors.dim()), cint(_dim(neighbors, 1)),
+        ptr(neighbors, _I32), i64(ranges.shape[0]), ptr(ranges, _I32),
+        cint(inv_bandwidth.shape[0]), ptr(inv_bandwidth, _F32), cint(inv_radii.shape[0]),
+        ptr(inv_radii, _F32), cint(mode), ptr(pdf)))
+    return pdf
+
+
+def compute_pdf_pt_grads(points, neighbors, sample_neigh_indices, inv_bandwidth, inv_radii,
+                         pdf_grads, mode):
+    """ComputePdfPtGrads (compute_pdf_ops.cpp:58-74): [N, D] gradient of
+    sum(pdf_grads * pdf) with respect to the points."""
+    out = torch.empty_like(points)
+    _lib.check(_lib.lib().mccnn_compute_pdf_pt_grads(
+        stream(), i64(points.shape[0]), cint(_dim(points, 1)), ptr(points, _F32),
+        i64(neighbors.shape[0]), cint(neighbors.dim()), cint(_dim(neighbors, 1)),
+        ptr(neighbors, _I32), i64(sample_neigh_indices.shape[0]),
+        ptr(sample_neigh_indices, _I32), cint(inv_bandwidth.shape[0]),
+        ptr(inv_bandwidth, _F32), cint(inv_radii.shape[0]), ptr(inv_radii, _F32),
+        i64(pdf_grads.shape[0]), ptr(pdf_grads, _F32), cint(mode), ptr(out)))
+    return out
+
+
+class _ComputePdf(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, points, neighbors, ranges, inv_bandwidth, inv_radii, mode):
+        ctx.save_for_backward(points, neighbors, ranges, inv_bandwidth, inv_radii)
+        ctx.mode = mode
+        return _compute_pdf_raw(points, neighbors, ranges, inv_bandwidth, inv_radii, mode)
+
+    @staticmethod
+    def backward(ctx, grad):
+        points, neighbors, ranges, inv_bandwidth, inv_radii = ctx.saved_tensors
+        g = compute_pdf_pt_grads(points, neighbors, ranges, inv_bandwidth, inv_radii,
+                                 grad.contiguous(), ctx.mode)
+        return g, None, None, None, None, None
+
+
+def compute_pdf_with_pt_grads(points, neighbors, sample_neigh_indices, inv_bandwidth,
+                              inv_radii, mode):
+    """ComputePdfWithPtGrads (compute_pdf_ops.cpp:43-56): Gaussian KDE per point
+    over its neighbour list; differentiable with respect to `points`."""
+    return _ComputePdf.apply(points, neighbors, sample_neigh_indices, inv_bandwidth,
+                             inv_radii, mode)
+
+
+def _basis_proj_raw(basis, features, neighbors, ranges):
+    out = torch.empty((ranges.shape[0], _dim(features, 1), _dim(basis, 1)), dtype=_F32,
+                      device=features.device)
+    _lib.check(_lib.lib().mccnn_basis_proj(
+        stream(), i64(basis.shape[0]), cint(_dim(basis, 1)), ptr(basis, _F32),
+        i64(features.shape[0]), cint(_dim(features, 1)), ptr(features, _F32),
+        i64(neighbors.shape[0]), cint(neighbors.dim()), cint(_dim(neighbors, 1)),
+        ptr(neighbors, _I32), i64(ranges.shape[0]), ptr(ranges, _I32), ptr(out)))
+    return out
+
+
+def basis_proj_grads(basis_neighbors, pt_features, neighbors, sample_neigh_indices,
+                     in_gradients):
+    """BasisProjGrads (basis_proj_ops.cpp:40-53) -> (basis_gradients [M, K],
+    feat_gradients [N_in, C])."""
+    dbasis = torch.empty_like(basis_neighbors)
+    dfeat = torch.empty_like(pt_features)
+    g = in_gradients
+    _lib.check(_lib.lib().mccnn_basis_proj_grads(
+        stream(), i64(basis_neighbors.shape[0]), cint(_dim(basis_neighbors, 1)),
+        ptr(basis_neighbors, _F32), i64(pt_features.shape[0]), cint(_dim(pt_features, 1)),
+        ptr(pt_features, _F32), i64(neighbors.shape[0]), cint(neighbors.dim()),
+        cint(_dim(neighbors, 1)), ptr(neighbors, _I32), i64(sample_neigh_indices.shape[0]),
+        ptr(sample_neigh_indices, _I32), cint(g.dim()), i64(_dim(g, 0)), i64(_dim(g, 1)),
+        i64(_dim(g, 2)), ptr(g, _F32), ptr(dbasis), ptr(dfeat)))
+    return dbasis, dfeat
+
+
+class _BasisProj(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, basis, features, neighbors, ranges):
+        ctx.save_for_backward(basis, features, neighbors, ranges)
+        return _basis_proj_raw(basis, features, neighbors, ranges)
+
+    @staticmethod
+    def backward(ctx, grad):
+        basis, features, neighbors, ranges = ctx.saved_tensors
+        dbasis, dfeat = basis_proj_grads(basis, features, neighbors, ranges, grad.contiguous())
+        return dbasis, dfeat, None, None
+
+
+def basis_proj(basis_neighbors, pt_features, neighbors, sample_neigh_indices):
+    """BasisProj (basis_proj_ops.cpp:25-38): [N_out, C, K] sum over the pairs of
+    each centre of feature (outer) basis; differentiable in basis and features."""
+    return _BasisProj.apply(basis_neighbors, pt_features, neighbors, sample_neigh_indices)

@@ -1,0 +1,311 @@
+"""Parity of the HIP ops against the CPU oracle, through the C ABI of
+libmccnn_hip.so (via the torch binding).  Integer outputs must be bit-exact;
+float outputs are held to 1e-5 relative, stated per test."""
+import numpy as np
+import pytest
+
+torch = pytest.importorskip("torch")
+
+pytestmark = pytest.mark.gpu
+
+REL = 1e-5
+
+
+@pytest.fixture(scope="module")
+def ops():
+    assert torch.cuda.is_available(), "GPU tests need a GPU"
+    from tensorflow_graphics_point_clouds_amd import tfg_custom_ops, _lib
+    _lib.lib()   # raises if the HIP library is not built
+    return tfg_custom_ops
+
+
+def dev(a, dtype=None):
+    t = torch.as_tensor(np.ascontiguousarray(a))
+    if dtype is not None:
+        t = t.to(dtype)
+    return t.cuda().contiguous()
+
+
+def _cloud(rng, batch, n, d, scale=1.0):
+    pts = (rng.random((n, d)) * scale).astype(np.float32)
+    bids = rng.integers(0, batch, n).astype(np.int32)
+    bids[:batch] = np.arange(batch)
+    return pts, bids
+
+
+def assert_rel(got, expect, mag=None, tol=REL):
+    """|got - expect| <= tol * mag elementwise, where mag is the sum of the
+    absolute values of the terms of each sum (default |expect|)."""
+    got, expect = np.asarray(got, np.float64), np.asarray(expect, np.float64)
+    mag = np.abs(expect) if mag is None else np.asarray(mag, np.float64)
+    err = np.abs(got - expect)
+    bad = err > tol * mag + 1e-30
+    assert not bad.any(), "max err/mag = %g at %d entries" % (
+        (err / np.maximum(mag, 1e-300)).max(), int(bad.sum()))
+
+
+def assert_normwise(got, expect, tol=REL):
+    """max |got - expect| <= tol * max |expect| (sums with cancellation)."""
+    got, expect = np.asarray(got, np.float64), np.asarray(expect, np.float64)
+    scale = np.abs(expect).max() if expect.size else 1.0
+    assert np.abs(got - expect).max(initial=0.0) <= tol * scale
+
+
+# ------------------------------------------------------------------ grid ----
+
+@pytest.mark.parametrize("d", [2, 3, 4, 5, 6])
+@pytest.mark.parametrize("batch,n,cell", [(1, 1000, 0.13), (5, 20000, 0.05), (32, 50000, 0.21)])
+def test_keys_sort_table_bit_exact(ops, oracle, d, batch, n, cell):
+    from tensorflow_graphics_point_clouds_amd import pc
+    rng = np.random.default_rng(1 + d + batch)
+    if d >= 5:
+        cell = max(cell, 0.21)
+    pts, bids = _cloud(rng, batch, n, d)
+    g = oracle.Grid(pts, bids, batch, cell)
+    keys = ops.compute_keys(dev(pts), dev(bids), dev(g.scaled_aabb_min), dev(g.num_cells),
+                            dev(g.inv_cell_sizes))
+    assert np.array_equal(keys.cpu().numpy(), g.keys)
+    # the glue kernels reproduce the grid set-up, the sort and the gathers
+    grid = pc.Grid(pc.PointCloud(dev(pts), dev(bids), batch), cell)
+    assert np.array_equal(grid._aabb_min.cpu().numpy(), g.aabb_min)
+    assert np.array_equal(grid._aabb_max.cpu().numpy(), g.aabb_max)
+    assert np.array_equal(grid._num_cells.cpu().numpy(), g.num_cells)
+    assert np.array_equal(grid._scaled_aabb_min.cpu().numpy(), g.scaled_aabb_min)
+    assert np.array_equal(grid._inv_cell_sizes.cpu().numpy(), g.inv_cell_sizes)
+    assert np.array_equal(grid._sorted_indices.cpu().numpy(), g.sorted_indices)
+    assert np.array_equal(grid._sorted_keys.cpu().numpy(), g.sorted_keys)
+    assert np.array_equal(grid._sorted_points.cpu().numpy(), g.sorted_points)
+    assert np.array_equal(grid._sorted_batch_ids.cpu().numpy(), g.sorted_batch_ids)
+    assert np.array_equal(grid.get_DS().cpu().numpy(), g.get_ds())
+
+
+@pytest.mark.parametrize("bits", [1, 7, 8, 9, 20, 33, 63])
+def test_sort_key_widths_and_ties(ops, bits):
+    """Stable descending order for every pass count, with many equal keys."""
+    from tensorflow_graphics_point_clouds_amd import _lib
+    from tensorflow_graphics_point_clouds_amd._lib import cint, i64, ptr, stream
+    rng = np.random.default_rng(bits)
+    n = 70001
+    hi = min(2 ** bits, 2 ** 62)
+    keys = rng.integers(0, hi, n, dtype=np.int64)
+    keys[::3] = keys[0]
+    k = dev(keys)
+    out_k = torch.empty_like(k)
+    out_i = torch.empty(n, dtype=torch.int32, device="cuda")
+    L = _lib.lib()
+    ws = _lib.workspace(L.mccnn_sort_keys_workspace_bytes(i64(n)), k.device)
+    _lib.check(L.mccnn_sort_keys_descending(stream(), i64(n), cint(bits), ptr(k), ptr(out_k),
+                                            ptr(out_i), ptr(ws), _lib.csize(ws.numel())))
+    expect = np.argsort(-keys, kind="stable")
+    assert np.array_equal(out_i.cpu().numpy(), expect)
+    assert np.array_equal(out_k.cpu().numpy(), keys[expect])
+
+
+# ------------------------------------------------------------- neighbours ----
+
+def _gpu_neighbors(ops, g, samples, sbids, radii, max_neighs=0):
+    inv_r = (np.float32(1.0) / radii).astype(np.float32)
+    return ops.find_neighbors(dev(samples), dev(sbids), dev(g.sorted_points), dev(g.sorted_keys),
+                              dev(g.get_ds()), dev(g.num_cells), dev(g.scaled_aabb_min),
+                              dev(g.inv_cell_sizes), dev(inv_r), max_neighs)
+
+
+@pytest.mark.parametrize("d,radius", [(2, 0.03), (3, 0.08), (3, 0.3), (4, 0.3), (5, 0.5), (6, 0.6)])
+@pytest.mark.parametrize("self_nbh", [True, False])
+def test_neighbors_bit_exact(ops, oracle, d, radius, self_nbh):
+    rng = np.random.default_rng(10 * d + int(self_nbh))
+    batch, n = 4, 6000 if d < 5 else 2500
+    pts, bids = _cloud(rng, batch, n, d)
+    g = oracle.Grid(pts, bids, batch, radius)
+    if self_nbh:
+        nbh = oracle.Neighborhood(g, radius)
+    else:
+        ctr, cb = _cloud(rng, batch, 1500, d, scale=1.2)
+        ctr -= 0.1                               # some centres outside the grid box
+        nbh = oracle.Neighborhood(g, radius, ctr, cb)
+    ranges, nbrs = _gpu_neighbors(ops, g, nbh.samples, nbh.sample_batch_ids, nbh.radii)
+    assert np.array_equal(ranges.cpu().numpy(), nbh.ranges)
+    assert np.array_equal(nbrs.cpu().numpy(), nbh.neighbors)
+
+
+@pytest.mark.parametrize("radius,expected", [(0.05, 1), (0.11, 7), (0.142, 19), (0.174, 27)])
+def test_neighbors_lattice_known_answer(ops, oracle, radius, expected):
+    t = np.linspace(0, 1, 10, endpoint=False)
+    pts = np.array(np.meshgrid(t, t, t)).T.reshape(-1, 3).astype(np.float32)
+    t2 = np.linspace(1 / 5, 1, 4, endpoint=False)
+    ctr = np.array(np.meshgrid(t2, t2, t2)).T.reshape(-1, 3).astype(np.float32)
+    g = oracle.Grid(pts, np.zeros(len(pts), np.int32), 1, radius)
+    ranges, _ = _gpu_neighbors(ops, g, ctr, np.zeros(len(ctr), np.int32),
+                               np.full(3, radius, np.float32))
+    counts = np.diff(np.concatenate([[0], ranges.cpu().numpy()]))
+    assert np.all(counts == expected)
+
+
+def test_neighbors_max_neighs_and_anisotropic_radii(ops, oracle):
+    rng = np.random.default_rng(77)
+    pts, bids = _cloud(rng, 2, 5000, 3)
+    radii = np.array([0.1, 0.05, 0.08], np.float32)
+    g = oracle.Grid(pts, bids, 2, radii)
+    for limit in (0, 4):
+        nbh = oracle.Neighborhood(g, radii, max_neighbors=limit)
+        ranges, nbrs = _gpu_neighbors(ops, g, nbh.samples, nbh.sample_batch_ids, radii, limit)
+        assert np.array_equal(ranges.cpu().numpy(), nbh.ranges)
+        assert np.array_equal(nbrs.cpu().numpy(), nbh.neighbors)
+
+
+def test_neighbors_clustered_cloud(ops, oracle):
+    """Heavy-tailed neighbour counts (blobs + noise), the shape of the scene-scale
+    configuration at 1/50 of its size."""
+    from tensorflow_graphics_point_clouds_amd import synthetic
+    cfg = synthetic.config3(scale=0.02)
+    g = oracle.Grid(cfg["points"], cfg["batch_ids"], cfg["batch_size"], cfg["radius"])
+    nbh = oracle.Neighborhood(g, cfg["radius"])
+    ranges, nbrs = _gpu_neighbors(ops, g, nbh.samples, nbh.sample_batch_ids, nbh.radii)
+    assert np.array_equal(ranges.cpu().numpy(), nbh.ranges)
+    assert np.array_equal(nbrs.cpu().numpy(), nbh.neighbors)
+
+
+# -------------------------------------------------------------------- pdf ----
+
+@pytest.mark.parametrize("d", [2, 3, 4])
+@pytest.mark.parametrize("mode", [0, 1])
+def test_pdf_and_point_grads(ops, oracle, d, mode):
+    rng = np.random.default_rng(20 + d)
+    pts, bids = _cloud(rng, 3, 4000, d)
+    radius = {2: 0.05, 3: 0.15, 4: 0.3}[d]
+    g = oracle.Grid(pts, bids, 3, radius)
+    nbh = oracle.Neighborhood(g, radius)
+    inv_bw = np.full(d, 1 / np.float32(0.2), np.float32)
+    expect = oracle.compute_pdf(g.sorted_points, nbh.neighbors, nbh.ranges, inv_bw,
+                                nbh.inv_radii, mode)
+    sp = dev(g.sorted_points).requires_grad_(True)
+    pdf = ops.compute_pdf_with_pt_grads(sp, dev(nbh.neighbors), dev(nbh.ranges), dev(inv_bw),
+                                        dev(nbh.inv_radii), mode)
+    assert_rel(pdf.detach().cpu().numpy(), expect)       # all terms positive: 1e-5 relative
+    up = rng.standard_normal(len(pts)).astype(np.float32)
+    pdf.backward(dev(up))
+    gexp = oracle.compute_pdf_pt_grads(g.sorted_points, nbh.neighbors, nbh.ranges, inv_bw,
+                                       nbh.inv_radii, up, mode)
+    assert_normwise(sp.grad.cpu().numpy(), gexp)
+
+
+# ------------------------------------------------------------- basis_proj ----
+
+@pytest.mark.parametrize("c,k", [(1, 8), (3, 16), (5, 32), (8, 8), (16, 16), (32, 32),
+                                 (64, 16), (128, 32), (24, 64), (64, 64)])
+def test_basis_proj_forward_and_grads(ops, oracle, c, k):
+    rng = np.random.default_rng(c * 100 + k)
+    n = 3000
+    pts, bids = _cloud(rng, 2, n, 3)
+    g = oracle.Grid(pts, bids, 2, 0.12)
+    ctr, cb = _cloud(rng, 2, 700, 3)
+    nbh = oracle.Neighborhood(g, 0.12, ctr, cb)
+    ids = nbh.original_neigh_ids
+    m = len(ids)
+    basis = rng.random((m, k)).astype(np.float32)
+    feat = rng.standard_normal((n, c)).astype(np.float32)
+    expect, mag = oracle.basis_proj(basis, feat, ids, nbh.ranges, with_magnitude=True)
+    tb, tf = dev(basis).requires_grad_(True), dev(feat).requires_grad_(True)
+    out = ops.basis_proj(tb, tf, dev(ids), dev(nbh.ranges))
+    assert out.shape == (700, c, k)
+    assert_rel(out.detach().cpu().numpy(), expect, mag)
+    up = rng.standard_normal((700, c, k)).astype(np.float32)
+    out.backward(dev(up))
+    db, df = oracle.basis_proj_grads(basis, feat, ids, nbh.ranges, up)
+    assert_normwise(tb.grad.cpu().numpy(), db)
+    assert_normwise(tf.grad.cpu().numpy(), df)
+
+
+def test_basis_proj_empty_neighbourhoods(ops, oracle):
+    """Centres without pairs give zero rows; a centre list with no pairs at all works."""
+    feat = np.ones((10, 8), np.float32)
+    ranges = np.array([0, 2, 2, 3], np.int32)
+    ids = np.array([[1, 1], [4, 1], [9, 3]], np.int32)
+    basis = np.arange(24, dtype=np.float32).reshape(3, 8)
+    out = ops.basis_proj(dev(basis), dev(feat), dev(ids), dev(ranges)).cpu().numpy()
+    expect = oracle.basis_proj(basis, feat, ids, ranges)
+    assert np.array_equal(out, expect.astype(np.float32))
+    none = ops.basis_proj(dev(np.zeros((0, 8), np.float32)), dev(feat),
+                          dev(np.zeros((0, 2), np.int32)), dev(np.zeros(4, np.int32)))
+    assert none.shape == (4, 8, 8) and float(none.abs().sum()) == 0.0
+
+
+def test_op_validation_errors(ops):
+    """The reference ops reject these with InvalidArgument."""
+    f = lambda *s: torch.zeros(*s, device="cuda")
+    i = lambda *s: torch.zeros(*s, dtype=torch.int32, device="cuda")
+    with pytest.raises(ValueError):      # 7 dimensions
+        ops.compute_keys(f(4, 7), i(4), f(1, 7), i(7), f(7))
+    with pytest.raises(ValueError):      # batch ids do not match
+        ops.compute_keys(f(4, 3), i(5), f(1, 3), i(3), f(3))
+    with pytest.raises(ValueError):      # K = 12
+        ops.basis_proj(f(5, 12), f(4, 8), i(5, 2), i(3))
+    with pytest.raises(ValueError):      # C = 12
+        ops.basis_proj(f(5, 8), f(4, 12), i(5, 2), i(3))
+    with pytest.raises(ValueError):      # basis rows != pairs
+        ops.basis_proj(f(6, 8), f(4, 8), i(5, 2), i(3))
+    with pytest.raises(ValueError):      # pairs need two columns
+        ops.basis_proj(f(5, 8), f(4, 8), i(5, 3), i(3))
+    with pytest.raises(ValueError):      # mode 2
+        ops.compute_pdf_with_pt_grads(f(4, 3), i(4, 2), i(4), f(3), f(3), 2)
+    with pytest.raises(ValueError):      # samples != points
+        ops.compute_pdf_with_pt_grads(f(4, 3), i(4, 2), i(5), f(3), f(3), 0)
+    with pytest.raises(ValueError):      # sampling mode
+        ops.sampling(f(4, 3), i(4), torch.zeros(4, dtype=torch.int64, device="cuda"), i(3),
+                     i(4, 2), i(4), 2)
+    with pytest.raises(ValueError):      # non-positive batch size
+        ops.build_grid_ds(torch.zeros(4, dtype=torch.int64, device="cuda"), i(3), [1, 1, 1], 0)
+    with pytest.raises(ValueError):      # grid table of the wrong rank
+        ops.find_neighbors(f(4, 3), i(4), f(4, 3), torch.zeros(4, dtype=torch.int64, device="cuda"),
+                           i(1, 1, 2), i(3), f(1, 3), f(3), f(3), 0)
+
+
+# --------------------------------------------------------------- sampling ----
+
+@pytest.mark.parametrize("d,batch,cell", [(2, 1, 0.04), (3, 4, 0.1), (3, 1, 0.3), (4, 3, 0.3)])
+@pytest.mark.parametrize("mode", [0, 1])
+def test_sampling_bit_exact(ops, oracle, d, batch, cell, mode):
+    rng = np.random.default_rng(33 + d + batch)
+    pts, bids = _cloud(rng, batch, 5000, d)
+    g = oracle.Grid(pts, bids, batch, cell)
+    nbh = oracle.Neighborhood(g, cell)
+    ep, eb, ei = oracle.sampling(g.sorted_points, g.sorted_batch_ids, g.sorted_keys, g.num_cells,
+                                 nbh.neighbors, nbh.ranges, mode)
+    gp, gb, gi = ops.sampling(dev(g.sorted_points), dev(g.sorted_batch_ids), dev(g.sorted_keys),
+                              dev(g.num_cells), dev(nbh.neighbors), dev(nbh.ranges), mode)
+    assert np.array_equal(gi.cpu().numpy(), ei)
+    assert np.array_equal(gb.cpu().numpy(), eb)
+    assert np.array_equal(gp.cpu().numpy(), ep)     # serial fp32 sums: same bits
+
+
+@pytest.mark.parametrize("n_sqrt,scale", [(6, 1), (100, 5)])
+def test_poisson_collinear_known_answer(ops, oracle, n_sqrt, scale):
+    from tensorflow_graphics_point_clouds_amd import pc
+    t = np.linspace(0, scale, num=n_sqrt)
+    pts = np.array(np.meshgrid(t, t)).T.reshape(-1, 2).astype(np.float32)
+    bids = np.repeat(np.arange(n_sqrt), n_sqrt).astype(np.int32)
+    cell = (scale * np.array([2, 2], dtype=np.float32) / n_sqrt).astype(np.float32)
+    cloud = pc.PointCloud(dev(pts), dev(bids), n_sqrt)
+    nbh = pc.Neighborhood(pc.Grid(cloud, cell), cell)
+    sampled, idx = pc.sample(nbh, "poisson")
+    assert sampled._points.shape[0] == n_sqrt ** 2 // 2
+    assert np.array_equal(pts[idx.cpu().numpy()], sampled._points.cpu().numpy())
+
+
+def test_point_hierarchy_matches_oracle(ops, oracle):
+    """Three cell-average levels (the ModelNet-shaped configuration): every level's
+    points, batch ids and neighbourhoods equal the oracle's, bit for bit."""
+    from tensorflow_graphics_point_clouds_amd import pc, synthetic
+    cfg = synthetic.config2(batch=4, points_per_cloud=512)
+    hier = pc.PointHierarchy(pc.PointCloud(dev(cfg["points"]), dev(cfg["batch_ids"]),
+                                           cfg["batch_size"]), cfg["radii"], "cell average")
+    pts, bids = cfg["points"], cfg["batch_ids"]
+    for level, r in enumerate(cfg["radii"]):
+        g = oracle.Grid(pts, bids, cfg["batch_size"], r)
+        nbh = oracle.Neighborhood(g, r)
+        gn = hier._neighborhoods[level]
+        assert np.array_equal(gn._neighbors.cpu().numpy(), nbh.neighbors)
+        pts, bids, _ = oracle.sampling(g.sorted_points, g.sorted_batch_ids, g.sorted_keys,
+                                       g.num_cells, nbh.neighbors, nbh.ranges, 1)
+        assert np.array_equal(hier._point_clouds[level + 1]._points.cpu().numpy(), pts)
+        assert np.array_equal(hier._point_clouds[level + 1]._batch_ids.cpu().numpy(), bids)
