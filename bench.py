@@ -1,0 +1,257 @@
+#!/usr/bin/env python3
+"""Benchmark of the MCCNN hot path on one MI355X.
+
+A step is one forward + backward pass of a Monte-Carlo convolution layer
+(64 -> 64 channels, 16-unit kernel MLP, radius 0.15) over the scene-scale batch:
+8 clustered clouds of 50k-150k points.  Grid, neighbourhood and densities are
+built once before the timed region (their times are reported separately);
+inputs are resident in HBM when timing starts.
+
+Prints ONE JSON line: points/sec (centre points per second of fwd+bwd), the
+roofline of the dominant kernel of the step (HIP events around every op call on
+the launch stream), per-op figures, the isolated basis_proj figures on the
+dense-neighbourhood case (C=128, K=32), and the host-CPU figure of the oracle on
+a bounded sample of the same workload.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
+FP32_MATRIX_PEAK_TFLOPS = 157.3
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def op_bytes(name, M, N_in, N_out, C, K, D):
+    """Algorithmic bytes of one launch of each op (fp32, int32 pair table)."""
+    if name == "basis_proj":
+        return 4 * (M * K + M * C + N_out * C * K) + 8 * M + 4 * N_out
+    if name == "basis_proj_grads":
+        return 4 * (2 * M * K + M * C + N_out * C * K + N_in * C) + 8 * M + 4 * N_out
+    if name == "mc_basis":
+        return M * (8 + 2 * 4 * D + 4) + 4 * M * K
+    if name == "mc_basis_grads":
+        return M * (8 + 2 * 4 * D + 4) + 4 * M * K
+    return None
+
+
+def build_scene(torch, pc, synthetic, scale):
+    import numpy as np
+    cfg = synthetic.config3(scale=scale)
+    dev = lambda a: torch.as_tensor(np.ascontiguousarray(a)).cuda()
+    cloud = pc.PointCloud(dev(cfg["points"]), dev(cfg["batch_ids"]), cfg["batch_size"])
+    return cfg, cloud
+
+
+def time_build(torch, pc, cloud, radius, reps=3):
+    """Grid + neighbourhood + density build, median of `reps` (ms)."""
+    out = {}
+    best = None
+    for _ in range(reps):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        grid = pc.Grid(cloud, radius)
+        grid.get_DS()
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        nbh = pc.Neighborhood(grid, radius, cloud)
+        torch.cuda.synchronize()
+        t2 = time.perf_counter()
+        nbh.get_pdf(bandwidth=0.2)
+        torch.cuda.synchronize()
+        t3 = time.perf_counter()
+        cur = dict(grid_ms=(t1 - t0) * 1e3, neighbors_ms=(t2 - t1) * 1e3,
+                   pdf_ms=(t3 - t2) * 1e3)
+        if best is None or sum(cur.values()) < sum(best.values()):
+            best = cur
+    out.update(best)
+    return grid, nbh, out
+
+
+def cpu_baseline(synthetic, sample_points=60000):
+    """MCConv fwd+bwd of the oracle (C with OpenMP, numpy GEMMs) on one cloud of
+    the same generator, cut to `sample_points` points."""
+    import numpy as np
+    from oracle import mccnn_oracle as orc
+    cfg = synthetic.config3(scale=1.0, batch=1)
+    pts = cfg["points"][:sample_points]
+    n = len(pts)
+    bids = np.zeros(n, np.int32)
+    r = np.float32(cfg["radius"])
+    g = orc.Grid(pts, bids, 1, r)
+    nbh = orc.Neighborhood(g, r, pts, bids)
+    pdf = nbh.pdf_per_pair(0.2).astype(np.float32)
+    ids = nbh.original_neigh_ids
+    rng = np.random.default_rng(0)
+    C, K, CO = cfg["c_in"], cfg["hidden"], cfg["c_out"]
+    w, b, wo = synthetic.mcconv_weights(rng, 3, C, CO, K, 1)
+    feat = rng.standard_normal((n, C)).astype(np.float32)
+    up = rng.standard_normal((n, CO)).astype(np.float32)
+    inv_r = np.float32(1.0) / r
+
+    def step():
+        diff = (pts[ids[:, 0]] - pts[ids[:, 1]]) * inv_r
+        z = diff @ w[0] + b[0]
+        basis = (np.maximum(z, 0) / pdf[:, None]).astype(np.float32)
+        proj = orc.basis_proj_f32(basis, feat, ids, nbh.ranges)
+        out = proj.reshape(n, C * K) @ wo[0]
+        dproj = (up @ wo[0].T).reshape(n, C, K)
+        dwo = proj.reshape(n, C * K).T @ up
+        dbasis, dfeat = orc.basis_proj_grads_f32(basis, feat, ids, nbh.ranges, dproj)
+        dz = dbasis * (z > 0) / pdf[:, None]
+        dw = diff.T @ dz
+        db = dz.sum(axis=0)
+        return out, dwo, dfeat, dw, db
+
+    step()
+    reps, t0 = 0, time.perf_counter()
+    while reps < 3 or time.perf_counter() - t0 < 10.0:
+        step()
+        reps += 1
+        if time.perf_counter() - t0 > 25.0:
+            break
+    dt = (time.perf_counter() - t0) / reps
+    cores = int(os.environ.get("OMP_NUM_THREADS", "0")) or len(os.sched_getaffinity(0))
+    return {"value": n / dt, "unit": "points/s", "cores": cores, "kind": "port",
+            "sample": "one config-3 cloud cut to %d points (%d pairs), %d fwd+bwd passes of "
+                      "the C/OpenMP oracle with numpy GEMMs" % (n, len(ids), reps)}
+
+
+def isolated_basis_proj(torch, pc, synthetic, tfg, _lib, radius=0.04, steps=5):
+    """basis_proj forward and gradients alone on 4 x 200k uniform points,
+    C=128, K=32 (the dense-neighbourhood case)."""
+    import numpy as np
+    cfg = synthetic.config4()
+    dev = lambda a: torch.as_tensor(np.ascontiguousarray(a)).cuda()
+    cloud = pc.PointCloud(dev(cfg["points"]), dev(cfg["batch_ids"]), cfg["batch_size"])
+    grid = pc.Grid(cloud, radius)
+    nbh = pc.Neighborhood(grid, radius, cloud)
+    ids, ranges = nbh._original_neigh_ids, nbh._samples_neigh_ranges
+    M, N, C, K = ids.shape[0], cloud._points.shape[0], cfg["c_in"], cfg["basis"]
+    gen = torch.Generator(device="cuda").manual_seed(4)
+    basis = torch.rand((M, K), device="cuda", generator=gen)
+    feat = torch.randn((N, C), device="cuda", generator=gen)
+    up = torch.randn((N, C, K), device="cuda", generator=gen)
+    for _ in range(2):
+        out = tfg._basis_proj_raw(basis, feat, ids, ranges)
+        tfg.basis_proj_grads(basis, feat, ids, ranges, up)
+    del out
+    _lib.start_timing()
+    for _ in range(steps):
+        tfg._basis_proj_raw(basis, feat, ids, ranges)
+        tfg.basis_proj_grads(basis, feat, ids, ranges, up)
+    t = _lib.collect_timing()
+    res = {"workload": "4x200k uniform, r=%.2f, C=%d, K=%d" % (radius, C, K), "pairs": M}
+    for name in ("basis_proj", "basis_proj_grads"):
+        ms = sum(t[name]) / len(t[name])
+        by = op_bytes(name, M, N, N, C, K, 3)
+        res[name] = {"ms": ms, "GBps": by / ms / 1e6, "frac_hbm_peak": by / ms / 1e6 / HBM_PEAK_GBS,
+                     "algorithmic_bytes": by}
+    return res
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--scale", type=float, default=1.0, help="shrink the point counts (tests)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the host-CPU baseline")
+    ap.add_argument("--no-isolated", action="store_true", help="skip the isolated basis_proj case")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        log("bench.py measures one GPU: this build has no multi-GPU path (clouds would be "
+            "sharded whole across GPUs with no exchange in the forward pass); run with --gpus 1")
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+    from tensorflow_graphics_point_clouds_amd import _lib, layers, pc, synthetic, tfg_custom_ops
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    _lib.lib()
+    torch.backends.cuda.matmul.allow_tf32 = False
+
+    cfg, cloud = build_scene(torch, pc, synthetic, args.scale)
+    radius = cfg["radius"]
+    grid, nbh, build_ms = time_build(torch, pc, cloud, radius)
+    N = cloud._points.shape[0]
+    M = nbh._neighbors.shape[0]
+    C, CO, K, D = cfg["c_in"], cfg["c_out"], cfg["hidden"], 3
+    log("scene: %d points, %d pairs (mean %.1f per point), build %s" % (N, M, M / N, build_ms))
+
+    conv = layers.MCConv(C, CO, D, num_mlps=1, mlp_size=[K], non_linearity_type="leaky_relu",
+                         seed=3)
+    gen = torch.Generator(device="cuda").manual_seed(3)
+    feats = torch.randn((N, C), device="cuda", generator=gen).requires_grad_(True)
+    up = torch.randn((N, CO), device="cuda", generator=gen)
+
+    def step():
+        out = conv(feats, cloud, cloud, radius, neighborhood=nbh)
+        out.backward(up)
+        feats.grad = None
+        for p in conv.parameters():
+            p.grad = None
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    _lib.start_timing()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    per_op = _lib.collect_timing()
+    ms_per_step = dt * 1e3 / args.steps
+
+    ops = {}
+    for name, vals in per_op.items():
+        ms = sum(vals) / len(vals)
+        by = op_bytes(name, M, N, N, C, K, D)
+        ops[name] = {"ms": round(ms, 4)}
+        if by:
+            ops[name].update(GBps=round(by / ms / 1e6, 1),
+                             frac_hbm_peak=round(by / ms / 1e6 / HBM_PEAK_GBS, 4),
+                             algorithmic_bytes=by)
+    kernel_ms = sum(v["ms"] for v in ops.values())
+    ops["dense_gemms_and_glue"] = {"ms": round(ms_per_step - kernel_ms, 4),
+                                   "flops": 3 * 2 * N * C * K * CO}
+    dominant = max((n for n in ops if "GBps" in ops[n]), key=lambda n: ops[n]["ms"])
+    roof = {"kernel": dominant, "bound": "hbm", "achieved": ops[dominant]["GBps"],
+            "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": ops[dominant]["frac_hbm_peak"],
+            "traffic": None, "ms": ops[dominant]["ms"]}
+
+    result = {
+        "metric": "MCConv layer fwd+bwd points/sec", "value": N / (ms_per_step * 1e-3),
+        "unit": "points/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "config 3: 8 clustered clouds of 50k-150k points (seed 1003), "
+                               "MCConv 64->64, 16-unit kernel MLP, radius 0.15, fp32, fwd+bwd, "
+                               "neighbourhood and densities prebuilt",
+                   "points": N, "pairs": M, "scale": args.scale},
+        "roofline": roof, "ops": ops, "build_ms": {k: round(v, 3) for k, v in build_ms.items()},
+        "points_per_s_with_build": N / ((ms_per_step + sum(build_ms.values())) * 1e-3),
+    }
+    if not args.no_isolated and args.scale == 1.0:
+        del feats, up
+        torch.cuda.empty_cache()
+        result["basis_proj_isolated"] = isolated_basis_proj(torch, pc, synthetic, tfg_custom_ops,
+                                                            _lib)
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(synthetic)
+    else:
+        result["cpu_baseline"] = None
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -80,3 +80,53 @@ def ptr(t, dtype=None):
 def workspace(nbytes, device):
     import torch
     return torch.empty(max(int(nbytes), 1), dtype=torch.uint8, device=device)
+
+
+# ------------------------------------------------------------------ timing ----
+# When a dict is installed with start_timing(), every op call made through
+# region() records a pair of events on torch's current stream, the stream the
+# kernels are launched on.  collect_timing() synchronises and returns, per op
+# name, the list of elapsed milliseconds.
+
+_timing = None
+
+
+def start_timing():
+    global _timing
+    _timing = {}
+
+
+class region:
+    def __init__(self, name):
+        self.name = name
+
+    def __enter__(self):
+        if _timing is not None:
+            import torch
+            self.start = torch.cuda.Event(enable_timing=True)
+            self.end = torch.cuda.Event(enable_timing=True)
+            self.start.record()
+        return self
+
+    def __exit__(self, *exc):
+        if _timing is not None:
+            self.end.record()
+            _timing.setdefault(self.name, []).append((self.start, self.end))
+        return False
+
+
+def collect_timing():
+    global _timing
+    import torch
+    torch.cuda.synchronize()
+    out = {k: [a.elapsed_time(b) for a, b in v] for k, v in (_timing or {}).items()}
+    _timing = None
+    return out
+
+
+def call(name, *args):
+    """Invoke entry point mccnn_<name>, raise on a non-zero status, and time it
+    when timing is active."""
+    fn = getattr(lib(), "mccnn_" + name)
+    with region(name):
+        check(fn(*args))

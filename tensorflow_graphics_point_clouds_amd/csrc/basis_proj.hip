@@ -106,6 +106,190 @@ __global__ void __launch_bounds__(256) basis_proj_grads_generic_kernel(
   }
 }
 
+// ---------------------------------------------------------------------------
+// Matrix-core forward path.  One wavefront owns a centre (and a chunk of kCW
+// channels) and accumulates the [channels x K] tile in MFMA accumulators while
+// it streams the centre's pairs:
+//   K = 32 / 64 : v_mfma_f32_32x32x2f32, rows = channels, columns = basis, two
+//                 pairs per instruction (lanes 0-31 feed pair 2t, 32-63 pair 2t+1)
+//   K = 16      : v_mfma_f32_16x16x4f32, rows = basis, columns = channels, four
+//                 pairs per instruction (one per 16-lane quarter)
+// Operands go from global memory straight into the MFMA register layout: a lane
+// reads kCPL consecutive channels of one feature row (up to 16 B) and its basis
+// column(s); kCPL tiles share the lane's row/column index, tile j holding the
+// channels {lane_channel_base + j}.  Neighbour ids are read 64 at a time,
+// coalesced, and broadcast with a lane shuffle.  Results leave with
+// non-temporal stores (write-once stream).
+
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+template <int N>
+struct FVec {
+  float v[N];
+};
+
+template <int N>
+__device__ __forceinline__ FVec<N> load_vec(const float *__restrict__ p, bool valid) {
+  FVec<N> r;
+#pragma unroll
+  for (int i = 0; i < N; ++i) r.v[i] = 0.0f;
+  if (valid) {
+    if constexpr (N % 4 == 0) {
+#pragma unroll
+      for (int i = 0; i < N / 4; ++i) {
+        const float4 t = reinterpret_cast<const float4 *>(p)[i];
+        r.v[4 * i] = t.x; r.v[4 * i + 1] = t.y; r.v[4 * i + 2] = t.z; r.v[4 * i + 3] = t.w;
+      }
+    } else if constexpr (N == 2) {
+      const float2 t = *reinterpret_cast<const float2 *>(p);
+      r.v[0] = t.x; r.v[1] = t.y;
+    } else {
+#pragma unroll
+      for (int i = 0; i < N; ++i) r.v[i] = p[i];
+    }
+  }
+  return r;
+}
+
+constexpr int kUnroll = 4;   // MFMA steps whose loads are issued together
+
+template <int K, int kCPL>
+__global__ void __launch_bounds__(256) basis_proj_mfma32_kernel(
+    int64_t n_out, int C, int chunks, const float *__restrict__ basis,
+    const float *__restrict__ feat, const int2 *__restrict__ nbrs,
+    const int *__restrict__ ranges, float *__restrict__ out) {
+  static_assert(K == 32 || K == 64, "32x32x2 path");
+  constexpr int kNT = K / 32;        // basis columns per lane
+  constexpr int kCW = 32 * kCPL;     // channels per wave
+  const int lane = lane_id();
+  const int64_t wid =
+      __builtin_amdgcn_readfirstlane((int)((blockIdx.x * (int64_t)blockDim.x + threadIdx.x) / kWave));
+  const int64_t centre = wid / chunks;
+  if (centre >= n_out) return;
+  const int chunk = (int)(wid - centre * chunks);
+  const int half = lane >> 5, col = lane & 31;
+  const int a = centre > 0 ? ranges[centre - 1] : 0, b = ranges[centre];
+  const float *fbase = feat + chunk * kCW + col * kCPL;
+  const float *bbase = basis + col * kNT;
+  v16f acc[kCPL][kNT];
+#pragma unroll
+  for (int j = 0; j < kCPL; ++j)
+#pragma unroll
+    for (int q = 0; q < kNT; ++q)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[j][q][r] = 0.0f;
+
+  for (int m0 = a; m0 < b; m0 += kWave) {
+    const int cnt = b - m0 < kWave ? b - m0 : kWave;
+    const int myidx = nbrs[m0 + (lane < cnt ? lane : 0)].x;
+    const int steps = (cnt + 1) >> 1;
+    for (int t = 0; t < steps; t += kUnroll) {
+      FVec<kCPL> f[kUnroll];
+      FVec<kNT> w[kUnroll];
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) {
+        const int n = 2 * (t + u) + half;
+        const bool valid = n < cnt;
+        const int idx = __shfl(myidx, n & (kWave - 1), kWave);
+        f[u] = load_vec<kCPL>(fbase + (int64_t)idx * C, valid);
+        w[u] = load_vec<kNT>(bbase + (int64_t)(m0 + n) * K, valid);
+      }
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u)
+#pragma unroll
+        for (int j = 0; j < kCPL; ++j)
+#pragma unroll
+          for (int q = 0; q < kNT; ++q)
+            acc[j][q] = __builtin_amdgcn_mfma_f32_32x32x2f32(f[u].v[j], w[u].v[q], acc[j][q], 0, 0, 0);
+    }
+  }
+  // D[i][col]: i = 8*(r/4) + (r%4) + 4*half is the lane-row whose channels are
+  // i*kCPL + j; column col holds basis columns col*kNT + q.
+  float *o = out + centre * (int64_t)C * K + (int64_t)chunk * kCW * K + col * kNT;
+#pragma unroll
+  for (int j = 0; j < kCPL; ++j)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int i = 8 * (r >> 2) + (r & 3) + 4 * half;
+      float *dst = o + (i * kCPL + j) * K;
+      if constexpr (kNT == 1) {
+        __builtin_nontemporal_store(acc[j][0][r], dst);
+      } else {
+        __builtin_nontemporal_store(acc[j][0][r], dst);
+        __builtin_nontemporal_store(acc[j][1][r], dst + 1);
+      }
+    }
+}
+
+template <int kCPL>
+__global__ void __launch_bounds__(256) basis_proj_mfma16_kernel(
+    int64_t n_out, int C, int chunks, const float *__restrict__ basis,
+    const float *__restrict__ feat, const int2 *__restrict__ nbrs,
+    const int *__restrict__ ranges, float *__restrict__ out) {
+  constexpr int K = 16;
+  constexpr int kCW = 16 * kCPL;
+  const int lane = lane_id();
+  const int64_t wid =
+      __builtin_amdgcn_readfirstlane((int)((blockIdx.x * (int64_t)blockDim.x + threadIdx.x) / kWave));
+  const int64_t centre = wid / chunks;
+  if (centre >= n_out) return;
+  const int chunk = (int)(wid - centre * chunks);
+  const int quarter = lane >> 4, col = lane & 15;
+  const int a = centre > 0 ? ranges[centre - 1] : 0, b = ranges[centre];
+  const float *fbase = feat + chunk * kCW + col * kCPL;
+  const float *bbase = basis + col;
+  v4f acc[kCPL];
+#pragma unroll
+  for (int j = 0; j < kCPL; ++j)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) acc[j][r] = 0.0f;
+
+  for (int m0 = a; m0 < b; m0 += kWave) {
+    const int cnt = b - m0 < kWave ? b - m0 : kWave;
+    const int myidx = nbrs[m0 + (lane < cnt ? lane : 0)].x;
+    const int steps = (cnt + 3) >> 2;
+    for (int t = 0; t < steps; t += kUnroll) {
+      FVec<kCPL> f[kUnroll];
+      float w[kUnroll];
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) {
+        const int n = 4 * (t + u) + quarter;
+        const bool valid = n < cnt;
+        const int idx = __shfl(myidx, n & (kWave - 1), kWave);
+        f[u] = load_vec<kCPL>(fbase + (int64_t)idx * C, valid);
+        w[u] = valid ? bbase[(int64_t)(m0 + n) * K] : 0.0f;
+      }
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u)
+#pragma unroll
+        for (int j = 0; j < kCPL; ++j)
+          acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(w[u], f[u].v[j], acc[j], 0, 0, 0);
+    }
+  }
+  // D[k][c]: rows k = 4*quarter + r, column col <-> channel col*kCPL + j:
+  // four consecutive basis columns per lane -> one 16-byte store.
+  float *o = out + centre * (int64_t)C * K + (int64_t)chunk * kCW * K + 4 * quarter;
+#pragma unroll
+  for (int j = 0; j < kCPL; ++j) {
+    float *dst = o + (col * kCPL + j) * K;
+    __builtin_nontemporal_store(acc[j], reinterpret_cast<v4f *>(dst));
+  }
+}
+
+// Channels per lane for the matrix-core path, 0 when the shape needs the generic
+// kernel.  Accumulator budget: at most 128 registers per lane.
+static int mfma_channels_per_lane(int C, int K) {
+  if (K == 16) {
+    for (int cpl = 8; cpl >= 1; cpl >>= 1)
+      if (C % (16 * cpl) == 0) return cpl;
+  } else if (K == 32 || K == 64) {
+    for (int cpl = 4; cpl >= 1; cpl >>= 1)
+      if (C % (32 * cpl) == 0) return cpl;
+  }
+  return 0;
+}
+
 static int check_basis_args(const char *op, int64_t basis_rows, int num_basis, int num_features,
                             int64_t num_neighbors, int neighbors_rank, int neighbors_cols) {
   MCCNN_REQUIRE(num_basis == 8 || num_basis == 16 || num_basis == 32 || num_basis == 64,
@@ -152,13 +336,53 @@ extern "C" int mccnn_basis_proj(mccnn_stream_t stream, int64_t basis_rows, int n
   if (num_samples == 0) return MCCNN_OK;
   MCCNN_REQUIRE(ranges && out && (num_neighbors == 0 || (basis && features && neighbors)),
                 "BasisProj received a null tensor");
+  hipStream_t s = as_stream(stream);
+  const int cpl = mfma_channels_per_lane(num_features, num_basis);
+  if (cpl > 0) {
+    const int lanes_per_pair = num_basis == 16 ? 16 : 32;
+    const int chunks = num_features / (lanes_per_pair * cpl);
+    const int64_t waves = num_samples * chunks;
+    MCCNN_REQUIRE(waves < ((int64_t)1 << 31), "BasisProj launch too large");
+    const dim3 grid(blocks_for(waves, 256 / kWave)), block(256);
+    const int2 *nb = (const int2 *)neighbors;
+#define MCCNN_FWD32(K_, CPL_)                                                                  \
+  hipLaunchKernelGGL((basis_proj_mfma32_kernel<K_, CPL_>), grid, block, 0, s, num_samples,     \
+                     num_features, chunks, basis, features, nb, ranges, out)
+#define MCCNN_FWD16(CPL_)                                                                      \
+  hipLaunchKernelGGL((basis_proj_mfma16_kernel<CPL_>), grid, block, 0, s, num_samples,         \
+                     num_features, chunks, basis, features, nb, ranges, out)
+    if (num_basis == 16) {
+      switch (cpl) {
+        case 8: MCCNN_FWD16(8); break;
+        case 4: MCCNN_FWD16(4); break;
+        case 2: MCCNN_FWD16(2); break;
+        default: MCCNN_FWD16(1); break;
+      }
+    } else if (num_basis == 32) {
+      switch (cpl) {
+        case 4: MCCNN_FWD32(32, 4); break;
+        case 2: MCCNN_FWD32(32, 2); break;
+        default: MCCNN_FWD32(32, 1); break;
+      }
+    } else {
+      switch (cpl) {
+        case 4: MCCNN_FWD32(64, 4); break;
+        case 2: MCCNN_FWD32(64, 2); break;
+        default: MCCNN_FWD32(64, 1); break;
+      }
+    }
+#undef MCCNN_FWD32
+#undef MCCNN_FWD16
+    MCCNN_LAUNCH_CHECK();
+    return MCCNN_OK;
+  }
   const int chunks = generic_chunks(num_features, num_basis);
   const int64_t waves = num_samples * chunks;
   MCCNN_REQUIRE(waves < ((int64_t)1 << 31), "BasisProj launch too large");
   const unsigned grid = blocks_for(waves, 256 / kWave);
   MCCNN_BASIS_SWITCH(num_basis,
                      hipLaunchKernelGGL(basis_proj_generic_kernel<K>, dim3(grid), dim3(256), 0,
-                                        as_stream(stream), num_samples, num_features, chunks,
+                                        s, num_samples, num_features, chunks,
                                         basis, features, (const int2 *)neighbors, ranges, out));
   MCCNN_LAUNCH_CHECK();
   return MCCNN_OK;

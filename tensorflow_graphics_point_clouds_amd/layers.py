@@ -24,11 +24,10 @@ class _MCBasis(torch.autograd.Function):
         num_mlps, dims, hidden = weights.shape
         k = num_mlps * hidden
         basis = torch.empty((neighbors.shape[0], k), dtype=_F32, device=weights.device)
-        _lib.check(_lib.lib().mccnn_mc_basis(
-            stream(), i64(neighbors.shape[0]), cint(dims), cint(k), cint(act),
+        _lib.call("mc_basis", stream(), i64(neighbors.shape[0]), cint(dims), cint(k), cint(act),
             ptr(points_in, _F32), ptr(points_out, _F32), ptr(neighbors, _I32),
             ptr(inv_radii, _F32), ptr(weights, _F32), ptr(biases, _F32), cint(num_mlps),
-            ptr(pdf, _F32), ptr(basis)))
+            ptr(pdf, _F32), ptr(basis))
         ctx.save_for_backward(weights, biases, points_in, points_out, neighbors, inv_radii, pdf)
         ctx.act = act
         return basis
@@ -42,12 +41,11 @@ class _MCBasis(torch.autograd.Function):
         ws = _lib.workspace(L.mccnn_mc_basis_grads_workspace_bytes(cint(dims), cint(k)),
                             weights.device)
         dw, db = torch.empty_like(weights), torch.empty_like(biases)
-        _lib.check(L.mccnn_mc_basis_grads(
-            stream(), i64(neighbors.shape[0]), cint(dims), cint(k), cint(ctx.act),
+        _lib.call("mc_basis_grads", stream(), i64(neighbors.shape[0]), cint(dims), cint(k), cint(ctx.act),
             ptr(points_in, _F32), ptr(points_out, _F32), ptr(neighbors, _I32),
             ptr(inv_radii, _F32), ptr(weights, _F32), ptr(biases, _F32), cint(num_mlps),
             ptr(pdf, _F32), ptr(grad.contiguous(), _F32), ptr(ws), _lib.csize(ws.numel()),
-            ptr(dw), ptr(db)))
+            ptr(dw), ptr(db))
         return dw, db, None, None, None, None, None, None
 
 
@@ -157,11 +155,10 @@ class KPConv(torch.nn.Module):
         ids = neighborhood._original_neigh_ids
         kp, k = self._num_kernel_points, self._num_basis
         basis = torch.empty((ids.shape[0], k), dtype=_F32, device=dev)
-        _lib.check(_lib.lib().mccnn_kp_basis(
-            stream(), i64(ids.shape[0]), cint(d), cint(kp), cint(k), cint(self._kind),
+        _lib.call("kp_basis", stream(), i64(ids.shape[0]), cint(d), cint(kp), cint(k), cint(self._kind),
             cfloat(sigma), ptr(point_cloud_in._points, _F32), ptr(point_cloud_out._points, _F32),
             ptr(ids, _I32), ptr(torch.reciprocal(radii), _F32), ptr(self._kernel_points, _F32),
-            ptr(None), ptr(basis), ptr(None)))
+            ptr(None), ptr(basis), ptr(None))
         proj = tfg_custom_ops.basis_proj(basis, features.contiguous(), ids,
                                          neighborhood._samples_neigh_ranges)
         c = self._num_features_in
@@ -177,10 +174,9 @@ class _LocalPool(torch.autograd.Function):
     def forward(ctx, features, neighbors, ranges, kind):
         out = torch.empty((ranges.shape[0], features.shape[1]), dtype=_F32,
                           device=features.device)
-        _lib.check(_lib.lib().mccnn_local_pool(
-            stream(), cint(kind), i64(features.shape[0]), cint(features.shape[1]),
+        _lib.call("local_pool", stream(), cint(kind), i64(features.shape[0]), cint(features.shape[1]),
             ptr(features, _F32), i64(neighbors.shape[0]), ptr(neighbors, _I32),
-            i64(ranges.shape[0]), ptr(ranges, _I32), ptr(out)))
+            i64(ranges.shape[0]), ptr(ranges, _I32), ptr(out))
         ctx.save_for_backward(features, neighbors, ranges, out)
         ctx.kind = kind
         return out
@@ -189,11 +185,10 @@ class _LocalPool(torch.autograd.Function):
     def backward(ctx, grad):
         features, neighbors, ranges, out = ctx.saved_tensors
         dfeat = torch.empty_like(features)
-        _lib.check(_lib.lib().mccnn_local_pool_grads(
-            stream(), cint(ctx.kind), i64(features.shape[0]), cint(features.shape[1]),
+        _lib.call("local_pool_grads", stream(), cint(ctx.kind), i64(features.shape[0]), cint(features.shape[1]),
             ptr(features, _F32), i64(neighbors.shape[0]), ptr(neighbors, _I32),
             i64(ranges.shape[0]), ptr(ranges, _I32), ptr(out, _F32),
-            ptr(grad.contiguous(), _F32), ptr(dfeat)))
+            ptr(grad.contiguous(), _F32), ptr(dfeat))
         return dfeat, None, None, None
 
 
@@ -225,9 +220,8 @@ class _GlobalPool(torch.autograd.Function):
     def forward(ctx, features, batch_ids, batch_size, kind):
         out = torch.empty((batch_size, features.shape[1]), dtype=_F32, device=features.device)
         counts = torch.empty(batch_size, dtype=_I32, device=features.device)
-        _lib.check(_lib.lib().mccnn_global_pool(
-            stream(), cint(kind), i64(features.shape[0]), cint(features.shape[1]),
-            ptr(features, _F32), ptr(batch_ids, _I32), cint(batch_size), ptr(out), ptr(counts)))
+        _lib.call("global_pool", stream(), cint(kind), i64(features.shape[0]), cint(features.shape[1]),
+            ptr(features, _F32), ptr(batch_ids, _I32), cint(batch_size), ptr(out), ptr(counts))
         ctx.save_for_backward(features, batch_ids, out, counts)
         ctx.kind, ctx.batch_size = kind, batch_size
         return out
@@ -237,10 +231,9 @@ class _GlobalPool(torch.autograd.Function):
         features, batch_ids, out, counts = ctx.saved_tensors
         dfeat = torch.empty_like(features)
         tie = torch.empty_like(out) if ctx.kind == 0 else None
-        _lib.check(_lib.lib().mccnn_global_pool_grads(
-            stream(), cint(ctx.kind), i64(features.shape[0]), cint(features.shape[1]),
+        _lib.call("global_pool_grads", stream(), cint(ctx.kind), i64(features.shape[0]), cint(features.shape[1]),
             ptr(features, _F32), ptr(batch_ids, _I32), cint(ctx.batch_size), ptr(out, _F32),
-            ptr(counts, _I32), ptr(grad.contiguous(), _F32), ptr(tie), ptr(dfeat)))
+            ptr(counts, _I32), ptr(grad.contiguous(), _F32), ptr(tie), ptr(dfeat))
         return dfeat, None, None, None
 
 

@@ -62,10 +62,9 @@ class Grid:
         self._num_cells = torch.empty(d, dtype=_I32, device=dev)
         self._scaled_aabb_min = torch.empty((b, d), dtype=_F32, device=dev)
         self._inv_cell_sizes = torch.empty(d, dtype=_F32, device=dev)
-        _lib.check(L.mccnn_grid_setup(
-            stream(), i64(n), cint(d), ptr(pc._points, _F32), ptr(pc._batch_ids, _I32), cint(b),
+        _lib.call("grid_setup", stream(), i64(n), cint(d), ptr(pc._points, _F32), ptr(pc._batch_ids, _I32), cint(b),
             ptr(self._cell_sizes), ptr(self._aabb_min), ptr(self._aabb_max),
-            ptr(self._num_cells), ptr(self._scaled_aabb_min), ptr(self._inv_cell_sizes)))
+            ptr(self._num_cells), ptr(self._scaled_aabb_min), ptr(self._inv_cell_sizes))
         self._cur_keys = tfg_custom_ops.compute_keys(
             pc._points, pc._batch_ids, self._scaled_aabb_min, self._num_cells,
             self._inv_cell_sizes)
@@ -78,14 +77,12 @@ class Grid:
         self._sorted_keys = torch.empty(n, dtype=_I64, device=dev)
         self._sorted_indices = torch.empty(n, dtype=_I32, device=dev)
         ws = _lib.workspace(L.mccnn_sort_keys_workspace_bytes(i64(n)), dev)
-        _lib.check(L.mccnn_sort_keys_descending(
-            stream(), i64(n), cint(key_bits), ptr(self._cur_keys), ptr(self._sorted_keys),
-            ptr(self._sorted_indices), ptr(ws), _lib.csize(ws.numel())))
+        _lib.call("sort_keys_descending", stream(), i64(n), cint(key_bits), ptr(self._cur_keys), ptr(self._sorted_keys),
+            ptr(self._sorted_indices), ptr(ws), _lib.csize(ws.numel()))
         self._sorted_points = torch.empty_like(pc._points)
         self._sorted_batch_ids = torch.empty_like(pc._batch_ids)
-        _lib.check(L.mccnn_gather_points(
-            stream(), i64(n), cint(d), ptr(pc._points), ptr(pc._batch_ids),
-            ptr(self._sorted_indices), ptr(self._sorted_points), ptr(self._sorted_batch_ids)))
+        _lib.call("gather_points", stream(), i64(n), cint(d), ptr(pc._points), ptr(pc._batch_ids),
+            ptr(self._sorted_indices), ptr(self._sorted_points), ptr(self._sorted_batch_ids))
         self._fast_DS = None
 
     def get_DS(self):
@@ -120,9 +117,8 @@ class Neighborhood:
             max_neighbors)
         # pairs addressed by original point ids (Neighborhood.py:246-250)
         self._original_neigh_ids = torch.empty_like(self._neighbors)
-        _lib.check(_lib.lib().mccnn_original_neighbor_ids(
-            stream(), i64(self._neighbors.shape[0]), ptr(self._neighbors, _I32),
-            ptr(grid._sorted_indices, _I32), ptr(self._original_neigh_ids)))
+        _lib.call("original_neighbor_ids", stream(), i64(self._neighbors.shape[0]), ptr(self._neighbors, _I32),
+            ptr(grid._sorted_indices, _I32), ptr(self._original_neigh_ids))
         self._pdf = None
         self._pdf_per_point = None
 
@@ -138,9 +134,8 @@ class Neighborhood:
                 self._grid._sorted_points, nbh._neighbors, nbh._samples_neigh_ranges,
                 torch.reciprocal(bw), nbh._inv_radii, mode.value)
             self._pdf = torch.empty(self._neighbors.shape[0], dtype=_F32, device=dev)
-            _lib.check(_lib.lib().mccnn_gather_pdf(
-                stream(), i64(self._neighbors.shape[0]), ptr(self._neighbors, _I32),
-                ptr(self._pdf_per_point.detach(), _F32), ptr(self._pdf)))
+            _lib.call("gather_pdf", stream(), i64(self._neighbors.shape[0]), ptr(self._neighbors, _I32),
+                ptr(self._pdf_per_point.detach(), _F32), ptr(self._pdf))
         if normalize:
             raise NotImplementedError("normalised densities are not part of the op path")
 
@@ -164,9 +159,8 @@ def sample(neighborhood, sample_mode="poisson"):
     original = None
     if mode == 0:
         original = torch.empty_like(idx)
-        _lib.check(_lib.lib().mccnn_gather_i32(
-            stream(), i64(idx.shape[0]), ptr(g._sorted_indices, _I32), ptr(idx, _I32),
-            ptr(original)))
+        _lib.call("gather_i32", stream(), i64(idx.shape[0]), ptr(g._sorted_indices, _I32), ptr(idx, _I32),
+            ptr(original))
     return PointCloud(pts, bids, g._batch_size), original
 
 

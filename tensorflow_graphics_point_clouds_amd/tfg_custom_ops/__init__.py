@@ -27,12 +27,11 @@ def _dim(t, axis, default=-1):
 def compute_keys(points, batch_ids, scaled_aabb_min, num_cells, inv_cell_sizes):
     """ComputeKeys (compute_keys_ops.cpp:29-41): int64 cell key per point."""
     keys = torch.empty(points.shape[0], dtype=_I64, device=points.device)
-    _lib.check(_lib.lib().mccnn_compute_keys(
-        stream(), i64(points.shape[0]), cint(_dim(points, 1)), ptr(points, _F32),
+    _lib.call("compute_keys", stream(), i64(points.shape[0]), cint(_dim(points, 1)), ptr(points, _F32),
         i64(batch_ids.shape[0]), ptr(batch_ids, _I32),
         i64(scaled_aabb_min.shape[0]), cint(_dim(scaled_aabb_min, 1)),
         ptr(scaled_aabb_min, _F32), cint(num_cells.shape[0]), ptr(num_cells, _I32),
-        cint(inv_cell_sizes.shape[0]), ptr(inv_cell_sizes, _F32), ptr(keys)))
+        cint(inv_cell_sizes.shape[0]), ptr(inv_cell_sizes, _F32), ptr(keys))
     return keys
 
 
@@ -48,9 +47,8 @@ def build_grid_ds(sorted_keys, num_cells, num_cells_host, batch_size):
     import ctypes
     host_arr = (ctypes.c_int32 * len(host))(*host)
     ds = torch.empty((batch_size, host[0], host[1], 2), dtype=_I32, device=sorted_keys.device)
-    _lib.check(_lib.lib().mccnn_build_grid_ds(
-        stream(), i64(sorted_keys.shape[0]), ptr(sorted_keys, _I64), cint(num_cells.shape[0]),
-        ptr(num_cells, _I32), cint(len(host)), host_arr, cint(batch_size), ptr(ds)))
+    _lib.call("build_grid_ds", stream(), i64(sorted_keys.shape[0]), ptr(sorted_keys, _I64), cint(num_cells.shape[0]),
+        ptr(num_cells, _I32), cint(len(host)), host_arr, cint(batch_size), ptr(ds))
     return ds
 
 
@@ -67,8 +65,7 @@ def find_neighbors(samples, samples_batch_ids, points, point_keys, grid_acc_ds, 
     ranges = torch.empty(ns, dtype=_I32, device=dev)
     total = ctypes.c_int64(0)
     dsr = grid_acc_ds.dim()
-    _lib.check(L.mccnn_find_neighbors_count(
-        stream(), i64(ns), cint(nd), ptr(samples, _F32), i64(samples_batch_ids.shape[0]),
+    _lib.call("find_neighbors_count", stream(), i64(ns), cint(nd), ptr(samples, _F32), i64(samples_batch_ids.shape[0]),
         ptr(samples_batch_ids, _I32), i64(points.shape[0]), cint(_dim(points, 1)),
         ptr(points, _F32), i64(point_keys.shape[0]), ptr(point_keys, _I64), cint(dsr),
         cint(_dim(grid_acc_ds, 0)), cint(_dim(grid_acc_ds, 1)), cint(_dim(grid_acc_ds, 2)),
@@ -76,15 +73,14 @@ def find_neighbors(samples, samples_batch_ids, points, point_keys, grid_acc_ds, 
         ptr(num_cells, _I32), cint(_dim(scaled_aabb_min, 1)), ptr(scaled_aabb_min, _F32),
         cint(inv_cell_sizes.shape[0]), ptr(inv_cell_sizes, _F32), cint(inv_radii.shape[0]),
         ptr(inv_radii, _F32), cint(max_neighs), ptr(ws), _lib.csize(ws.numel()), ptr(ranges),
-        ctypes.byref(total)))
+        ctypes.byref(total))
     m = int(total.value)
     neighbors = torch.empty((m, 2), dtype=_I32, device=dev)
-    _lib.check(L.mccnn_find_neighbors_fill(
-        stream(), i64(ns), cint(nd), ptr(samples, _F32), ptr(samples_batch_ids, _I32),
+    _lib.call("find_neighbors_fill", stream(), i64(ns), cint(nd), ptr(samples, _F32), ptr(samples_batch_ids, _I32),
         i64(points.shape[0]), ptr(points, _F32), ptr(point_keys, _I64), ptr(grid_acc_ds, _I32),
         ptr(num_cells, _I32), ptr(scaled_aabb_min, _F32), ptr(inv_cell_sizes, _F32),
         ptr(inv_radii, _F32), cint(max_neighs), ptr(ws), _lib.csize(ws.numel()), ptr(ranges),
-        i64(m), ptr(neighbors)))
+        i64(m), ptr(neighbors))
     return ranges, neighbors
 
 
@@ -97,32 +93,29 @@ def sampling(points, batch_ids, point_keys, num_cells, neighbors, sample_neigh_i
     dev = points.device
     ws = _lib.workspace(L.mccnn_sampling_workspace_bytes(i64(n)), dev)
     total = ctypes.c_int64(0)
-    _lib.check(L.mccnn_sampling_count(
-        stream(), cint(mode), i64(n), cint(nd), ptr(points, _F32), i64(batch_ids.shape[0]),
+    _lib.call("sampling_count", stream(), cint(mode), i64(n), cint(nd), ptr(points, _F32), i64(batch_ids.shape[0]),
         ptr(batch_ids, _I32), i64(point_keys.shape[0]), ptr(point_keys, _I64),
         cint(num_cells.shape[0]), ptr(num_cells, _I32), i64(neighbors.shape[0]),
         cint(neighbors.dim()), cint(_dim(neighbors, 1)), ptr(neighbors, _I32),
         i64(sample_neigh_indices.shape[0]), ptr(sample_neigh_indices, _I32), ptr(ws),
-        _lib.csize(ws.numel()), ctypes.byref(total)))
+        _lib.csize(ws.numel()), ctypes.byref(total))
     s = int(total.value)
     out_pts = torch.empty((s, nd), dtype=_F32, device=dev)
     out_bids = torch.empty(s, dtype=_I32, device=dev)
     out_idx = torch.empty(s, dtype=_I32, device=dev)
-    _lib.check(L.mccnn_sampling_fill(
-        stream(), cint(mode), i64(n), cint(nd), ptr(points, _F32), ptr(batch_ids, _I32),
+    _lib.call("sampling_fill", stream(), cint(mode), i64(n), cint(nd), ptr(points, _F32), ptr(batch_ids, _I32),
         ptr(point_keys, _I64), ptr(num_cells, _I32), ptr(ws), _lib.csize(ws.numel()), i64(s),
-        ptr(out_pts), ptr(out_bids), ptr(out_idx)))
+        ptr(out_pts), ptr(out_bids), ptr(out_idx))
     return out_pts, out_bids, out_idx
 
 
 def _compute_pdf_raw(points, neighbors, ranges, inv_bandwidth, inv_radii, mode):
     pdf = torch.empty(ranges.shape[0], dtype=_F32, device=points.device)
-    _lib.check(_lib.lib().mccnn_compute_pdf(
-        stream(), i64(points.shape[0]), cint(_dim(points, 1)), ptr(points, _F32),
+    _lib.call("compute_pdf", stream(), i64(points.shape[0]), cint(_dim(points, 1)), ptr(points, _F32),
         i64(neighbors.shape[0]), cint(neighbors.dim()), cint(_dim(neighbors, 1)),
         ptr(neighbors, _I32), i64(ranges.shape[0]), ptr(ranges, _I32),
         cint(inv_bandwidth.shape[0]), ptr(inv_bandwidth, _F32), cint(inv_radii.shape[0]),
-        ptr(inv_radii, _F32), cint(mode), ptr(pdf)))
+        ptr(inv_radii, _F32), cint(mode), ptr(pdf))
     return pdf
 
 
@@ -131,13 +124,12 @@ def compute_pdf_pt_grads(points, neighbors, sample_neigh_indices, inv_bandwidth,
     """ComputePdfPtGrads (compute_pdf_ops.cpp:58-74): [N, D] gradient of
     sum(pdf_grads * pdf) with respect to the points."""
     out = torch.empty_like(points)
-    _lib.check(_lib.lib().mccnn_compute_pdf_pt_grads(
-        stream(), i64(points.shape[0]), cint(_dim(points, 1)), ptr(points, _F32),
+    _lib.call("compute_pdf_pt_grads", stream(), i64(points.shape[0]), cint(_dim(points, 1)), ptr(points, _F32),
         i64(neighbors.shape[0]), cint(neighbors.dim()), cint(_dim(neighbors, 1)),
         ptr(neighbors, _I32), i64(sample_neigh_indices.shape[0]),
         ptr(sample_neigh_indices, _I32), cint(inv_bandwidth.shape[0]),
         ptr(inv_bandwidth, _F32), cint(inv_radii.shape[0]), ptr(inv_radii, _F32),
-        i64(pdf_grads.shape[0]), ptr(pdf_grads, _F32), cint(mode), ptr(out)))
+        i64(pdf_grads.shape[0]), ptr(pdf_grads, _F32), cint(mode), ptr(out))
     return out
 
 
@@ -167,11 +159,10 @@ def compute_pdf_with_pt_grads(points, neighbors, sample_neigh_indices, inv_bandw
 def _basis_proj_raw(basis, features, neighbors, ranges):
     out = torch.empty((ranges.shape[0], _dim(features, 1), _dim(basis, 1)), dtype=_F32,
                       device=features.device)
-    _lib.check(_lib.lib().mccnn_basis_proj(
-        stream(), i64(basis.shape[0]), cint(_dim(basis, 1)), ptr(basis, _F32),
+    _lib.call("basis_proj", stream(), i64(basis.shape[0]), cint(_dim(basis, 1)), ptr(basis, _F32),
         i64(features.shape[0]), cint(_dim(features, 1)), ptr(features, _F32),
         i64(neighbors.shape[0]), cint(neighbors.dim()), cint(_dim(neighbors, 1)),
-        ptr(neighbors, _I32), i64(ranges.shape[0]), ptr(ranges, _I32), ptr(out)))
+        ptr(neighbors, _I32), i64(ranges.shape[0]), ptr(ranges, _I32), ptr(out))
     return out
 
 
@@ -182,13 +173,12 @@ def basis_proj_grads(basis_neighbors, pt_features, neighbors, sample_neigh_indic
     dbasis = torch.empty_like(basis_neighbors)
     dfeat = torch.empty_like(pt_features)
     g = in_gradients
-    _lib.check(_lib.lib().mccnn_basis_proj_grads(
-        stream(), i64(basis_neighbors.shape[0]), cint(_dim(basis_neighbors, 1)),
+    _lib.call("basis_proj_grads", stream(), i64(basis_neighbors.shape[0]), cint(_dim(basis_neighbors, 1)),
         ptr(basis_neighbors, _F32), i64(pt_features.shape[0]), cint(_dim(pt_features, 1)),
         ptr(pt_features, _F32), i64(neighbors.shape[0]), cint(neighbors.dim()),
         cint(_dim(neighbors, 1)), ptr(neighbors, _I32), i64(sample_neigh_indices.shape[0]),
         ptr(sample_neigh_indices, _I32), cint(g.dim()), i64(_dim(g, 0)), i64(_dim(g, 1)),
-        i64(_dim(g, 2)), ptr(g, _F32), ptr(dbasis), ptr(dfeat)))
+        i64(_dim(g, 2)), ptr(g, _F32), ptr(dbasis), ptr(dfeat))
     return dbasis, dfeat
 
 
