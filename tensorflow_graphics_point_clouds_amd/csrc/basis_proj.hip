@@ -277,6 +277,152 @@ __global__ void __launch_bounds__(256) basis_proj_mfma16_kernel(
   }
 }
 
+// ---------------------------------------------------------------------------
+// Matrix-core gradient path.  One wavefront owns a centre and walks its pairs in
+// tiles of 32 (K = 32) or 16 (K = 16).  Per tile, two contractions:
+//   dbasis^T [K x pairs]   = G^T [K x C] * F^T [C x pairs]   (reduction over c)
+//   dfeat    [pairs x C]   = B [pairs x K] * G^T [K x C]     (reduction over k)
+// with G = in_grad[centre] ([C, K]).  The reduction index of an MFMA may be
+// permuted freely as long as both operands agree, so each lane is given a
+// CONTIGUOUS run of the reduction index: its share of a feature row, of a basis
+// row and of a G row are 16-byte vector loads.  dbasis rows leave as contiguous
+// 16-byte stores (each pair belongs to exactly one centre: no atomics); dfeat
+// rows are added with one fp32 atomic per element, 64/128 consecutive bytes per
+// row and instruction.
+
+template <int C>
+__global__ void __launch_bounds__(256) basis_proj_grads_mfma32_kernel(
+    int64_t n_out, const float *__restrict__ basis, const float *__restrict__ feat,
+    const int2 *__restrict__ nbrs, const int *__restrict__ ranges,
+    const float *__restrict__ in_grad, float *__restrict__ dbasis, float *__restrict__ dfeat) {
+  constexpr int K = 32;
+  constexpr int kHalfC = C / 2;      // reduction run of a lane in the dbasis product
+  const int lane = lane_id();
+  const int64_t centre =
+      __builtin_amdgcn_readfirstlane((int)((blockIdx.x * (int64_t)blockDim.x + threadIdx.x) / kWave));
+  if (centre >= n_out) return;
+  const int half = lane >> 5, col = lane & 31;
+  const int a = centre > 0 ? ranges[centre - 1] : 0, b = ranges[centre];
+  if (b <= a) return;
+  const float *gi = in_grad + centre * (int64_t)C * K;
+  // A operand of the dbasis product: G[c = half*C/2 + s][k = col]
+  float gk[kHalfC];
+#pragma unroll
+  for (int s = 0; s < kHalfC; ++s) gk[s] = gi[(half * kHalfC + s) * K + col];
+
+  for (int m0 = a; m0 < b; m0 += 32) {
+    const int cnt = b - m0 < 32 ? b - m0 : 32;
+    const bool valid = col < cnt;
+    const int idx = nbrs[m0 + (valid ? col : 0)].x;
+    // ---- dbasis: D[i = k][j = pair]; B operand F[nbr_col][half*C/2 + s]
+    {
+      const FVec<kHalfC> f = load_vec<kHalfC>(feat + (int64_t)idx * C + half * kHalfC, valid);
+      v16f acc;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
+#pragma unroll
+      for (int s = 0; s < kHalfC; ++s)
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(gk[s], f.v[s], acc, 0, 0, 0);
+      // rows k = 8q + 4*half + (0..3) of column pair `col`
+      if (valid) {
+        float *dst = dbasis + (int64_t)(m0 + col) * K + 4 * half;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          v4f v = {acc[4 * q], acc[4 * q + 1], acc[4 * q + 2], acc[4 * q + 3]};
+          __builtin_nontemporal_store(v, reinterpret_cast<v4f *>(dst + 8 * q));
+        }
+      }
+    }
+    // ---- dfeat: D[i = pair][j = channel]; A operand B[pair col][k = 16*half + s]
+    {
+      const FVec<16> w = load_vec<16>(basis + (int64_t)(m0 + col) * K + 16 * half, valid);
+#pragma unroll 1
+      for (int ct = 0; ct < C; ct += 32) {
+        const FVec<16> gt = load_vec<16>(gi + (ct + col) * K + 16 * half, true);
+        v16f acc;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
+#pragma unroll
+        for (int s = 0; s < 16; ++s)
+          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(w.v[s], gt.v[s], acc, 0, 0, 0);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int n = 8 * (r >> 2) + (r & 3) + 4 * half;
+          const int nidx = __shfl(idx, n, kWave);
+          if (n < cnt) unsafeAtomicAdd(dfeat + (int64_t)nidx * C + ct + col, acc[r]);
+        }
+      }
+    }
+  }
+}
+
+template <int C>
+__global__ void __launch_bounds__(256) basis_proj_grads_mfma16_kernel(
+    int64_t n_out, const float *__restrict__ basis, const float *__restrict__ feat,
+    const int2 *__restrict__ nbrs, const int *__restrict__ ranges,
+    const float *__restrict__ in_grad, float *__restrict__ dbasis, float *__restrict__ dfeat) {
+  constexpr int K = 16;
+  constexpr int kQuarterC = C / 4;
+  constexpr int kTiles = C / 16;
+  const int lane = lane_id();
+  const int64_t centre =
+      __builtin_amdgcn_readfirstlane((int)((blockIdx.x * (int64_t)blockDim.x + threadIdx.x) / kWave));
+  if (centre >= n_out) return;
+  const int quarter = lane >> 4, col = lane & 15;
+  const int a = centre > 0 ? ranges[centre - 1] : 0, b = ranges[centre];
+  if (b <= a) return;
+  const float *gi = in_grad + centre * (int64_t)C * K;
+  // dbasis product, A operand: G[c = quarter*C/4 + s][k = col]
+  float gk[kQuarterC];
+#pragma unroll
+  for (int s = 0; s < kQuarterC; ++s) gk[s] = gi[(quarter * kQuarterC + s) * K + col];
+  // dfeat product, B operand of channel tile t: G[c = 16 t + col][k = 4*quarter + s]
+  FVec<4> gt[kTiles];
+#pragma unroll
+  for (int t = 0; t < kTiles; ++t) gt[t] = load_vec<4>(gi + (16 * t + col) * K + 4 * quarter, true);
+
+  for (int m0 = a; m0 < b; m0 += 16) {
+    const int cnt = b - m0 < 16 ? b - m0 : 16;
+    const bool valid = col < cnt;
+    const int idx = nbrs[m0 + (valid ? col : 0)].x;
+    {
+      const FVec<kQuarterC> f =
+          load_vec<kQuarterC>(feat + (int64_t)idx * C + quarter * kQuarterC, valid);
+      v4f acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+      for (int s = 0; s < kQuarterC; ++s)
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(gk[s], f.v[s], acc, 0, 0, 0);
+      // D[i = k][j = pair]: rows k = 4*quarter + (0..3)
+      if (valid)
+        __builtin_nontemporal_store(
+            acc, reinterpret_cast<v4f *>(dbasis + (int64_t)(m0 + col) * K + 4 * quarter));
+    }
+    {
+      const FVec<4> w = load_vec<4>(basis + (int64_t)(m0 + col) * K + 4 * quarter, valid);
+#pragma unroll
+      for (int t = 0; t < kTiles; ++t) {
+        v4f acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int s = 0; s < 4; ++s)
+          acc = __builtin_amdgcn_mfma_f32_16x16x4f32(w.v[s], gt[t].v[s], acc, 0, 0, 0);
+        // D[i = pair][j = channel]: rows pair = 4*quarter + r, column channel 16 t + col
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int n = 4 * quarter + r;
+          const int nidx = __shfl(idx, n, kWave);
+          if (n < cnt) unsafeAtomicAdd(dfeat + (int64_t)nidx * C + 16 * t + col, acc[r]);
+        }
+      }
+    }
+  }
+}
+
+static bool mfma_grads_supported(int C, int K) {
+  if (K == 32) return C == 32 || C == 64 || C == 128;
+  if (K == 16) return C == 16 || C == 32 || C == 64 || C == 128;
+  return false;
+}
+
 // Channels per lane for the matrix-core path, 0 when the shape needs the generic
 // kernel.  Accumulator budget: at most 128 registers per lane.
 static int mfma_channels_per_lane(int C, int K) {
@@ -415,6 +561,31 @@ extern "C" int mccnn_basis_proj_grads(mccnn_stream_t stream, int64_t basis_rows,
   if (num_samples == 0 || num_neighbors == 0) return MCCNN_OK;
   MCCNN_REQUIRE(ranges && basis && features && neighbors && in_grads && basis_grads_out,
                 "BasisProjGrads received a null tensor");
+  const int2 *nb = (const int2 *)neighbors;
+  if (mfma_grads_supported(num_features, num_basis)) {
+    MCCNN_REQUIRE(num_samples < ((int64_t)1 << 31), "BasisProjGrads launch too large");
+    const dim3 grid(blocks_for(num_samples, 256 / kWave)), block(256);
+#define MCCNN_BWD(KERNEL_, C_)                                                              \
+  hipLaunchKernelGGL((KERNEL_<C_>), grid, block, 0, s, num_samples, basis, features, nb,   \
+                     ranges, in_grads, basis_grads_out, feature_grads_out)
+    if (num_basis == 32) {
+      switch (num_features) {
+        case 32: MCCNN_BWD(basis_proj_grads_mfma32_kernel, 32); break;
+        case 64: MCCNN_BWD(basis_proj_grads_mfma32_kernel, 64); break;
+        default: MCCNN_BWD(basis_proj_grads_mfma32_kernel, 128); break;
+      }
+    } else {
+      switch (num_features) {
+        case 16: MCCNN_BWD(basis_proj_grads_mfma16_kernel, 16); break;
+        case 32: MCCNN_BWD(basis_proj_grads_mfma16_kernel, 32); break;
+        case 64: MCCNN_BWD(basis_proj_grads_mfma16_kernel, 64); break;
+        default: MCCNN_BWD(basis_proj_grads_mfma16_kernel, 128); break;
+      }
+    }
+#undef MCCNN_BWD
+    MCCNN_LAUNCH_CHECK();
+    return MCCNN_OK;
+  }
   const int chunks = generic_chunks(num_features, num_basis);
   if (chunks > 1) {
     rc = fill_zero(s, basis_grads_out, sizeof(float) * (size_t)num_neighbors * num_basis);
@@ -425,8 +596,7 @@ extern "C" int mccnn_basis_proj_grads(mccnn_stream_t stream, int64_t basis_rows,
   const unsigned grid = blocks_for(waves, 256 / kWave);
   MCCNN_BASIS_SWITCH(num_basis, hipLaunchKernelGGL(basis_proj_grads_generic_kernel<K>, dim3(grid),
                                                    dim3(256), 0, s, num_samples, num_features,
-                                                   chunks, basis, features,
-                                                   (const int2 *)neighbors, ranges, in_grads,
+                                                   chunks, basis, features, nb, ranges, in_grads,
                                                    basis_grads_out, feature_grads_out));
   MCCNN_LAUNCH_CHECK();
   return MCCNN_OK;
