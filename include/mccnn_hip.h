@@ -208,6 +208,28 @@ int mccnn_basis_proj_grads(mccnn_stream_t stream, int64_t basis_rows,
                            const float *in_grads, float *basis_grads_out,
                            float *feature_grads_out);
 
+/* The two ops above with a visiting order for the centres: centre_order
+ * [num_samples] is a permutation of the centre indices (NULL = natural order).
+ * Results are identical; only the schedule changes.  Passing the centres in
+ * spatial order (e.g. sorted by grid cell key) keeps the feature rows shared by
+ * neighbouring centres in L2.  No counterpart in the reference, whose kernels
+ * always walk the centres in index order. */
+int mccnn_basis_proj_ordered(mccnn_stream_t stream, int64_t basis_rows,
+                             int num_basis, const float *basis, int64_t num_pts,
+                             int num_features, const float *features,
+                             int64_t num_neighbors, int neighbors_rank,
+                             int neighbors_cols, const int32_t *neighbors,
+                             int64_t num_samples, const int32_t *ranges,
+                             const int32_t *centre_order, float *out);
+int mccnn_basis_proj_grads_ordered(
+    mccnn_stream_t stream, int64_t basis_rows, int num_basis, const float *basis,
+    int64_t num_pts, int num_features, const float *features,
+    int64_t num_neighbors, int neighbors_rank, int neighbors_cols,
+    const int32_t *neighbors, int64_t num_samples, const int32_t *ranges,
+    const int32_t *centre_order, int in_grads_rank, int64_t in_grads_dim0,
+    int64_t in_grads_dim1, int64_t in_grads_dim2, const float *in_grads,
+    float *basis_grads_out, float *feature_grads_out);
+
 /* ------------------------------------------------------------- sampling --- */
 
 /* Sampling: sampling/cc/ops/sampling_ops.cpp:33-204, split at the host

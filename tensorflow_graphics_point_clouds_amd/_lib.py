@@ -7,7 +7,8 @@ import os
 import subprocess
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libmccnn_hip.so")
+# MCCNN_HIP_LIBRARY selects another build of the same library (e.g. an experiment).
+LIB_PATH = os.environ.get("MCCNN_HIP_LIBRARY") or os.path.join(_HERE, "libmccnn_hip.so")
 CSRC_DIR = os.path.join(_HERE, "csrc")
 
 _lib = None

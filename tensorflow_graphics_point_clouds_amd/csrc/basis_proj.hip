@@ -20,18 +20,40 @@ namespace mccnn {
 
 constexpr int kAcc = 16;   // accumulators per lane in the generic kernels
 
+// Wave slot -> centre.  `order` (optional) is a permutation of the centres that
+// fixes the visiting order; it is a scheduling hint only.  (Dealing contiguous
+// slot ranges to the 8 XCDs and visiting the centres in cell order were both
+// measured and left out: the feature rows already hit the memory-side cache,
+// and concentrating the feature-gradient atomics of neighbouring centres in
+// time made them slower.)
+constexpr int kWavesPerBlock = 256 / kWave;
+
+__device__ __forceinline__ int64_t wave_slot() {
+  return __builtin_amdgcn_readfirstlane(
+      (int)(blockIdx.x * kWavesPerBlock + threadIdx.x / kWave));
+}
+
+__device__ __forceinline__ int64_t centre_of(int64_t slot_centre, const int *__restrict__ order) {
+  return order ? (int64_t)__builtin_amdgcn_readfirstlane(order[slot_centre]) : slot_centre;
+}
+
+static unsigned wave_grid(int64_t waves) {
+  const int64_t blocks = (waves + kWavesPerBlock - 1) / kWavesPerBlock;
+  return (unsigned)(blocks < 1 ? 1 : blocks);
+}
+
 template <int K>
 __global__ void __launch_bounds__(256) basis_proj_generic_kernel(
     int64_t n_out, int C, int chunks, const float *__restrict__ basis,
     const float *__restrict__ feat, const int2 *__restrict__ nbrs,
-    const int *__restrict__ ranges, float *__restrict__ out) {
+    const int *__restrict__ ranges, const int *__restrict__ order, float *__restrict__ out) {
   constexpr int kChanStep = kWave / K;            // channels covered by one j
   const int lane = lane_id();
-  const int64_t wid =
-      __builtin_amdgcn_readfirstlane((int)((blockIdx.x * (int64_t)blockDim.x + threadIdx.x) / kWave));
-  const int64_t centre = wid / chunks;
-  if (centre >= n_out) return;
-  const int chunk = (int)(wid - centre * chunks);
+  const int64_t wid = wave_slot();
+  const int64_t slot_centre = wid / chunks;
+  if (slot_centre >= n_out) return;
+  const int chunk = (int)(wid - slot_centre * chunks);
+  const int64_t centre = centre_of(slot_centre, order);
   const int c0 = chunk * kAcc * kChanStep + lane / K;
   const int k = lane % K;
   const int a = centre > 0 ? ranges[centre - 1] : 0, b = ranges[centre];
@@ -61,15 +83,15 @@ template <int K>
 __global__ void __launch_bounds__(256) basis_proj_grads_generic_kernel(
     int64_t n_out, int C, int chunks, const float *__restrict__ basis,
     const float *__restrict__ feat, const int2 *__restrict__ nbrs,
-    const int *__restrict__ ranges, const float *__restrict__ in_grad,
+    const int *__restrict__ ranges, const int *__restrict__ order, const float *__restrict__ in_grad,
     float *__restrict__ dbasis, float *__restrict__ dfeat) {
   constexpr int kChanStep = kWave / K;
   const int lane = lane_id();
-  const int64_t wid =
-      __builtin_amdgcn_readfirstlane((int)((blockIdx.x * (int64_t)blockDim.x + threadIdx.x) / kWave));
-  const int64_t centre = wid / chunks;
-  if (centre >= n_out) return;
-  const int chunk = (int)(wid - centre * chunks);
+  const int64_t wid = wave_slot();
+  const int64_t slot_centre = wid / chunks;
+  if (slot_centre >= n_out) return;
+  const int chunk = (int)(wid - slot_centre * chunks);
+  const int64_t centre = centre_of(slot_centre, order);
   const int c0 = chunk * kAcc * kChanStep + lane / K;
   const int k = lane % K;
   const int a = centre > 0 ? ranges[centre - 1] : 0, b = ranges[centre];
@@ -158,16 +180,16 @@ template <int K, int kCPL>
 __global__ void __launch_bounds__(256) basis_proj_mfma32_kernel(
     int64_t n_out, int C, int chunks, const float *__restrict__ basis,
     const float *__restrict__ feat, const int2 *__restrict__ nbrs,
-    const int *__restrict__ ranges, float *__restrict__ out) {
+    const int *__restrict__ ranges, const int *__restrict__ order, float *__restrict__ out) {
   static_assert(K == 32 || K == 64, "32x32x2 path");
   constexpr int kNT = K / 32;        // basis columns per lane
   constexpr int kCW = 32 * kCPL;     // channels per wave
   const int lane = lane_id();
-  const int64_t wid =
-      __builtin_amdgcn_readfirstlane((int)((blockIdx.x * (int64_t)blockDim.x + threadIdx.x) / kWave));
-  const int64_t centre = wid / chunks;
-  if (centre >= n_out) return;
-  const int chunk = (int)(wid - centre * chunks);
+  const int64_t wid = wave_slot();
+  const int64_t slot_centre = wid / chunks;
+  if (slot_centre >= n_out) return;
+  const int chunk = (int)(wid - slot_centre * chunks);
+  const int64_t centre = centre_of(slot_centre, order);
   const int half = lane >> 5, col = lane & 31;
   const int a = centre > 0 ? ranges[centre - 1] : 0, b = ranges[centre];
   const float *fbase = feat + chunk * kCW + col * kCPL;
@@ -226,15 +248,15 @@ template <int kCPL>
 __global__ void __launch_bounds__(256) basis_proj_mfma16_kernel(
     int64_t n_out, int C, int chunks, const float *__restrict__ basis,
     const float *__restrict__ feat, const int2 *__restrict__ nbrs,
-    const int *__restrict__ ranges, float *__restrict__ out) {
+    const int *__restrict__ ranges, const int *__restrict__ order, float *__restrict__ out) {
   constexpr int K = 16;
   constexpr int kCW = 16 * kCPL;
   const int lane = lane_id();
-  const int64_t wid =
-      __builtin_amdgcn_readfirstlane((int)((blockIdx.x * (int64_t)blockDim.x + threadIdx.x) / kWave));
-  const int64_t centre = wid / chunks;
-  if (centre >= n_out) return;
-  const int chunk = (int)(wid - centre * chunks);
+  const int64_t wid = wave_slot();
+  const int64_t slot_centre = wid / chunks;
+  if (slot_centre >= n_out) return;
+  const int chunk = (int)(wid - slot_centre * chunks);
+  const int64_t centre = centre_of(slot_centre, order);
   const int quarter = lane >> 4, col = lane & 15;
   const int a = centre > 0 ? ranges[centre - 1] : 0, b = ranges[centre];
   const float *fbase = feat + chunk * kCW + col * kCPL;
@@ -293,14 +315,14 @@ __global__ void __launch_bounds__(256) basis_proj_mfma16_kernel(
 template <int C>
 __global__ void __launch_bounds__(256) basis_proj_grads_mfma32_kernel(
     int64_t n_out, const float *__restrict__ basis, const float *__restrict__ feat,
-    const int2 *__restrict__ nbrs, const int *__restrict__ ranges,
+    const int2 *__restrict__ nbrs, const int *__restrict__ ranges, const int *__restrict__ order,
     const float *__restrict__ in_grad, float *__restrict__ dbasis, float *__restrict__ dfeat) {
   constexpr int K = 32;
   constexpr int kHalfC = C / 2;      // reduction run of a lane in the dbasis product
   const int lane = lane_id();
-  const int64_t centre =
-      __builtin_amdgcn_readfirstlane((int)((blockIdx.x * (int64_t)blockDim.x + threadIdx.x) / kWave));
-  if (centre >= n_out) return;
+  const int64_t slot_centre = wave_slot();
+  if (slot_centre >= n_out) return;
+  const int64_t centre = centre_of(slot_centre, order);
   const int half = lane >> 5, col = lane & 31;
   const int a = centre > 0 ? ranges[centre - 1] : 0, b = ranges[centre];
   if (b <= a) return;
@@ -359,15 +381,15 @@ __global__ void __launch_bounds__(256) basis_proj_grads_mfma32_kernel(
 template <int C>
 __global__ void __launch_bounds__(256) basis_proj_grads_mfma16_kernel(
     int64_t n_out, const float *__restrict__ basis, const float *__restrict__ feat,
-    const int2 *__restrict__ nbrs, const int *__restrict__ ranges,
+    const int2 *__restrict__ nbrs, const int *__restrict__ ranges, const int *__restrict__ order,
     const float *__restrict__ in_grad, float *__restrict__ dbasis, float *__restrict__ dfeat) {
   constexpr int K = 16;
   constexpr int kQuarterC = C / 4;
   constexpr int kTiles = C / 16;
   const int lane = lane_id();
-  const int64_t centre =
-      __builtin_amdgcn_readfirstlane((int)((blockIdx.x * (int64_t)blockDim.x + threadIdx.x) / kWave));
-  if (centre >= n_out) return;
+  const int64_t slot_centre = wave_slot();
+  if (slot_centre >= n_out) return;
+  const int64_t centre = centre_of(slot_centre, order);
   const int quarter = lane >> 4, col = lane & 15;
   const int a = centre > 0 ? ranges[centre - 1] : 0, b = ranges[centre];
   if (b <= a) return;
@@ -468,11 +490,14 @@ static int generic_chunks(int C, int K) {
 
 using namespace mccnn;
 
-extern "C" int mccnn_basis_proj(mccnn_stream_t stream, int64_t basis_rows, int num_basis,
-                                const float *basis, int64_t num_pts, int num_features,
-                                const float *features, int64_t num_neighbors, int neighbors_rank,
-                                int neighbors_cols, const int32_t *neighbors,
-                                int64_t num_samples, const int32_t *ranges, float *out) {
+extern "C" int mccnn_basis_proj_ordered(mccnn_stream_t stream, int64_t basis_rows, int num_basis,
+                                        const float *basis, int64_t num_pts, int num_features,
+                                        const float *features, int64_t num_neighbors,
+                                        int neighbors_rank, int neighbors_cols,
+                                        const int32_t *neighbors, int64_t num_samples,
+                                        const int32_t *ranges, const int32_t *centre_order,
+                                        float *out) {
+  const int32_t *order = centre_order;
   int rc = check_basis_args("BasisProj", basis_rows, num_basis, num_features, num_neighbors,
                             neighbors_rank, neighbors_cols);
   if (rc != MCCNN_OK) return rc;
@@ -489,14 +514,14 @@ extern "C" int mccnn_basis_proj(mccnn_stream_t stream, int64_t basis_rows, int n
     const int chunks = num_features / (lanes_per_pair * cpl);
     const int64_t waves = num_samples * chunks;
     MCCNN_REQUIRE(waves < ((int64_t)1 << 31), "BasisProj launch too large");
-    const dim3 grid(blocks_for(waves, 256 / kWave)), block(256);
+    const dim3 grid(wave_grid(waves)), block(256);
     const int2 *nb = (const int2 *)neighbors;
 #define MCCNN_FWD32(K_, CPL_)                                                                  \
   hipLaunchKernelGGL((basis_proj_mfma32_kernel<K_, CPL_>), grid, block, 0, s, num_samples,     \
-                     num_features, chunks, basis, features, nb, ranges, out)
+                     num_features, chunks, basis, features, nb, ranges, order, out)
 #define MCCNN_FWD16(CPL_)                                                                      \
   hipLaunchKernelGGL((basis_proj_mfma16_kernel<CPL_>), grid, block, 0, s, num_samples,         \
-                     num_features, chunks, basis, features, nb, ranges, out)
+                     num_features, chunks, basis, features, nb, ranges, order, out)
     if (num_basis == 16) {
       switch (cpl) {
         case 8: MCCNN_FWD16(8); break;
@@ -525,24 +550,24 @@ extern "C" int mccnn_basis_proj(mccnn_stream_t stream, int64_t basis_rows, int n
   const int chunks = generic_chunks(num_features, num_basis);
   const int64_t waves = num_samples * chunks;
   MCCNN_REQUIRE(waves < ((int64_t)1 << 31), "BasisProj launch too large");
-  const unsigned grid = blocks_for(waves, 256 / kWave);
+  const unsigned grid = wave_grid(waves);
   MCCNN_BASIS_SWITCH(num_basis,
                      hipLaunchKernelGGL(basis_proj_generic_kernel<K>, dim3(grid), dim3(256), 0,
                                         s, num_samples, num_features, chunks,
-                                        basis, features, (const int2 *)neighbors, ranges, out));
+                                        basis, features, (const int2 *)neighbors, ranges, order,
+                                        out));
   MCCNN_LAUNCH_CHECK();
   return MCCNN_OK;
 }
 
-extern "C" int mccnn_basis_proj_grads(mccnn_stream_t stream, int64_t basis_rows, int num_basis,
-                                      const float *basis, int64_t num_pts, int num_features,
-                                      const float *features, int64_t num_neighbors,
-                                      int neighbors_rank, int neighbors_cols,
-                                      const int32_t *neighbors, int64_t num_samples,
-                                      const int32_t *ranges, int in_grads_rank,
-                                      int64_t in_grads_dim0, int64_t in_grads_dim1,
-                                      int64_t in_grads_dim2, const float *in_grads,
-                                      float *basis_grads_out, float *feature_grads_out) {
+extern "C" int mccnn_basis_proj_grads_ordered(
+    mccnn_stream_t stream, int64_t basis_rows, int num_basis, const float *basis, int64_t num_pts,
+    int num_features, const float *features, int64_t num_neighbors, int neighbors_rank,
+    int neighbors_cols, const int32_t *neighbors, int64_t num_samples, const int32_t *ranges,
+    const int32_t *centre_order, int in_grads_rank, int64_t in_grads_dim0, int64_t in_grads_dim1,
+    int64_t in_grads_dim2, const float *in_grads, float *basis_grads_out,
+    float *feature_grads_out) {
+  const int32_t *order = centre_order;
   int rc = check_basis_args("BasisProjGrads", basis_rows, num_basis, num_features, num_neighbors,
                             neighbors_rank, neighbors_cols);
   if (rc != MCCNN_OK) return rc;
@@ -564,10 +589,10 @@ extern "C" int mccnn_basis_proj_grads(mccnn_stream_t stream, int64_t basis_rows,
   const int2 *nb = (const int2 *)neighbors;
   if (mfma_grads_supported(num_features, num_basis)) {
     MCCNN_REQUIRE(num_samples < ((int64_t)1 << 31), "BasisProjGrads launch too large");
-    const dim3 grid(blocks_for(num_samples, 256 / kWave)), block(256);
+    const dim3 grid(wave_grid(num_samples)), block(256);
 #define MCCNN_BWD(KERNEL_, C_)                                                              \
   hipLaunchKernelGGL((KERNEL_<C_>), grid, block, 0, s, num_samples, basis, features, nb,   \
-                     ranges, in_grads, basis_grads_out, feature_grads_out)
+                     ranges, order, in_grads, basis_grads_out, feature_grads_out)
     if (num_basis == 32) {
       switch (num_features) {
         case 32: MCCNN_BWD(basis_proj_grads_mfma32_kernel, 32); break;
@@ -593,11 +618,38 @@ extern "C" int mccnn_basis_proj_grads(mccnn_stream_t stream, int64_t basis_rows,
   }
   const int64_t waves = num_samples * chunks;
   MCCNN_REQUIRE(waves < ((int64_t)1 << 31), "BasisProjGrads launch too large");
-  const unsigned grid = blocks_for(waves, 256 / kWave);
+  const unsigned grid = wave_grid(waves);
   MCCNN_BASIS_SWITCH(num_basis, hipLaunchKernelGGL(basis_proj_grads_generic_kernel<K>, dim3(grid),
                                                    dim3(256), 0, s, num_samples, num_features,
-                                                   chunks, basis, features, nb, ranges, in_grads,
+                                                   chunks, basis, features, nb, ranges, order,
+                                                   in_grads,
                                                    basis_grads_out, feature_grads_out));
   MCCNN_LAUNCH_CHECK();
   return MCCNN_OK;
+}
+
+extern "C" int mccnn_basis_proj(mccnn_stream_t stream, int64_t basis_rows, int num_basis,
+                                const float *basis, int64_t num_pts, int num_features,
+                                const float *features, int64_t num_neighbors, int neighbors_rank,
+                                int neighbors_cols, const int32_t *neighbors,
+                                int64_t num_samples, const int32_t *ranges, float *out) {
+  return mccnn_basis_proj_ordered(stream, basis_rows, num_basis, basis, num_pts, num_features,
+                                  features, num_neighbors, neighbors_rank, neighbors_cols,
+                                  neighbors, num_samples, ranges, nullptr, out);
+}
+
+extern "C" int mccnn_basis_proj_grads(mccnn_stream_t stream, int64_t basis_rows, int num_basis,
+                                      const float *basis, int64_t num_pts, int num_features,
+                                      const float *features, int64_t num_neighbors,
+                                      int neighbors_rank, int neighbors_cols,
+                                      const int32_t *neighbors, int64_t num_samples,
+                                      const int32_t *ranges, int in_grads_rank,
+                                      int64_t in_grads_dim0, int64_t in_grads_dim1,
+                                      int64_t in_grads_dim2, const float *in_grads,
+                                      float *basis_grads_out, float *feature_grads_out) {
+  return mccnn_basis_proj_grads_ordered(stream, basis_rows, num_basis, basis, num_pts,
+                                        num_features, features, num_neighbors, neighbors_rank,
+                                        neighbors_cols, neighbors, num_samples, ranges, nullptr,
+                                        in_grads_rank, in_grads_dim0, in_grads_dim1, in_grads_dim2,
+                                        in_grads, basis_grads_out, feature_grads_out);
 }

@@ -104,7 +104,8 @@ class MCConv(torch.nn.Module):
                                self._act)
         proj = tfg_custom_ops.basis_proj(basis, features.contiguous(),
                                          neighborhood._original_neigh_ids,
-                                         neighborhood._samples_neigh_ranges)
+                                         neighborhood._samples_neigh_ranges,
+                                         neighborhood._centre_order)
         n, c, l, h = proj.shape[0], self._num_features_in, self._num_mlps, self._hidden
         if l == 1:
             return proj.reshape(n, c * h) @ self.final_weights[0]
@@ -160,7 +161,8 @@ class KPConv(torch.nn.Module):
             ptr(ids, _I32), ptr(torch.reciprocal(radii), _F32), ptr(self._kernel_points, _F32),
             ptr(None), ptr(basis), ptr(None))
         proj = tfg_custom_ops.basis_proj(basis, features.contiguous(), ids,
-                                         neighborhood._samples_neigh_ranges)
+                                         neighborhood._samples_neigh_ranges,
+                                         neighborhood._centre_order)
         c = self._num_features_in
         if k == kp:
             return proj.reshape(-1, c * k) @ self.weights

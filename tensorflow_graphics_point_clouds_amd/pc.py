@@ -46,6 +46,17 @@ class PointCloud:
         self._dimension = self._points.shape[1]
 
 
+def _sort_keys(keys, key_bits):
+    """Stable descending sort -> (sorted keys, int32 permutation)."""
+    n, dev = keys.shape[0], keys.device
+    sorted_keys = torch.empty(n, dtype=_I64, device=dev)
+    sorted_indices = torch.empty(n, dtype=_I32, device=dev)
+    ws = _lib.workspace(_lib.lib().mccnn_sort_keys_workspace_bytes(i64(n)), dev)
+    _lib.call("sort_keys_descending", stream(), i64(n), cint(key_bits), ptr(keys, _I64),
+              ptr(sorted_keys), ptr(sorted_indices), ptr(ws), _lib.csize(ws.numel()))
+    return sorted_keys, sorted_indices
+
+
 class Grid:
     """Regular grid over a point cloud (pylib/pc/Grid.py:32-84): grid shape from
     the per-cloud bounding boxes, cell keys, stable descending sort, gathers."""
@@ -73,12 +84,8 @@ class Grid:
         total = b
         for v in self._num_cells_host:
             total *= v
-        key_bits = max(1, (total - 1).bit_length())
-        self._sorted_keys = torch.empty(n, dtype=_I64, device=dev)
-        self._sorted_indices = torch.empty(n, dtype=_I32, device=dev)
-        ws = _lib.workspace(L.mccnn_sort_keys_workspace_bytes(i64(n)), dev)
-        _lib.call("sort_keys_descending", stream(), i64(n), cint(key_bits), ptr(self._cur_keys), ptr(self._sorted_keys),
-            ptr(self._sorted_indices), ptr(ws), _lib.csize(ws.numel()))
+        self._key_bits = max(1, (total - 1).bit_length())
+        self._sorted_keys, self._sorted_indices = _sort_keys(self._cur_keys, self._key_bits)
         self._sorted_points = torch.empty_like(pc._points)
         self._sorted_batch_ids = torch.empty_like(pc._batch_ids)
         _lib.call("gather_points", stream(), i64(n), cint(d), ptr(pc._points), ptr(pc._batch_ids),
@@ -121,6 +128,18 @@ class Neighborhood:
             ptr(grid._sorted_indices, _I32), ptr(self._original_neigh_ids))
         self._pdf = None
         self._pdf_per_point = None
+        # optional visiting order of the centres for the projection kernels
+        self._centre_order = None
+
+    def compute_centre_order(self):
+        """Rank the centres by their cell key in the grid (a scheduling hint for
+        `basis_proj`; the grid's own sorted points already are in that order)."""
+        s, grid = self._point_cloud_sampled, self._grid
+        if not self._equal_samples and s._points.shape[0] > 0:
+            keys = tfg_custom_ops.compute_keys(s._points, s._batch_ids, grid._scaled_aabb_min,
+                                               grid._num_cells, grid._inv_cell_sizes)
+            self._centre_order = _sort_keys(keys, grid._key_bits)[1]
+        return self._centre_order
 
     def compute_pdf(self, bandwidth=0.2, mode=KDEMode.constant, normalize=False):
         d = self._grid._point_cloud._dimension

@@ -156,46 +156,57 @@ def compute_pdf_with_pt_grads(points, neighbors, sample_neigh_indices, inv_bandw
                              inv_radii, mode)
 
 
-def _basis_proj_raw(basis, features, neighbors, ranges):
+def _basis_proj_raw(basis, features, neighbors, ranges, centre_order=None):
     out = torch.empty((ranges.shape[0], _dim(features, 1), _dim(basis, 1)), dtype=_F32,
                       device=features.device)
-    _lib.call("basis_proj", stream(), i64(basis.shape[0]), cint(_dim(basis, 1)), ptr(basis, _F32),
-        i64(features.shape[0]), cint(_dim(features, 1)), ptr(features, _F32),
-        i64(neighbors.shape[0]), cint(neighbors.dim()), cint(_dim(neighbors, 1)),
-        ptr(neighbors, _I32), i64(ranges.shape[0]), ptr(ranges, _I32), ptr(out))
+    _lib.call("basis_proj_ordered", stream(), i64(basis.shape[0]), cint(_dim(basis, 1)),
+              ptr(basis, _F32), i64(features.shape[0]), cint(_dim(features, 1)),
+              ptr(features, _F32), i64(neighbors.shape[0]), cint(neighbors.dim()),
+              cint(_dim(neighbors, 1)), ptr(neighbors, _I32), i64(ranges.shape[0]),
+              ptr(ranges, _I32), ptr(centre_order, _I32 if centre_order is not None else None),
+              ptr(out))
     return out
 
 
 def basis_proj_grads(basis_neighbors, pt_features, neighbors, sample_neigh_indices,
-                     in_gradients):
+                     in_gradients, centre_order=None):
     """BasisProjGrads (basis_proj_ops.cpp:40-53) -> (basis_gradients [M, K],
     feat_gradients [N_in, C])."""
     dbasis = torch.empty_like(basis_neighbors)
     dfeat = torch.empty_like(pt_features)
     g = in_gradients
-    _lib.call("basis_proj_grads", stream(), i64(basis_neighbors.shape[0]), cint(_dim(basis_neighbors, 1)),
-        ptr(basis_neighbors, _F32), i64(pt_features.shape[0]), cint(_dim(pt_features, 1)),
-        ptr(pt_features, _F32), i64(neighbors.shape[0]), cint(neighbors.dim()),
-        cint(_dim(neighbors, 1)), ptr(neighbors, _I32), i64(sample_neigh_indices.shape[0]),
-        ptr(sample_neigh_indices, _I32), cint(g.dim()), i64(_dim(g, 0)), i64(_dim(g, 1)),
-        i64(_dim(g, 2)), ptr(g, _F32), ptr(dbasis), ptr(dfeat))
+    _lib.call("basis_proj_grads_ordered", stream(), i64(basis_neighbors.shape[0]),
+              cint(_dim(basis_neighbors, 1)), ptr(basis_neighbors, _F32),
+              i64(pt_features.shape[0]), cint(_dim(pt_features, 1)), ptr(pt_features, _F32),
+              i64(neighbors.shape[0]), cint(neighbors.dim()), cint(_dim(neighbors, 1)),
+              ptr(neighbors, _I32), i64(sample_neigh_indices.shape[0]),
+              ptr(sample_neigh_indices, _I32),
+              ptr(centre_order, _I32 if centre_order is not None else None), cint(g.dim()),
+              i64(_dim(g, 0)), i64(_dim(g, 1)), i64(_dim(g, 2)), ptr(g, _F32), ptr(dbasis),
+              ptr(dfeat))
     return dbasis, dfeat
 
 
 class _BasisProj(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, basis, features, neighbors, ranges):
+    def forward(ctx, basis, features, neighbors, ranges, centre_order):
         ctx.save_for_backward(basis, features, neighbors, ranges)
-        return _basis_proj_raw(basis, features, neighbors, ranges)
+        ctx.centre_order = centre_order
+        return _basis_proj_raw(basis, features, neighbors, ranges, centre_order)
 
     @staticmethod
     def backward(ctx, grad):
         basis, features, neighbors, ranges = ctx.saved_tensors
-        dbasis, dfeat = basis_proj_grads(basis, features, neighbors, ranges, grad.contiguous())
-        return dbasis, dfeat, None, None
+        dbasis, dfeat = basis_proj_grads(basis, features, neighbors, ranges, grad.contiguous(),
+                                         ctx.centre_order)
+        return dbasis, dfeat, None, None, None
 
 
-def basis_proj(basis_neighbors, pt_features, neighbors, sample_neigh_indices):
+def basis_proj(basis_neighbors, pt_features, neighbors, sample_neigh_indices,
+               centre_order=None):
     """BasisProj (basis_proj_ops.cpp:25-38): [N_out, C, K] sum over the pairs of
-    each centre of feature (outer) basis; differentiable in basis and features."""
-    return _BasisProj.apply(basis_neighbors, pt_features, neighbors, sample_neigh_indices)
+    each centre of feature (outer) basis; differentiable in basis and features.
+    `centre_order` (optional int32 permutation of the centres, e.g. their order by
+    grid cell) only changes the order in which centres are processed."""
+    return _BasisProj.apply(basis_neighbors, pt_features, neighbors, sample_neigh_indices,
+                            centre_order)

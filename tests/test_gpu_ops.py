@@ -309,3 +309,88 @@ def test_point_hierarchy_matches_oracle(ops, oracle):
                                        g.num_cells, nbh.neighbors, nbh.ranges, 1)
         assert np.array_equal(hier._point_clouds[level + 1]._points.cpu().numpy(), pts)
         assert np.array_equal(hier._point_clouds[level + 1]._batch_ids.cpu().numpy(), bids)
+
+
+def test_basis_proj_visiting_order_does_not_change_results(ops, oracle):
+    """The *_ordered entry points only reschedule: forward and basis gradients
+    are bit-identical for any permutation of the centres, feature gradients (float
+    atomics) agree normwise."""
+    rng = np.random.default_rng(123)
+    n, c, k = 4000, 64, 16
+    pts, bids = _cloud(rng, 2, n, 3)
+    g = oracle.Grid(pts, bids, 2, 0.1)
+    nbh = oracle.Neighborhood(g, 0.1, pts, bids)
+    ids = nbh.original_neigh_ids
+    basis = rng.random((len(ids), k)).astype(np.float32)
+    feat = rng.standard_normal((n, c)).astype(np.float32)
+    up = rng.standard_normal((n, c, k)).astype(np.float32)
+    order = dev(rng.permutation(n).astype(np.int32))
+    args = (dev(basis), dev(feat), dev(ids), dev(nbh.ranges))
+    a = ops._basis_proj_raw(*args)
+    b = ops._basis_proj_raw(*args, order)
+    assert torch.equal(a, b)
+    da, fa = ops.basis_proj_grads(*args, dev(up))
+    db, fb = ops.basis_proj_grads(*args, dev(up), order)
+    assert torch.equal(da, db)
+    assert_normwise(fb.cpu().numpy(), fa.cpu().numpy())
+
+
+def test_full_size_invariants(ops):
+    """Scene-scale batch at its real size (8 clouds, ~760k points): properties
+    that need no oracle.  Sortedness and permutation of the grid sort, the column
+    table against the keys, ranges non-decreasing with last == M, pairs grouped by
+    centre and ascending inside a centre, every point its own neighbour, the
+    neighbourhood symmetric, and linearity / adjointness of basis_proj."""
+    from tensorflow_graphics_point_clouds_amd import pc, synthetic
+    cfg = synthetic.config3()
+    cloud = pc.PointCloud(dev(cfg["points"]), dev(cfg["batch_ids"]), cfg["batch_size"])
+    grid = pc.Grid(cloud, cfg["radius"])
+    n = cloud._points.shape[0]
+    keys = grid._sorted_keys
+    assert bool((keys[1:] <= keys[:-1]).all())
+    assert torch.equal(torch.sort(grid._sorted_indices.long()).values,
+                       torch.arange(n, device="cuda"))
+    assert torch.equal(grid._cur_keys[grid._sorted_indices.long()], keys)
+    ties = keys[1:] == keys[:-1]
+    assert bool((grid._sorted_indices[1:][ties] > grid._sorted_indices[:-1][ties]).all())
+    nc = grid._num_cells_host
+    ds = grid.get_DS().reshape(-1, 2).long()
+    col = torch.div(keys, nc[2], rounding_mode="floor")
+    occupied = torch.unique(col)
+    counts = torch.bincount(col, minlength=ds.shape[0])
+    assert torch.equal((ds[:, 1] - ds[:, 0]), counts)
+    assert bool((col[ds[occupied, 0]] == occupied).all())
+
+    nbh = pc.Neighborhood(grid, cfg["radius"])          # centres = sorted points
+    ranges, nbrs = nbh._samples_neigh_ranges.long(), nbh._neighbors.long()
+    m = nbrs.shape[0]
+    assert int(ranges[-1]) == m and bool((ranges[1:] >= ranges[:-1]).all())
+    starts = torch.cat([ranges.new_zeros(1), ranges[:-1]])
+    centre_of_pair = torch.repeat_interleave(torch.arange(n, device="cuda"), ranges - starts)
+    assert torch.equal(nbrs[:, 1], centre_of_pair)
+    same = nbrs[1:, 1] == nbrs[:-1, 1]
+    assert bool((nbrs[1:, 0][same] > nbrs[:-1, 0][same]).all())
+    assert int((nbrs[:, 0] == nbrs[:, 1]).sum()) == n                     # self pairs
+    assert bool((grid._sorted_batch_ids[nbrs[:, 0]] == grid._sorted_batch_ids[nbrs[:, 1]]).all())
+    fwd = nbrs[:, 0] * n + nbrs[:, 1]
+    bwd = nbrs[:, 1] * n + nbrs[:, 0]
+    assert torch.equal(torch.sort(fwd).values, torch.sort(bwd).values)    # symmetry
+    d = (grid._sorted_points[nbrs[:, 0]] - grid._sorted_points[nbrs[:, 1]]).norm(dim=1)
+    assert float(d.max()) < cfg["radius"] * (1 + 1e-6)
+
+    # basis_proj: linear in the features, and <up, proj(B, F)> == <dB, B> == <dF, F>
+    gen = torch.Generator(device="cuda").manual_seed(0)
+    ids = nbh._original_neigh_ids
+    basis = torch.rand((m, 16), device="cuda", generator=gen)
+    f1 = torch.randn((n, 64), device="cuda", generator=gen)
+    f2 = torch.randn((n, 64), device="cuda", generator=gen)
+    r32 = nbh._samples_neigh_ranges
+    p1 = ops._basis_proj_raw(basis, f1, ids, r32)
+    p2 = ops._basis_proj_raw(basis, f2, ids, r32)
+    p12 = ops._basis_proj_raw(basis, f1 + 2 * f2, ids, r32)
+    assert float((p12 - (p1 + 2 * p2)).abs().max()) <= 1e-5 * float(p12.abs().max())
+    up = torch.randn(p1.shape, device="cuda", generator=gen)
+    db, df = ops.basis_proj_grads(basis, f1, ids, r32, up)
+    lhs = float((up.double() * p1.double()).sum())
+    assert abs(float((db.double() * basis.double()).sum()) - lhs) <= 1e-5 * abs(lhs) + 1e-3
+    assert abs(float((df.double() * f1.double()).sum()) - lhs) <= 1e-5 * abs(lhs) + 1e-3
