@@ -43,6 +43,21 @@ def op_bytes(name, M, N_in, N_out, C, K, D):
     return None
 
 
+def measured_traffic(op, workload):
+    """HBM-side bytes per launch from the committed counter summary (scaled
+    FETCH_SIZE + WRITE_SIZE), or None when the summary has no line for it."""
+    path = os.path.join(ROOT, "profiles", "basis_proj_hbm_traffic.txt")
+    try:
+        for line in open(path):
+            parts = line.split()
+            if len(parts) == 4 and parts[0] == "traffic_bytes" and parts[1] == op \
+                    and parts[2] == workload:
+                return int(parts[3])
+    except OSError:
+        pass
+    return None
+
+
 def build_scene(torch, pc, synthetic, scale):
     import numpy as np
     cfg = synthetic.config3(scale=scale)
@@ -168,6 +183,9 @@ def main():
     ap.add_argument("--scale", type=float, default=1.0, help="shrink the point counts (tests)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the host-CPU baseline")
     ap.add_argument("--no-isolated", action="store_true", help="skip the isolated basis_proj case")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="only run a 1 GiB device copy three times (reference point for the "
+                         "FETCH_SIZE / WRITE_SIZE counters) and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         log("bench.py measures one GPU: this build has no multi-GPU path (clouds would be "
@@ -176,8 +194,17 @@ def main():
 
     import numpy as np
     import torch
-    from tensorflow_graphics_point_clouds_amd import _lib, layers, pc, synthetic, tfg_custom_ops
     assert torch.cuda.is_available(), "bench.py needs a GPU"
+    if args.calibrate_copy:
+        src = torch.ones(1 << 28, dtype=torch.float32, device="cuda")      # 1 GiB
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"calibration": "3 device copies of 1 GiB (2^30 bytes read, 2^30 written "
+                                         "each)"}))
+        return
+    from tensorflow_graphics_point_clouds_amd import _lib, layers, pc, synthetic, tfg_custom_ops
     _lib.lib()
     torch.backends.cuda.matmul.allow_tf32 = False
 
@@ -229,7 +256,9 @@ def main():
     dominant = max((n for n in ops if "GBps" in ops[n]), key=lambda n: ops[n]["ms"])
     roof = {"kernel": dominant, "bound": "hbm", "achieved": ops[dominant]["GBps"],
             "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": ops[dominant]["frac_hbm_peak"],
-            "traffic": None, "ms": ops[dominant]["ms"]}
+            "traffic": measured_traffic(dominant, "config3_C%d_K%d" % (C, K))
+            if args.scale == 1.0 else None,
+            "ms": ops[dominant]["ms"]}
 
     result = {
         "metric": "MCConv layer fwd+bwd points/sec", "value": N / (ms_per_step * 1e-3),
