@@ -40,6 +40,10 @@ def op_bytes(name, M, N_in, N_out, C, K, D):
         return M * (8 + 2 * 4 * D + 4) + 4 * M * K
     if name == "mc_basis_grads":
         return M * (8 + 2 * 4 * D + 4) + 4 * M * K
+    if name == "mc_conv_project":        # basis evaluated in registers: no [M, K] traffic
+        return M * (8 + 4 * D + 4) + 4 * (M * C + N_out * C * K) + 4 * N_out * (1 + D)
+    if name == "mc_conv_project_grads":
+        return M * (8 + 4 * D + 4) + 4 * (M * C + N_out * C * K + N_in * C) + 4 * N_out * (1 + D)
     return None
 
 
@@ -138,6 +142,67 @@ def cpu_baseline(synthetic, sample_points=60000):
     return {"value": n / dt, "unit": "points/s", "cores": cores, "kind": "port",
             "sample": "one config-3 cloud cut to %d points (%d pairs), %d fwd+bwd passes of "
                       "the C/OpenMP oracle with numpy GEMMs" % (n, len(ids), reps)}
+
+
+def per_op_times(torch, pc, layers, synthetic, _lib, radius=0.04, reps=5):
+    """Every op of the path on the dense case (4 x 200k uniform points, radius
+    0.04): average milliseconds from HIP events around each C-ABI call, with
+    algorithmic GB/s where a byte count is defined.  Dynamic-size ops include
+    their one host synchronisation."""
+    import numpy as np
+    cfg = synthetic.config4()
+    dev = lambda a: torch.as_tensor(np.ascontiguousarray(a)).cuda()
+    cloud = pc.PointCloud(dev(cfg["points"]), dev(cfg["batch_ids"]), cfg["batch_size"])
+    N, D, B = cloud._points.shape[0], 3, cfg["batch_size"]
+    feats = torch.randn((N, 64), device="cuda")
+
+    def run():
+        grid = pc.Grid(cloud, radius)
+        grid.get_DS()
+        nbh = pc.Neighborhood(grid, radius)                    # self neighbourhood
+        nbh.compute_pdf(bandwidth=0.2)
+        g = torch.ones(N, device="cuda")
+        pts = grid._sorted_points
+        from tensorflow_graphics_point_clouds_amd import tfg_custom_ops as tfg
+        tfg.compute_pdf_pt_grads(pts, nbh._neighbors, nbh._samples_neigh_ranges,
+                                 torch.full((3,), 5.0, device="cuda"), nbh._inv_radii, g, 0)
+        pc.sample(nbh, "poisson")
+        pc.sample(nbh, "average")
+        layers.MaxPooling()(feats, cloud, None, radius, neighborhood=nbh)
+        layers.AveragePooling()(feats, cloud, None, radius, neighborhood=nbh)
+        layers.GlobalMaxPooling()(feats, cloud)
+        return grid, nbh
+
+    run()
+    torch.cuda.synchronize()
+    _lib.start_timing()
+    for _ in range(reps):
+        grid, nbh = run()
+    t = _lib.collect_timing()
+    M = nbh._neighbors.shape[0]
+    ncol = B * grid._num_cells_host[0] * grid._num_cells_host[1]
+    passes = (grid._key_bits + 7) // 8
+    by = {
+        "compute_keys": N * (4 * D + 4 + 8),
+        "sort_keys_descending": passes * 2 * 12 * N,
+        "gather_points": 2 * N * (4 * D + 4) + 4 * N,
+        "build_grid_ds": 8 * N + 8 * ncol,
+        "find_neighbors_count": N * (4 * D + 4) + N * (4 * D + 8) + 8 * ncol + 4 * N,
+        "find_neighbors_fill": N * (4 * D) + N * (4 * D) + 8 * M,
+        "compute_pdf": N * 4 * D + 8 * M + 4 * N + M * 4 * D + 4 * N,
+        "compute_pdf_pt_grads": N * 4 * D + 8 * M + 8 * N + M * 4 * D + 2 * N * 4 * D,
+        "local_pool": 4 * M * 64 + 8 * M + 4 * N * 64,
+    }
+    out = {"workload": "4x200k uniform, r=%.2f, self neighbourhood, %d pairs; pooling C=64"
+                       % (radius, M)}
+    for name, vals in sorted(t.items()):
+        ms = sum(vals) / reps
+        entry = {"ms": round(ms, 4), "calls_per_pass": len(vals) // reps}
+        if name in by:
+            entry["GBps"] = round(by[name] * (len(vals) // reps) / ms / 1e6, 1)
+            entry["frac_hbm_peak"] = round(entry["GBps"] / HBM_PEAK_GBS, 4)
+        out[name] = entry
+    return out
 
 
 def isolated_basis_proj(torch, pc, synthetic, tfg, _lib, radius=0.04, steps=5):
@@ -277,6 +342,8 @@ def main():
         torch.cuda.empty_cache()
         result["basis_proj_isolated"] = isolated_basis_proj(torch, pc, synthetic, tfg_custom_ops,
                                                             _lib)
+        torch.cuda.empty_cache()
+        result["per_op_dense_case"] = per_op_times(torch, pc, layers, synthetic, _lib)
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(synthetic)
     else:

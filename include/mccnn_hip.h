@@ -331,6 +331,35 @@ int mccnn_mc_basis_grads(mccnn_stream_t stream, int64_t num_neighbors,
                          size_t workspace_bytes, float *weight_grads_out,
                          float *bias_grads_out);
 
+/* Fused Monte-Carlo convolution projection: mccnn_mc_basis followed by
+ * mccnn_basis_proj (MCConv.py:163-177) in one kernel that evaluates the basis in
+ * registers, and the matching backward (gradients of features, kernel weights
+ * and biases from the upstream [N_out, C, K] gradient).  Same results as the
+ * separate entry points up to fp32 summation order; the [M, K] basis and its
+ * gradient are never written.  mccnn_mc_conv_supported() tells whether a shape
+ * is covered (D in {2,3}, K = 16, C in {16,32,64,128}); other shapes return
+ * MCCNN_INVALID_ARGUMENT and must use the separate entry points.  No
+ * counterpart among the reference's ops, which materialise the basis in
+ * TensorFlow. */
+int mccnn_mc_conv_supported(int num_dims, int num_features, int num_basis);
+int mccnn_mc_conv_project(mccnn_stream_t stream, int num_dims, int64_t num_pts,
+                          const float *points_in, int num_features,
+                          const float *features, int64_t num_samples,
+                          const float *points_out, int64_t num_neighbors,
+                          const int32_t *neighbors, const int32_t *ranges,
+                          const float *inv_radii, int num_basis, int num_mlps,
+                          int activation, const float *weights,
+                          const float *biases, const float *pdf, float *out);
+size_t mccnn_mc_conv_project_grads_workspace_bytes(int num_dims, int num_basis);
+int mccnn_mc_conv_project_grads(
+    mccnn_stream_t stream, int num_dims, int64_t num_pts, const float *points_in,
+    int num_features, const float *features, int64_t num_samples,
+    const float *points_out, int64_t num_neighbors, const int32_t *neighbors,
+    const int32_t *ranges, const float *inv_radii, int num_basis, int num_mlps,
+    int activation, const float *weights, const float *biases, const float *pdf,
+    const float *in_grads, void *workspace, size_t workspace_bytes,
+    float *feature_grads_out, float *weight_grads_out, float *bias_grads_out);
+
 /* Per-pair kernel-point weights, pylib/pc/layers/KPConv.py:29-57,193-213:
  *   d[m,k] = || delta_m - (kernel_points[k] + offsets[ctr_m,k]) ||
  *   kind 0: max(1 - d/sigma, 0);  kind 1: exp(-(d/(sigma/3))^2)

@@ -15,32 +15,11 @@
 // k = l % K is fixed and its channel advances by 64/K per j.
 #include "common.h"
 #include "fill.h"
+#include "mfma.h"
 
 namespace mccnn {
 
 constexpr int kAcc = 16;   // accumulators per lane in the generic kernels
-
-// Wave slot -> centre.  `order` (optional) is a permutation of the centres that
-// fixes the visiting order; it is a scheduling hint only.  (Dealing contiguous
-// slot ranges to the 8 XCDs and visiting the centres in cell order were both
-// measured and left out: the feature rows already hit the memory-side cache,
-// and concentrating the feature-gradient atomics of neighbouring centres in
-// time made them slower.)
-constexpr int kWavesPerBlock = 256 / kWave;
-
-__device__ __forceinline__ int64_t wave_slot() {
-  return __builtin_amdgcn_readfirstlane(
-      (int)(blockIdx.x * kWavesPerBlock + threadIdx.x / kWave));
-}
-
-__device__ __forceinline__ int64_t centre_of(int64_t slot_centre, const int *__restrict__ order) {
-  return order ? (int64_t)__builtin_amdgcn_readfirstlane(order[slot_centre]) : slot_centre;
-}
-
-static unsigned wave_grid(int64_t waves) {
-  const int64_t blocks = (waves + kWavesPerBlock - 1) / kWavesPerBlock;
-  return (unsigned)(blocks < 1 ? 1 : blocks);
-}
 
 template <int K>
 __global__ void __launch_bounds__(256) basis_proj_generic_kernel(
@@ -142,37 +121,6 @@ __global__ void __launch_bounds__(256) basis_proj_grads_generic_kernel(
 // channels {lane_channel_base + j}.  Neighbour ids are read 64 at a time,
 // coalesced, and broadcast with a lane shuffle.  Results leave with
 // non-temporal stores (write-once stream).
-
-typedef float v16f __attribute__((ext_vector_type(16)));
-typedef float v4f __attribute__((ext_vector_type(4)));
-
-template <int N>
-struct FVec {
-  float v[N];
-};
-
-template <int N>
-__device__ __forceinline__ FVec<N> load_vec(const float *__restrict__ p, bool valid) {
-  FVec<N> r;
-#pragma unroll
-  for (int i = 0; i < N; ++i) r.v[i] = 0.0f;
-  if (valid) {
-    if constexpr (N % 4 == 0) {
-#pragma unroll
-      for (int i = 0; i < N / 4; ++i) {
-        const float4 t = reinterpret_cast<const float4 *>(p)[i];
-        r.v[4 * i] = t.x; r.v[4 * i + 1] = t.y; r.v[4 * i + 2] = t.z; r.v[4 * i + 3] = t.w;
-      }
-    } else if constexpr (N == 2) {
-      const float2 t = *reinterpret_cast<const float2 *>(p);
-      r.v[0] = t.x; r.v[1] = t.y;
-    } else {
-#pragma unroll
-      for (int i = 0; i < N; ++i) r.v[i] = p[i];
-    }
-  }
-  return r;
-}
 
 constexpr int kUnroll = 4;   // MFMA steps whose loads are issued together
 

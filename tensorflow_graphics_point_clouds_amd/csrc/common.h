@@ -128,6 +128,20 @@ __device__ __forceinline__ float wave_sum(float v) {
   return v;
 }
 
+// Activations of the kernel MLP (pylib/pc/layers/MCConv.py:27-31; leaky slope
+// 0.2 and ELU alpha 1 are the TensorFlow defaults the reference relies on).
+__device__ __forceinline__ float act_fwd(int act, float z) {
+  if (act == MCCNN_ACT_RELU) return z > 0.0f ? z : 0.0f;
+  if (act == MCCNN_ACT_LEAKY_RELU) return z > 0.0f ? z : 0.2f * z;
+  return z > 0.0f ? z : expm1f(z);
+}
+
+__device__ __forceinline__ float act_bwd(int act, float z) {
+  if (act == MCCNN_ACT_RELU) return z > 0.0f ? 1.0f : 0.0f;
+  if (act == MCCNN_ACT_LEAKY_RELU) return z > 0.0f ? 1.0f : 0.2f;
+  return z > 0.0f ? 1.0f : expf(z);
+}
+
 #endif  // __HIPCC__
 
 }  // namespace mccnn

@@ -9,18 +9,6 @@
 
 namespace mccnn {
 
-__device__ __forceinline__ float act_fwd(int act, float z) {
-  if (act == MCCNN_ACT_RELU) return z > 0.0f ? z : 0.0f;
-  if (act == MCCNN_ACT_LEAKY_RELU) return z > 0.0f ? z : 0.2f * z;
-  return z > 0.0f ? z : expm1f(z);
-}
-
-__device__ __forceinline__ float act_bwd(int act, float z) {
-  if (act == MCCNN_ACT_RELU) return z > 0.0f ? 1.0f : 0.0f;
-  if (act == MCCNN_ACT_LEAKY_RELU) return z > 0.0f ? 1.0f : 0.2f;
-  return z > 0.0f ? 1.0f : expf(z);
-}
-
 // delta = (p_in[nbr] - p_out[ctr]) * inv_radii
 template <int D>
 __device__ __forceinline__ void pair_delta(const float *__restrict__ pin,

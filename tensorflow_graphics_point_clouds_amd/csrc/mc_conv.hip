@@ -1,0 +1,384 @@
+// Fused Monte-Carlo convolution projection (pylib/pc/layers/MCConv.py:137-177,
+// 264-269): the per-pair kernel-MLP basis
+//     basis[m, j] = act(delta_m . W[:, j] + b[j]) / pdf[m],
+//     delta_m = (p_in[nbr_m] - p_out[centre]) * inv_radii
+// is evaluated in registers inside the matrix-core projection kernels, so the
+// [M, K] basis tensor and its gradient never reach HBM.  Forward produces the
+// same [N_out, C, K] projection as mc_basis + basis_proj; backward produces the
+// feature gradient and the kernel-MLP weight / bias gradients from the upstream
+// [N_out, C, K] gradient.  K = 16 (v_mfma_f32_16x16x4f32), D = 2 or 3,
+// C in {16, 32, 64, 128}; other shapes use the separate kernels.
+#include "common.h"
+#include "fill.h"
+#include "mfma.h"
+
+namespace mccnn {
+
+constexpr int kFusedUnroll = 4;
+constexpr int kFusedK = 16;
+
+template <int D>
+struct McParams {
+  const float *pin;        // [N_in, D]
+  const float *pout;       // [N_out, D]
+  const float *inv_radii;  // [D]
+  const float *weights;    // [L, D, H]
+  const float *biases;     // [L*H]
+  const float *pdf;        // [M]
+  int hidden;              // H
+  int act;
+};
+
+// Weight column j of the flattened [D, L*H] kernel matrix.
+template <int D>
+__device__ __forceinline__ void load_weight_column(const McParams<D> &p, int j, float *w,
+                                                   float *bias) {
+  const int l = j / p.hidden, h = j - l * p.hidden;
+#pragma unroll
+  for (int d = 0; d < D; ++d) w[d] = p.weights[(l * D + d) * p.hidden + h];
+  *bias = p.biases[j];
+}
+
+template <int kCPL, int D>
+__global__ void __launch_bounds__(256) mc_conv_project16_kernel(
+    int64_t n_out, int C, int chunks, const float *__restrict__ feat,
+    const int2 *__restrict__ nbrs, const int *__restrict__ ranges, McParams<D> p,
+    float *__restrict__ out) {
+  constexpr int K = kFusedK;
+  constexpr int kCW = 16 * kCPL;
+  const int lane = lane_id();
+  const int64_t wid = wave_slot();
+  const int64_t centre = wid / chunks;
+  if (centre >= n_out) return;
+  const int chunk = (int)(wid - centre * chunks);
+  const int quarter = lane >> 4, col = lane & 15;
+  const int a = centre > 0 ? ranges[centre - 1] : 0, b = ranges[centre];
+  const float *fbase = feat + chunk * kCW + col * kCPL;
+  float wcol[D], ctr[D], ir[D], bcol;
+  load_weight_column<D>(p, col, wcol, &bcol);
+#pragma unroll
+  for (int d = 0; d < D; ++d) {
+    ctr[d] = p.pout[centre * D + d];
+    ir[d] = p.inv_radii[d];
+  }
+  v4f acc[kCPL];
+#pragma unroll
+  for (int j = 0; j < kCPL; ++j)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) acc[j][r] = 0.0f;
+
+  for (int m0 = a; m0 < b; m0 += kWave) {
+    const int cnt = b - m0 < kWave ? b - m0 : kWave;
+    const int myidx = nbrs[m0 + (lane < cnt ? lane : 0)].x;
+    const int steps = (cnt + 3) >> 2;
+    for (int t = 0; t < steps; t += kFusedUnroll) {
+      FVec<kCPL> f[kFusedUnroll];
+      float w[kFusedUnroll];
+#pragma unroll
+      for (int u = 0; u < kFusedUnroll; ++u) {
+        const int n = 4 * (t + u) + quarter;
+        const bool valid = n < cnt;
+        const int idx = __shfl(myidx, n & (kWave - 1), kWave);
+        f[u] = load_vec<kCPL>(fbase + (int64_t)idx * C, valid);
+        w[u] = 0.0f;
+        if (valid) {
+          float z = bcol;
+#pragma unroll
+          for (int d = 0; d < D; ++d)
+            z += (p.pin[(int64_t)idx * D + d] - ctr[d]) * ir[d] * wcol[d];
+          w[u] = act_fwd(p.act, z) / p.pdf[m0 + n];
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < kFusedUnroll; ++u)
+#pragma unroll
+        for (int j = 0; j < kCPL; ++j)
+          acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(w[u], f[u].v[j], acc[j], 0, 0, 0);
+    }
+  }
+  float *o = out + centre * (int64_t)C * K + (int64_t)chunk * kCW * K + 4 * quarter;
+#pragma unroll
+  for (int j = 0; j < kCPL; ++j)
+    __builtin_nontemporal_store(acc[j], reinterpret_cast<v4f *>(o + (col * kCPL + j) * K));
+}
+
+constexpr int kFusedGradBlocks = 2048;
+
+// Persistent wavefronts stride over the centres.  Per tile of 16 pairs:
+//   dbasis^T [k x pair] by MFMA (reduction over channels), turned in registers
+//   into dz = dbasis * act'(z) / pdf and accumulated into per-lane partial sums
+//   of dW[d][k] = sum delta_d * dz and db[k] = sum dz (lane (pair, quarter) owns
+//   k = 4*quarter .. +3);
+//   dfeat [pair x channel] by MFMA with the recomputed basis as A operand,
+//   added to the feature gradient with fp32 atomics.
+// At the end the partial sums are reduced over the 16 pair-lanes and the waves
+// of the block and written to partials[block][(D+1)][K].
+template <int C, int D>
+__global__ void __launch_bounds__(256) mc_conv_project_grads16_kernel(
+    int64_t n_out, const float *__restrict__ feat, const int2 *__restrict__ nbrs,
+    const int *__restrict__ ranges, McParams<D> p, const float *__restrict__ in_grad,
+    float *__restrict__ dfeat, float *__restrict__ partials) {
+  constexpr int K = kFusedK;
+  constexpr int kQuarterC = C / 4;
+  constexpr int kTiles = C / 16;
+  __shared__ float red[kWavesPerBlock][(D + 1) * K];
+  const int lane = lane_id(), wave = threadIdx.x / kWave;
+  const int quarter = lane >> 4, col = lane & 15;
+  float wk[4][D], bk[4], ir[D];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) load_weight_column<D>(p, 4 * quarter + r, wk[r], &bk[r]);
+#pragma unroll
+  for (int d = 0; d < D; ++d) ir[d] = p.inv_radii[d];
+  float dw[4][D], db[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    db[r] = 0.0f;
+#pragma unroll
+    for (int d = 0; d < D; ++d) dw[r][d] = 0.0f;
+  }
+  const int64_t total_waves = (int64_t)gridDim.x * kWavesPerBlock;
+  for (int64_t centre = wave_slot(); centre < n_out; centre += total_waves) {
+    const int a = centre > 0 ? ranges[centre - 1] : 0, b = ranges[centre];
+    if (b <= a) continue;
+    const float *gi = in_grad + centre * (int64_t)C * K;
+    float gk[kQuarterC];
+#pragma unroll
+    for (int s = 0; s < kQuarterC; ++s) gk[s] = gi[(quarter * kQuarterC + s) * K + col];
+    FVec<4> gt[kTiles];
+#pragma unroll
+    for (int t = 0; t < kTiles; ++t)
+      gt[t] = load_vec<4>(gi + (16 * t + col) * K + 4 * quarter, true);
+    float ctr[D];
+#pragma unroll
+    for (int d = 0; d < D; ++d) ctr[d] = p.pout[centre * D + d];
+
+    for (int m0 = a; m0 < b; m0 += 16) {
+      const int cnt = b - m0 < 16 ? b - m0 : 16;
+      const bool valid = col < cnt;
+      const int idx = nbrs[m0 + (valid ? col : 0)].x;
+      // this lane's pair: delta, and for its four basis columns z, basis and act'/pdf
+      float delta[D], basis4[4], dact4[4];
+      {
+        const float inv_pdf = valid ? 1.0f / p.pdf[m0 + col] : 0.0f;
+#pragma unroll
+        for (int d = 0; d < D; ++d)
+          delta[d] = valid ? (p.pin[(int64_t)idx * D + d] - ctr[d]) * ir[d] : 0.0f;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          float z = bk[r];
+#pragma unroll
+          for (int d = 0; d < D; ++d) z += delta[d] * wk[r][d];
+          basis4[r] = valid ? act_fwd(p.act, z) * inv_pdf : 0.0f;
+          dact4[r] = act_bwd(p.act, z) * inv_pdf;
+        }
+      }
+      {
+        const FVec<kQuarterC> f =
+            load_vec<kQuarterC>(feat + (int64_t)idx * C + quarter * kQuarterC, valid);
+        v4f acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int s = 0; s < kQuarterC; ++s)
+          acc = __builtin_amdgcn_mfma_f32_16x16x4f32(gk[s], f.v[s], acc, 0, 0, 0);
+        // acc[r] = dbasis[pair col][k = 4*quarter + r]
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const float dz = acc[r] * dact4[r];
+          db[r] += dz;
+#pragma unroll
+          for (int d = 0; d < D; ++d) dw[r][d] += delta[d] * dz;
+        }
+      }
+#pragma unroll
+      for (int t = 0; t < kTiles; ++t) {
+        v4f acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int s = 0; s < 4; ++s)
+          acc = __builtin_amdgcn_mfma_f32_16x16x4f32(basis4[s], gt[t].v[s], acc, 0, 0, 0);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int n = 4 * quarter + r;
+          const int nidx = __shfl(idx, n, kWave);
+          if (n < cnt) unsafeAtomicAdd(dfeat + (int64_t)nidx * C + 16 * t + col, acc[r]);
+        }
+      }
+    }
+  }
+  // reduce over the 16 pair-lanes of each quarter
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+#pragma unroll
+    for (int off = 8; off > 0; off >>= 1) {
+      db[r] += __shfl_xor(db[r], off, kWave);
+#pragma unroll
+      for (int d = 0; d < D; ++d) dw[r][d] += __shfl_xor(dw[r][d], off, kWave);
+    }
+  }
+  if (col == 0) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int k = 4 * quarter + r;
+#pragma unroll
+      for (int d = 0; d < D; ++d) red[wave][d * K + k] = dw[r][d];
+      red[wave][D * K + k] = db[r];
+    }
+  }
+  __syncthreads();
+  if (threadIdx.x < (D + 1) * K) {
+    float s = 0.0f;
+#pragma unroll
+    for (int w = 0; w < kWavesPerBlock; ++w) s += red[w][threadIdx.x];
+    partials[(int64_t)blockIdx.x * (D + 1) * K + threadIdx.x] = s;
+  }
+}
+
+// weight_grads [L, D, H], bias_grads [L*H] from partials [blocks][(D+1)][K].
+__global__ void mc_conv_reduce_kernel(int blocks, int D, int K, int H,
+                                      const float *__restrict__ partials,
+                                      float *__restrict__ dweights, float *__restrict__ dbiases) {
+  const int t = blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= (D + 1) * K) return;
+  const int q = t / K, j = t - q * K;
+  float s = 0.0f;
+  for (int b = 0; b < blocks; ++b) s += partials[(int64_t)b * (D + 1) * K + t];
+  const int l = j / H, h = j - l * H;
+  if (q < D) dweights[(l * D + q) * H + h] = s;
+  else dbiases[j] = s;
+}
+
+static bool fused_supported(int D, int C, int K) {
+  return (D == 2 || D == 3) && K == kFusedK && (C == 16 || C == 32 || C == 64 || C == 128);
+}
+
+static int check_fused_args(const char *op, int num_dims, int num_features, int num_basis,
+                            int num_mlps, int activation, int64_t num_neighbors,
+                            int64_t num_samples) {
+  MCCNN_REQUIRE(fused_supported(num_dims, num_features, num_basis),
+                "%s supports D in {2,3}, K = 16 and C in {16,32,64,128} (got D=%d, K=%d, C=%d); "
+                "use mc_basis + basis_proj for other shapes", op, num_dims, num_basis,
+                num_features);
+  MCCNN_REQUIRE(num_mlps > 0 && num_basis % num_mlps == 0,
+                "%s expects the number of basis functions to be divisible by the number of "
+                "kernel MLPs", op);
+  MCCNN_REQUIRE(activation >= 0 && activation <= 2, "%s expects a known activation", op);
+  MCCNN_REQUIRE(num_neighbors >= 0 && num_neighbors < ((int64_t)1 << 31) && num_samples >= 0 &&
+                    num_samples < ((int64_t)1 << 31),
+                "%s expects sizes in [0, 2^31)", op);
+  return MCCNN_OK;
+}
+
+}  // namespace mccnn
+
+using namespace mccnn;
+
+extern "C" int mccnn_mc_conv_supported(int num_dims, int num_features, int num_basis) {
+  return fused_supported(num_dims, num_features, num_basis) ? 1 : 0;
+}
+
+extern "C" int mccnn_mc_conv_project(mccnn_stream_t stream, int num_dims, int64_t num_pts,
+                                     const float *points_in, int num_features,
+                                     const float *features, int64_t num_samples,
+                                     const float *points_out, int64_t num_neighbors,
+                                     const int32_t *neighbors, const int32_t *ranges,
+                                     const float *inv_radii, int num_basis, int num_mlps,
+                                     int activation, const float *weights, const float *biases,
+                                     const float *pdf, float *out) {
+  int rc = check_fused_args("mc_conv_project", num_dims, num_features, num_basis, num_mlps,
+                            activation, num_neighbors, num_samples);
+  if (rc != MCCNN_OK) return rc;
+  MCCNN_REQUIRE(num_pts >= 0, "mc_conv_project expects a non-negative size");
+  if (num_samples == 0) return MCCNN_OK;
+  MCCNN_REQUIRE(ranges && out && points_out && inv_radii && weights && biases &&
+                    (num_neighbors == 0 || (points_in && features && neighbors && pdf)),
+                "mc_conv_project received a null tensor");
+  hipStream_t s = as_stream(stream);
+  int cpl = 1;
+  for (int c = 8; c >= 1; c >>= 1)
+    if (num_features % (16 * c) == 0) { cpl = c; break; }
+  const int chunks = num_features / (16 * cpl);
+  const dim3 grid(wave_grid(num_samples * chunks)), block(256);
+  const int2 *nb = (const int2 *)neighbors;
+#define MCCNN_FUSED_FWD(CPL_, D_)                                                              \
+  {                                                                                            \
+    McParams<D_> prm{points_in, points_out, inv_radii, weights, biases, pdf,                   \
+                     num_basis / num_mlps, activation};                                        \
+    hipLaunchKernelGGL((mc_conv_project16_kernel<CPL_, D_>), grid, block, 0, s, num_samples,   \
+                       num_features, chunks, features, nb, ranges, prm, out);                  \
+  }
+#define MCCNN_FUSED_FWD_D(CPL_) \
+  if (num_dims == 3) MCCNN_FUSED_FWD(CPL_, 3) else MCCNN_FUSED_FWD(CPL_, 2)
+  switch (cpl) {
+    case 8: MCCNN_FUSED_FWD_D(8); break;
+    case 4: MCCNN_FUSED_FWD_D(4); break;
+    case 2: MCCNN_FUSED_FWD_D(2); break;
+    default: MCCNN_FUSED_FWD_D(1); break;
+  }
+#undef MCCNN_FUSED_FWD_D
+#undef MCCNN_FUSED_FWD
+  MCCNN_LAUNCH_CHECK();
+  return MCCNN_OK;
+}
+
+extern "C" size_t mccnn_mc_conv_project_grads_workspace_bytes(int num_dims, int num_basis) {
+  if (!valid_dims(num_dims) || num_basis <= 0) return 0;
+  return align256(sizeof(float) * (size_t)kFusedGradBlocks * (num_dims + 1) * num_basis);
+}
+
+extern "C" int mccnn_mc_conv_project_grads(
+    mccnn_stream_t stream, int num_dims, int64_t num_pts, const float *points_in,
+    int num_features, const float *features, int64_t num_samples, const float *points_out,
+    int64_t num_neighbors, const int32_t *neighbors, const int32_t *ranges,
+    const float *inv_radii, int num_basis, int num_mlps, int activation, const float *weights,
+    const float *biases, const float *pdf, const float *in_grads, void *workspace,
+    size_t workspace_bytes, float *feature_grads_out, float *weight_grads_out,
+    float *bias_grads_out) {
+  int rc = check_fused_args("mc_conv_project_grads", num_dims, num_features, num_basis, num_mlps,
+                            activation, num_neighbors, num_samples);
+  if (rc != MCCNN_OK) return rc;
+  MCCNN_REQUIRE(num_pts >= 0, "mc_conv_project_grads expects a non-negative size");
+  MCCNN_REQUIRE(workspace && weight_grads_out && bias_grads_out && weights && biases &&
+                    inv_radii,
+                "mc_conv_project_grads received a null tensor");
+  MCCNN_REQUIRE(workspace_bytes >=
+                    mccnn_mc_conv_project_grads_workspace_bytes(num_dims, num_basis),
+                "mc_conv_project_grads workspace too small");
+  hipStream_t s = as_stream(stream);
+  if (num_pts > 0) {
+    MCCNN_REQUIRE(feature_grads_out, "mc_conv_project_grads received a null tensor");
+    rc = fill_zero(s, feature_grads_out, sizeof(float) * (size_t)num_pts * num_features);
+    if (rc != MCCNN_OK) return rc;
+  }
+  MCCNN_REQUIRE(num_samples == 0 || num_neighbors == 0 ||
+                    (points_in && points_out && features && neighbors && ranges && pdf &&
+                     in_grads),
+                "mc_conv_project_grads received a null tensor");
+  int64_t blocks64 = (num_samples + kWavesPerBlock - 1) / kWavesPerBlock;
+  int blocks = (int)(blocks64 > kFusedGradBlocks ? kFusedGradBlocks : blocks64);
+  if (blocks < 1) blocks = 1;
+  const dim3 grid(blocks), block(256);
+  const int2 *nb = (const int2 *)neighbors;
+#define MCCNN_FUSED_BWD(C_, D_)                                                                \
+  {                                                                                            \
+    McParams<D_> prm{points_in, points_out, inv_radii, weights, biases, pdf,                   \
+                     num_basis / num_mlps, activation};                                        \
+    hipLaunchKernelGGL((mc_conv_project_grads16_kernel<C_, D_>), grid, block, 0, s,            \
+                       num_samples, features, nb, ranges, prm, in_grads, feature_grads_out,    \
+                       (float *)workspace);                                                    \
+  }
+#define MCCNN_FUSED_BWD_D(C_) \
+  if (num_dims == 3) MCCNN_FUSED_BWD(C_, 3) else MCCNN_FUSED_BWD(C_, 2)
+  switch (num_features) {
+    case 16: MCCNN_FUSED_BWD_D(16); break;
+    case 32: MCCNN_FUSED_BWD_D(32); break;
+    case 64: MCCNN_FUSED_BWD_D(64); break;
+    default: MCCNN_FUSED_BWD_D(128); break;
+  }
+#undef MCCNN_FUSED_BWD_D
+#undef MCCNN_FUSED_BWD
+  MCCNN_LAUNCH_CHECK();
+  const int outs = (num_dims + 1) * num_basis;
+  hipLaunchKernelGGL(mc_conv_reduce_kernel, dim3(blocks_for(outs, 64)), dim3(64), 0, s, blocks,
+                     num_dims, num_basis, num_basis / num_mlps, (const float *)workspace,
+                     weight_grads_out, bias_grads_out);
+  MCCNN_LAUNCH_CHECK();
+  return MCCNN_OK;
+}

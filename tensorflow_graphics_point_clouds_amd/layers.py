@@ -49,6 +49,49 @@ class _MCBasis(torch.autograd.Function):
         return dw, db, None, None, None, None, None, None
 
 
+class _MCConvProject(torch.autograd.Function):
+    """mc_basis followed by basis_proj in one kernel (the basis is evaluated in
+    registers); differentiable in the kernel weights, biases and the features."""
+
+    @staticmethod
+    def forward(ctx, weights, biases, features, points_in, points_out, neighbors, ranges,
+                inv_radii, pdf, act):
+        num_mlps, dims, hidden = weights.shape
+        k = num_mlps * hidden
+        out = torch.empty((ranges.shape[0], features.shape[1], k), dtype=_F32,
+                          device=features.device)
+        _lib.call("mc_conv_project", stream(), cint(dims), i64(features.shape[0]),
+                  ptr(points_in, _F32), cint(features.shape[1]), ptr(features, _F32),
+                  i64(ranges.shape[0]), ptr(points_out, _F32), i64(neighbors.shape[0]),
+                  ptr(neighbors, _I32), ptr(ranges, _I32), ptr(inv_radii, _F32), cint(k),
+                  cint(num_mlps), cint(act), ptr(weights, _F32), ptr(biases, _F32),
+                  ptr(pdf, _F32), ptr(out))
+        ctx.save_for_backward(weights, biases, features, points_in, points_out, neighbors,
+                              ranges, inv_radii, pdf)
+        ctx.act = act
+        return out
+
+    @staticmethod
+    def backward(ctx, grad):
+        (weights, biases, features, points_in, points_out, neighbors, ranges, inv_radii,
+         pdf) = ctx.saved_tensors
+        num_mlps, dims, hidden = weights.shape
+        k = num_mlps * hidden
+        L = _lib.lib()
+        ws = _lib.workspace(L.mccnn_mc_conv_project_grads_workspace_bytes(cint(dims), cint(k)),
+                            weights.device)
+        dfeat = torch.empty_like(features)
+        dw, db = torch.empty_like(weights), torch.empty_like(biases)
+        _lib.call("mc_conv_project_grads", stream(), cint(dims), i64(features.shape[0]),
+                  ptr(points_in, _F32), cint(features.shape[1]), ptr(features, _F32),
+                  i64(ranges.shape[0]), ptr(points_out, _F32), i64(neighbors.shape[0]),
+                  ptr(neighbors, _I32), ptr(ranges, _I32), ptr(inv_radii, _F32), cint(k),
+                  cint(num_mlps), cint(ctx.act), ptr(weights, _F32), ptr(biases, _F32),
+                  ptr(pdf, _F32), ptr(grad.contiguous(), _F32), ptr(ws), _lib.csize(ws.numel()),
+                  ptr(dfeat), ptr(dw), ptr(db))
+        return dw, db, dfeat, None, None, None, None, None, None, None
+
+
 def _truncated_normal(shape, std, generator, device):
     t = torch.empty(shape, dtype=_F32)
     torch.nn.init.trunc_normal_(t, mean=0.0, std=std, a=-2 * std, b=2 * std,
@@ -62,7 +105,7 @@ class MCConv(torch.nn.Module):
 
     def __init__(self, num_features_in, num_features_out, num_dims, num_mlps=4, mlp_size=(8,),
                  non_linearity_type="leaky_relu", weights=None, biases=None,
-                 final_weights=None, device="cuda", seed=0):
+                 final_weights=None, device="cuda", seed=0, fused=True):
         super().__init__()
         if num_features_out % num_mlps != 0:
             raise ValueError("The number of output features must be divisible by the number"
@@ -87,6 +130,8 @@ class MCConv(torch.nn.Module):
         self.biases = torch.nn.Parameter(biases.to(_F32).contiguous())
         self.final_weights = torch.nn.Parameter(final_weights.to(_F32).contiguous())
         self.last_neighborhood = None
+        # evaluate the kernel MLP inside the projection kernel when the shape allows
+        self.fused = fused
 
     def forward(self, features, point_cloud_in, point_cloud_out, radius, neighborhood=None,
                 bandwidth=0.2):
@@ -98,14 +143,23 @@ class MCConv(torch.nn.Module):
             neighborhood = pc.Neighborhood(grid, radii, point_cloud_out)
         self.last_neighborhood = neighborhood
         pdf = neighborhood.get_pdf(bandwidth=bandwidth, mode=pc.KDEMode.constant)
-        basis = _MCBasis.apply(self.weights, self.biases.reshape(self._num_mlps, self._hidden),
-                               point_cloud_in._points, point_cloud_out._points,
-                               neighborhood._original_neigh_ids, torch.reciprocal(radii), pdf,
-                               self._act)
-        proj = tfg_custom_ops.basis_proj(basis, features.contiguous(),
-                                         neighborhood._original_neigh_ids,
-                                         neighborhood._samples_neigh_ranges,
-                                         neighborhood._centre_order)
+        biases = self.biases.reshape(self._num_mlps, self._hidden)
+        k = self._num_mlps * self._hidden
+        if self.fused and _lib.lib().mccnn_mc_conv_supported(cint(d), cint(self._num_features_in),
+                                                             cint(k)):
+            proj = _MCConvProject.apply(self.weights, biases, features.contiguous(),
+                                        point_cloud_in._points, point_cloud_out._points,
+                                        neighborhood._original_neigh_ids,
+                                        neighborhood._samples_neigh_ranges,
+                                        torch.reciprocal(radii), pdf, self._act)
+        else:
+            basis = _MCBasis.apply(self.weights, biases, point_cloud_in._points,
+                                   point_cloud_out._points, neighborhood._original_neigh_ids,
+                                   torch.reciprocal(radii), pdf, self._act)
+            proj = tfg_custom_ops.basis_proj(basis, features.contiguous(),
+                                             neighborhood._original_neigh_ids,
+                                             neighborhood._samples_neigh_ranges,
+                                             neighborhood._centre_order)
         n, c, l, h = proj.shape[0], self._num_features_in, self._num_mlps, self._hidden
         if l == 1:
             return proj.reshape(n, c * h) @ self.final_weights[0]
