@@ -230,6 +230,33 @@ int mccnn_basis_proj_grads_ordered(
     int64_t in_grads_dim1, int64_t in_grads_dim2, const float *in_grads,
     float *basis_grads_out, float *feature_grads_out);
 
+/* Pair lists grouped by neighbour point, the transposed view of a pair table:
+ * point_ranges_out [num_pts] (inclusive end offsets) and pair_order_out [M], the
+ * pair indices sorted by neighbours[:,0], ties in ascending pair index.  No
+ * counterpart in the reference (whose backward scatters with atomics); it is
+ * built once per neighbourhood and reused by every backward pass. */
+size_t mccnn_transpose_neighbors_workspace_bytes(int64_t num_neighbors,
+                                                 int64_t num_pts);
+int mccnn_transpose_neighbors(mccnn_stream_t stream, int64_t num_neighbors,
+                              const int32_t *neighbors, int64_t num_pts,
+                              void *workspace, size_t workspace_bytes,
+                              int32_t *point_ranges_out, int32_t *pair_order_out);
+
+/* BasisProjGrads without atomics: the feature gradient of each pair is written
+ * to pair_rows_workspace [M, C] and then summed per point over the lists of
+ * mccnn_transpose_neighbors, in a fixed order (bit-reproducible, unlike the
+ * atomic scatter of the reference, basis_proj_grads_kernels.cu.cc:120-140).
+ * K in {16, 32}, C in {16, 32, 64, 128} (C >= 32 for K = 32). */
+int mccnn_basis_proj_grads_gathered(
+    mccnn_stream_t stream, int64_t basis_rows, int num_basis, const float *basis,
+    int64_t num_pts, int num_features, const float *features,
+    int64_t num_neighbors, int neighbors_rank, int neighbors_cols,
+    const int32_t *neighbors, int64_t num_samples, const int32_t *ranges,
+    int in_grads_rank, int64_t in_grads_dim0, int64_t in_grads_dim1,
+    int64_t in_grads_dim2, const float *in_grads, const int32_t *point_ranges,
+    const int32_t *pair_order, float *pair_rows_workspace,
+    float *basis_grads_out, float *feature_grads_out);
+
 /* ------------------------------------------------------------- sampling --- */
 
 /* Sampling: sampling/cc/ops/sampling_ops.cpp:33-204, split at the host
@@ -338,7 +365,9 @@ int mccnn_mc_basis_grads(mccnn_stream_t stream, int64_t num_neighbors,
  * separate entry points up to fp32 summation order; the [M, K] basis and its
  * gradient are never written.  mccnn_mc_conv_supported() tells whether a shape
  * is covered (D in {2,3}, K = 16, C in {16,32,64,128}); other shapes return
- * MCCNN_INVALID_ARGUMENT and must use the separate entry points.  No
+ * MCCNN_INVALID_ARGUMENT and must use the separate entry points.  The last three
+ * inputs of the backward select the atomic-free feature gradient of
+ * mccnn_basis_proj_grads_gathered (all NULL = atomics).  No
  * counterpart among the reference's ops, which materialise the basis in
  * TensorFlow. */
 int mccnn_mc_conv_supported(int num_dims, int num_features, int num_basis);
@@ -358,7 +387,9 @@ int mccnn_mc_conv_project_grads(
     const int32_t *ranges, const float *inv_radii, int num_basis, int num_mlps,
     int activation, const float *weights, const float *biases, const float *pdf,
     const float *in_grads, void *workspace, size_t workspace_bytes,
-    float *feature_grads_out, float *weight_grads_out, float *bias_grads_out);
+    const int32_t *point_ranges, const int32_t *pair_order,
+    float *pair_rows_workspace, float *feature_grads_out,
+    float *weight_grads_out, float *bias_grads_out);
 
 /* Per-pair kernel-point weights, pylib/pc/layers/KPConv.py:29-57,193-213:
  *   d[m,k] = || delta_m - (kernel_points[k] + offsets[ctr_m,k]) ||

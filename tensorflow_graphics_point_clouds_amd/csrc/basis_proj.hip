@@ -264,7 +264,8 @@ template <int C>
 __global__ void __launch_bounds__(256) basis_proj_grads_mfma32_kernel(
     int64_t n_out, const float *__restrict__ basis, const float *__restrict__ feat,
     const int2 *__restrict__ nbrs, const int *__restrict__ ranges, const int *__restrict__ order,
-    const float *__restrict__ in_grad, float *__restrict__ dbasis, float *__restrict__ dfeat) {
+    const float *__restrict__ in_grad, float *__restrict__ dbasis, float *__restrict__ dfeat,
+    float *__restrict__ pair_rows) {
   constexpr int K = 32;
   constexpr int kHalfC = C / 2;      // reduction run of a lane in the dbasis product
   const int lane = lane_id();
@@ -319,7 +320,10 @@ __global__ void __launch_bounds__(256) basis_proj_grads_mfma32_kernel(
         for (int r = 0; r < 16; ++r) {
           const int n = 8 * (r >> 2) + (r & 3) + 4 * half;
           const int nidx = __shfl(idx, n, kWave);
-          if (n < cnt) unsafeAtomicAdd(dfeat + (int64_t)nidx * C + ct + col, acc[r]);
+          if (n < cnt) {
+            if (pair_rows) pair_rows[(int64_t)(m0 + n) * C + ct + col] = acc[r];
+            else unsafeAtomicAdd(dfeat + (int64_t)nidx * C + ct + col, acc[r]);
+          }
         }
       }
     }
@@ -330,7 +334,8 @@ template <int C>
 __global__ void __launch_bounds__(256) basis_proj_grads_mfma16_kernel(
     int64_t n_out, const float *__restrict__ basis, const float *__restrict__ feat,
     const int2 *__restrict__ nbrs, const int *__restrict__ ranges, const int *__restrict__ order,
-    const float *__restrict__ in_grad, float *__restrict__ dbasis, float *__restrict__ dfeat) {
+    const float *__restrict__ in_grad, float *__restrict__ dbasis, float *__restrict__ dfeat,
+    float *__restrict__ pair_rows) {
   constexpr int K = 16;
   constexpr int kQuarterC = C / 4;
   constexpr int kTiles = C / 16;
@@ -380,11 +385,65 @@ __global__ void __launch_bounds__(256) basis_proj_grads_mfma16_kernel(
         for (int r = 0; r < 4; ++r) {
           const int n = 4 * quarter + r;
           const int nidx = __shfl(idx, n, kWave);
-          if (n < cnt) unsafeAtomicAdd(dfeat + (int64_t)nidx * C + 16 * t + col, acc[r]);
+          if (n < cnt) {
+            if (pair_rows) pair_rows[(int64_t)(m0 + n) * C + 16 * t + col] = acc[r];
+            else unsafeAtomicAdd(dfeat + (int64_t)nidx * C + 16 * t + col, acc[r]);
+          }
         }
       }
     }
   }
+}
+
+// Second phase of the atomic-free feature gradient: dfeat[n, :] = sum of the
+// per-pair rows of the pairs whose neighbour is n.  point_ranges (inclusive ends)
+// and pair_order list those pairs per point, in ascending pair index, so the sum
+// has a fixed order.  kLanes lanes per point, one float4 each (C = 4 * kLanes).
+template <int kLanes>
+__global__ void __launch_bounds__(256) dfeat_gather_kernel(
+    int64_t n_in, const int *__restrict__ point_ranges, const int *__restrict__ pair_order,
+    const float *__restrict__ pair_rows, float *__restrict__ dfeat) {
+  constexpr int C = 4 * kLanes;
+  const int64_t n = (int64_t)blockIdx.x * (256 / kLanes) + threadIdx.x / kLanes;
+  if (n >= n_in) return;
+  const int sub = threadIdx.x % kLanes;
+  const int a = n > 0 ? point_ranges[n - 1] : 0, b = point_ranges[n];
+  float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+  int j = a;
+  for (; j + 4 <= b; j += 4) {
+    float4 v[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      v[u] = *reinterpret_cast<const float4 *>(pair_rows + (int64_t)pair_order[j + u] * C + 4 * sub);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      acc.x += v[u].x; acc.y += v[u].y; acc.z += v[u].z; acc.w += v[u].w;
+    }
+  }
+  for (; j < b; ++j) {
+    const float4 v =
+        *reinterpret_cast<const float4 *>(pair_rows + (int64_t)pair_order[j] * C + 4 * sub);
+    acc.x += v.x; acc.y += v.y; acc.z += v.z; acc.w += v.w;
+  }
+  *reinterpret_cast<float4 *>(dfeat + n * C + 4 * sub) = acc;
+}
+
+int launch_dfeat_gather(hipStream_t s, int64_t num_pts, int C, const int *point_ranges,
+                        const int *pair_order, const float *pair_rows, float *dfeat) {
+  if (num_pts == 0) return MCCNN_OK;
+  const int lanes = C / 4;
+  const dim3 grid(blocks_for(num_pts, 256 / lanes)), block(256);
+  switch (lanes) {
+    case 4: hipLaunchKernelGGL(dfeat_gather_kernel<4>, grid, block, 0, s, num_pts, point_ranges, pair_order, pair_rows, dfeat); break;
+    case 8: hipLaunchKernelGGL(dfeat_gather_kernel<8>, grid, block, 0, s, num_pts, point_ranges, pair_order, pair_rows, dfeat); break;
+    case 16: hipLaunchKernelGGL(dfeat_gather_kernel<16>, grid, block, 0, s, num_pts, point_ranges, pair_order, pair_rows, dfeat); break;
+    case 32: hipLaunchKernelGGL(dfeat_gather_kernel<32>, grid, block, 0, s, num_pts, point_ranges, pair_order, pair_rows, dfeat); break;
+    default:
+      set_error("feature-gradient gather supports C in {16, 32, 64, 128} (got %d)", C);
+      return MCCNN_INVALID_ARGUMENT;
+  }
+  MCCNN_LAUNCH_CHECK();
+  return MCCNN_OK;
 }
 
 static bool mfma_grads_supported(int C, int K) {
@@ -508,14 +567,22 @@ extern "C" int mccnn_basis_proj_ordered(mccnn_stream_t stream, int64_t basis_row
   return MCCNN_OK;
 }
 
-extern "C" int mccnn_basis_proj_grads_ordered(
+static int basis_proj_grads_impl(
     mccnn_stream_t stream, int64_t basis_rows, int num_basis, const float *basis, int64_t num_pts,
     int num_features, const float *features, int64_t num_neighbors, int neighbors_rank,
     int neighbors_cols, const int32_t *neighbors, int64_t num_samples, const int32_t *ranges,
-    const int32_t *centre_order, int in_grads_rank, int64_t in_grads_dim0, int64_t in_grads_dim1,
-    int64_t in_grads_dim2, const float *in_grads, float *basis_grads_out,
+    const int32_t *order, int in_grads_rank, int64_t in_grads_dim0, int64_t in_grads_dim1,
+    int64_t in_grads_dim2, const float *in_grads, const int32_t *point_ranges,
+    const int32_t *pair_order, float *pair_rows, float *basis_grads_out,
     float *feature_grads_out) {
-  const int32_t *order = centre_order;
+  const bool gathered = pair_rows != nullptr;
+  if (gathered) {
+    MCCNN_REQUIRE(point_ranges && pair_order,
+                  "BasisProjGrads needs the transposed pair lists with a pair-row workspace");
+    MCCNN_REQUIRE(mfma_grads_supported(num_features, num_basis),
+                  "the gathered feature gradient supports K in {16,32} and C in {16,32,64,128} "
+                  "(C >= 32 for K = 32)");
+  }
   int rc = check_basis_args("BasisProjGrads", basis_rows, num_basis, num_features, num_neighbors,
                             neighbors_rank, neighbors_cols);
   if (rc != MCCNN_OK) return rc;
@@ -526,7 +593,7 @@ extern "C" int mccnn_basis_proj_grads_ordered(
                     num_neighbors < ((int64_t)1 << 31),
                 "BasisProjGrads expects sizes in [0, 2^31)");
   hipStream_t s = as_stream(stream);
-  if (num_pts > 0) {
+  if (num_pts > 0 && (!gathered || num_samples == 0 || num_neighbors == 0)) {
     MCCNN_REQUIRE(feature_grads_out, "BasisProjGrads received a null tensor");
     rc = fill_zero(s, feature_grads_out, sizeof(float) * (size_t)num_pts * num_features);
     if (rc != MCCNN_OK) return rc;
@@ -540,7 +607,7 @@ extern "C" int mccnn_basis_proj_grads_ordered(
     const dim3 grid(wave_grid(num_samples)), block(256);
 #define MCCNN_BWD(KERNEL_, C_)                                                              \
   hipLaunchKernelGGL((KERNEL_<C_>), grid, block, 0, s, num_samples, basis, features, nb,   \
-                     ranges, order, in_grads, basis_grads_out, feature_grads_out)
+                     ranges, order, in_grads, basis_grads_out, feature_grads_out, pair_rows)
     if (num_basis == 32) {
       switch (num_features) {
         case 32: MCCNN_BWD(basis_proj_grads_mfma32_kernel, 32); break;
@@ -557,6 +624,9 @@ extern "C" int mccnn_basis_proj_grads_ordered(
     }
 #undef MCCNN_BWD
     MCCNN_LAUNCH_CHECK();
+    if (gathered)
+      return launch_dfeat_gather(s, num_pts, num_features, point_ranges, pair_order, pair_rows,
+                                 feature_grads_out);
     return MCCNN_OK;
   }
   const int chunks = generic_chunks(num_features, num_basis);
@@ -586,6 +656,36 @@ extern "C" int mccnn_basis_proj(mccnn_stream_t stream, int64_t basis_rows, int n
                                   neighbors, num_samples, ranges, nullptr, out);
 }
 
+extern "C" int mccnn_basis_proj_grads_ordered(
+    mccnn_stream_t stream, int64_t basis_rows, int num_basis, const float *basis, int64_t num_pts,
+    int num_features, const float *features, int64_t num_neighbors, int neighbors_rank,
+    int neighbors_cols, const int32_t *neighbors, int64_t num_samples, const int32_t *ranges,
+    const int32_t *centre_order, int in_grads_rank, int64_t in_grads_dim0, int64_t in_grads_dim1,
+    int64_t in_grads_dim2, const float *in_grads, float *basis_grads_out,
+    float *feature_grads_out) {
+  return basis_proj_grads_impl(stream, basis_rows, num_basis, basis, num_pts, num_features,
+                               features, num_neighbors, neighbors_rank, neighbors_cols, neighbors,
+                               num_samples, ranges, centre_order, in_grads_rank, in_grads_dim0,
+                               in_grads_dim1, in_grads_dim2, in_grads, nullptr, nullptr, nullptr,
+                               basis_grads_out, feature_grads_out);
+}
+
+extern "C" int mccnn_basis_proj_grads_gathered(
+    mccnn_stream_t stream, int64_t basis_rows, int num_basis, const float *basis, int64_t num_pts,
+    int num_features, const float *features, int64_t num_neighbors, int neighbors_rank,
+    int neighbors_cols, const int32_t *neighbors, int64_t num_samples, const int32_t *ranges,
+    int in_grads_rank, int64_t in_grads_dim0, int64_t in_grads_dim1, int64_t in_grads_dim2,
+    const float *in_grads, const int32_t *point_ranges, const int32_t *pair_order,
+    float *pair_rows_workspace, float *basis_grads_out, float *feature_grads_out) {
+  MCCNN_REQUIRE(pair_rows_workspace || num_neighbors == 0,
+                "BasisProjGrads (gathered) needs a [num_neighbors, C] workspace");
+  return basis_proj_grads_impl(stream, basis_rows, num_basis, basis, num_pts, num_features,
+                               features, num_neighbors, neighbors_rank, neighbors_cols, neighbors,
+                               num_samples, ranges, nullptr, in_grads_rank, in_grads_dim0,
+                               in_grads_dim1, in_grads_dim2, in_grads, point_ranges, pair_order,
+                               pair_rows_workspace, basis_grads_out, feature_grads_out);
+}
+
 extern "C" int mccnn_basis_proj_grads(mccnn_stream_t stream, int64_t basis_rows, int num_basis,
                                       const float *basis, int64_t num_pts, int num_features,
                                       const float *features, int64_t num_neighbors,
@@ -595,9 +695,9 @@ extern "C" int mccnn_basis_proj_grads(mccnn_stream_t stream, int64_t basis_rows,
                                       int64_t in_grads_dim0, int64_t in_grads_dim1,
                                       int64_t in_grads_dim2, const float *in_grads,
                                       float *basis_grads_out, float *feature_grads_out) {
-  return mccnn_basis_proj_grads_ordered(stream, basis_rows, num_basis, basis, num_pts,
-                                        num_features, features, num_neighbors, neighbors_rank,
-                                        neighbors_cols, neighbors, num_samples, ranges, nullptr,
-                                        in_grads_rank, in_grads_dim0, in_grads_dim1, in_grads_dim2,
-                                        in_grads, basis_grads_out, feature_grads_out);
+  return basis_proj_grads_impl(stream, basis_rows, num_basis, basis, num_pts, num_features,
+                               features, num_neighbors, neighbors_rank, neighbors_cols, neighbors,
+                               num_samples, ranges, nullptr, in_grads_rank, in_grads_dim0,
+                               in_grads_dim1, in_grads_dim2, in_grads, nullptr, nullptr, nullptr,
+                               basis_grads_out, feature_grads_out);
 }

@@ -110,23 +110,34 @@ constexpr int kFusedGradBlocks = 2048;
 //   of dW[d][k] = sum delta_d * dz and db[k] = sum dz (lane (pair, quarter) owns
 //   k = 4*quarter .. +3);
 //   dfeat [pair x channel] by MFMA with the recomputed basis as A operand,
-//   added to the feature gradient with fp32 atomics.
+//   added to the feature gradient with fp32 atomics, or (pair_rows given)
+//   stored per pair for the atomic-free gather that follows.
 // At the end the partial sums are reduced over the 16 pair-lanes and the waves
 // of the block and written to partials[block][(D+1)][K].
-template <int C, int D>
+// kDB / kDF select the two halves (weight-gradient half, feature-gradient half);
+// launching them as two kernels keeps each under ~90 registers, which more than
+// pays for reading the upstream gradient twice.
+template <int C, int D, bool kDB, bool kDF>
 __global__ void __launch_bounds__(256) mc_conv_project_grads16_kernel(
     int64_t n_out, const float *__restrict__ feat, const int2 *__restrict__ nbrs,
     const int *__restrict__ ranges, McParams<D> p, const float *__restrict__ in_grad,
-    float *__restrict__ dfeat, float *__restrict__ partials) {
+    float *__restrict__ dfeat, float *__restrict__ pair_rows, float *__restrict__ partials) {
   constexpr int K = kFusedK;
   constexpr int kQuarterC = C / 4;
   constexpr int kTiles = C / 16;
   __shared__ float red[kWavesPerBlock][(D + 1) * K];
+  __shared__ float wlds[K * (D + 1)];     // column j: D weights then the bias
   const int lane = lane_id(), wave = threadIdx.x / kWave;
   const int quarter = lane >> 4, col = lane & 15;
-  float wk[4][D], bk[4], ir[D];
+  if (threadIdx.x < K) {
+    float w[D], bias;
+    load_weight_column<D>(p, threadIdx.x, w, &bias);
 #pragma unroll
-  for (int r = 0; r < 4; ++r) load_weight_column<D>(p, 4 * quarter + r, wk[r], &bk[r]);
+    for (int d = 0; d < D; ++d) wlds[threadIdx.x * (D + 1) + d] = w[d];
+    wlds[threadIdx.x * (D + 1) + D] = bias;
+  }
+  __syncthreads();
+  float ir[D];
 #pragma unroll
   for (int d = 0; d < D; ++d) ir[d] = p.inv_radii[d];
   float dw[4][D], db[4];
@@ -142,12 +153,10 @@ __global__ void __launch_bounds__(256) mc_conv_project_grads16_kernel(
     if (b <= a) continue;
     const float *gi = in_grad + centre * (int64_t)C * K;
     float gk[kQuarterC];
+    if (kDB) {
 #pragma unroll
-    for (int s = 0; s < kQuarterC; ++s) gk[s] = gi[(quarter * kQuarterC + s) * K + col];
-    FVec<4> gt[kTiles];
-#pragma unroll
-    for (int t = 0; t < kTiles; ++t)
-      gt[t] = load_vec<4>(gi + (16 * t + col) * K + 4 * quarter, true);
+      for (int s = 0; s < kQuarterC; ++s) gk[s] = gi[(quarter * kQuarterC + s) * K + col];
+    }
     float ctr[D];
 #pragma unroll
     for (int d = 0; d < D; ++d) ctr[d] = p.pout[centre * D + d];
@@ -156,25 +165,25 @@ __global__ void __launch_bounds__(256) mc_conv_project_grads16_kernel(
       const int cnt = b - m0 < 16 ? b - m0 : 16;
       const bool valid = col < cnt;
       const int idx = nbrs[m0 + (valid ? col : 0)].x;
-      // this lane's pair: delta, and for its four basis columns z, basis and act'/pdf
-      float delta[D], basis4[4], dact4[4];
-      {
-        const float inv_pdf = valid ? 1.0f / p.pdf[m0 + col] : 0.0f;
+      FVec<kQuarterC> f;
+      if (kDB) f = load_vec<kQuarterC>(feat + (int64_t)idx * C + quarter * kQuarterC, valid);
+      const float inv_pdf = valid ? 1.0f / p.pdf[m0 + col] : 0.0f;
+      float delta[D];
 #pragma unroll
-        for (int d = 0; d < D; ++d)
-          delta[d] = valid ? (p.pin[(int64_t)idx * D + d] - ctr[d]) * ir[d] : 0.0f;
+      for (int d = 0; d < D; ++d)
+        delta[d] = valid ? (p.pin[(int64_t)idx * D + d] - ctr[d]) * ir[d] : 0.0f;
+      // for this lane's pair and its four basis columns: basis and act'/pdf
+      float basis4[4], dact4[4];
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          float z = bk[r];
+      for (int r = 0; r < 4; ++r) {
+        const float *wr = wlds + (4 * quarter + r) * (D + 1);
+        float z = wr[D];
 #pragma unroll
-          for (int d = 0; d < D; ++d) z += delta[d] * wk[r][d];
-          basis4[r] = valid ? act_fwd(p.act, z) * inv_pdf : 0.0f;
-          dact4[r] = act_bwd(p.act, z) * inv_pdf;
-        }
+        for (int d = 0; d < D; ++d) z += delta[d] * wr[d];
+        basis4[r] = valid ? act_fwd(p.act, z) * inv_pdf : 0.0f;
+        dact4[r] = act_bwd(p.act, z) * inv_pdf;
       }
-      {
-        const FVec<kQuarterC> f =
-            load_vec<kQuarterC>(feat + (int64_t)idx * C + quarter * kQuarterC, valid);
+      if (kDB) {
         v4f acc = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
         for (int s = 0; s < kQuarterC; ++s)
@@ -189,20 +198,36 @@ __global__ void __launch_bounds__(256) mc_conv_project_grads16_kernel(
         }
       }
 #pragma unroll
-      for (int t = 0; t < kTiles; ++t) {
+      for (int t = 0; t < (kDF ? kTiles : 0); ++t) {
+        // B operand of channel tile t: G[c = 16 t + col][k = 4*quarter + s] (L1 resident)
+        const FVec<4> gt = load_vec<4>(gi + (16 * t + col) * K + 4 * quarter, true);
         v4f acc = {0.0f, 0.0f, 0.0f, 0.0f};
+        if (pair_rows) {
+          // rows = channels, columns = pairs: this lane holds channels
+          // 16 t + 4*quarter .. +3 of pair `col` -> one 16-byte store
 #pragma unroll
-        for (int s = 0; s < 4; ++s)
-          acc = __builtin_amdgcn_mfma_f32_16x16x4f32(basis4[s], gt[t].v[s], acc, 0, 0, 0);
+          for (int s = 0; s < 4; ++s)
+            acc = __builtin_amdgcn_mfma_f32_16x16x4f32(gt.v[s], basis4[s], acc, 0, 0, 0);
+          if (valid)
+            __builtin_nontemporal_store(
+                acc, reinterpret_cast<v4f *>(pair_rows + (int64_t)(m0 + col) * C + 16 * t +
+                                             4 * quarter));
+        } else {
+          // rows = pairs, columns = channels: 64 consecutive bytes per row and atomic
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const int n = 4 * quarter + r;
-          const int nidx = __shfl(idx, n, kWave);
-          if (n < cnt) unsafeAtomicAdd(dfeat + (int64_t)nidx * C + 16 * t + col, acc[r]);
+          for (int s = 0; s < 4; ++s)
+            acc = __builtin_amdgcn_mfma_f32_16x16x4f32(basis4[s], gt.v[s], acc, 0, 0, 0);
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int n = 4 * quarter + r;
+            const int nidx = __shfl(idx, n, kWave);
+            if (n < cnt) unsafeAtomicAdd(dfeat + (int64_t)nidx * C + 16 * t + col, acc[r]);
+          }
         }
       }
     }
   }
+  if (!kDB) return;
   // reduce over the 16 pair-lanes of each quarter
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
@@ -231,15 +256,19 @@ __global__ void __launch_bounds__(256) mc_conv_project_grads16_kernel(
   }
 }
 
-// weight_grads [L, D, H], bias_grads [L*H] from partials [blocks][(D+1)][K].
-__global__ void mc_conv_reduce_kernel(int blocks, int D, int K, int H,
-                                      const float *__restrict__ partials,
-                                      float *__restrict__ dweights, float *__restrict__ dbiases) {
-  const int t = blockIdx.x * blockDim.x + threadIdx.x;
+// weight_grads [L, D, H], bias_grads [L*H] from partials [blocks][(D+1)][K]: one
+// wavefront per output, lanes stride over the blocks, fixed summation order.
+__global__ void __launch_bounds__(256) mc_conv_reduce_kernel(int blocks, int D, int K, int H,
+                                                             const float *__restrict__ partials,
+                                                             float *__restrict__ dweights,
+                                                             float *__restrict__ dbiases) {
+  const int t = blockIdx.x * (256 / kWave) + threadIdx.x / kWave;
   if (t >= (D + 1) * K) return;
   const int q = t / K, j = t - q * K;
   float s = 0.0f;
-  for (int b = 0; b < blocks; ++b) s += partials[(int64_t)b * (D + 1) * K + t];
+  for (int b = lane_id(); b < blocks; b += kWave) s += partials[(int64_t)b * (D + 1) * K + t];
+  s = wave_sum(s);
+  if (lane_id() != 0) return;
   const int l = j / H, h = j - l * H;
   if (q < D) dweights[(l * D + q) * H + h] = s;
   else dbiases[j] = s;
@@ -329,8 +358,14 @@ extern "C" int mccnn_mc_conv_project_grads(
     int64_t num_neighbors, const int32_t *neighbors, const int32_t *ranges,
     const float *inv_radii, int num_basis, int num_mlps, int activation, const float *weights,
     const float *biases, const float *pdf, const float *in_grads, void *workspace,
-    size_t workspace_bytes, float *feature_grads_out, float *weight_grads_out,
+    size_t workspace_bytes, const int32_t *point_ranges, const int32_t *pair_order,
+    float *pair_rows_workspace, float *feature_grads_out, float *weight_grads_out,
     float *bias_grads_out) {
+  float *pair_rows = pair_rows_workspace;
+  const bool gathered = pair_rows != nullptr;
+  MCCNN_REQUIRE(!gathered || (point_ranges && pair_order),
+                "mc_conv_project_grads needs the transposed pair lists with a pair-row "
+                "workspace");
   int rc = check_fused_args("mc_conv_project_grads", num_dims, num_features, num_basis, num_mlps,
                             activation, num_neighbors, num_samples);
   if (rc != MCCNN_OK) return rc;
@@ -342,7 +377,7 @@ extern "C" int mccnn_mc_conv_project_grads(
                     mccnn_mc_conv_project_grads_workspace_bytes(num_dims, num_basis),
                 "mc_conv_project_grads workspace too small");
   hipStream_t s = as_stream(stream);
-  if (num_pts > 0) {
+  if (num_pts > 0 && (!gathered || num_samples == 0 || num_neighbors == 0)) {
     MCCNN_REQUIRE(feature_grads_out, "mc_conv_project_grads received a null tensor");
     rc = fill_zero(s, feature_grads_out, sizeof(float) * (size_t)num_pts * num_features);
     if (rc != MCCNN_OK) return rc;
@@ -355,14 +390,18 @@ extern "C" int mccnn_mc_conv_project_grads(
   int blocks = (int)(blocks64 > kFusedGradBlocks ? kFusedGradBlocks : blocks64);
   if (blocks < 1) blocks = 1;
   const dim3 grid(blocks), block(256);
+  const dim3 grid2(wave_grid(num_samples));      // the feature half keeps no running sums
   const int2 *nb = (const int2 *)neighbors;
 #define MCCNN_FUSED_BWD(C_, D_)                                                                \
   {                                                                                            \
     McParams<D_> prm{points_in, points_out, inv_radii, weights, biases, pdf,                   \
                      num_basis / num_mlps, activation};                                        \
-    hipLaunchKernelGGL((mc_conv_project_grads16_kernel<C_, D_>), grid, block, 0, s,            \
-                       num_samples, features, nb, ranges, prm, in_grads, feature_grads_out,    \
-                       (float *)workspace);                                                    \
+    hipLaunchKernelGGL((mc_conv_project_grads16_kernel<C_, D_, true, false>), grid, block, 0,  \
+                       s, num_samples, features, nb, ranges, prm, in_grads, feature_grads_out, \
+                       pair_rows, (float *)workspace);                                         \
+    hipLaunchKernelGGL((mc_conv_project_grads16_kernel<C_, D_, false, true>), grid2, block, 0, \
+                       s, num_samples, features, nb, ranges, prm, in_grads, feature_grads_out, \
+                       pair_rows, (float *)workspace);                                         \
   }
 #define MCCNN_FUSED_BWD_D(C_) \
   if (num_dims == 3) MCCNN_FUSED_BWD(C_, 3) else MCCNN_FUSED_BWD(C_, 2)
@@ -376,9 +415,13 @@ extern "C" int mccnn_mc_conv_project_grads(
 #undef MCCNN_FUSED_BWD
   MCCNN_LAUNCH_CHECK();
   const int outs = (num_dims + 1) * num_basis;
-  hipLaunchKernelGGL(mc_conv_reduce_kernel, dim3(blocks_for(outs, 64)), dim3(64), 0, s, blocks,
+  hipLaunchKernelGGL(mc_conv_reduce_kernel, dim3(blocks_for(outs, 256 / kWave)), dim3(256), 0, s,
+                     blocks,
                      num_dims, num_basis, num_basis / num_mlps, (const float *)workspace,
                      weight_grads_out, bias_grads_out);
   MCCNN_LAUNCH_CHECK();
+  if (gathered && num_samples > 0 && num_neighbors > 0)
+    return launch_dfeat_gather(s, num_pts, num_features, point_ranges, pair_order, pair_rows,
+                               feature_grads_out);
   return MCCNN_OK;
 }

@@ -28,6 +28,11 @@ static unsigned wave_grid(int64_t waves) {
 }
 
 
+// dfeat[n, :] = sum over the pairs listed for point n of pair_rows[pair, :]
+// (defined in basis_proj.hip).
+int launch_dfeat_gather(hipStream_t s, int64_t num_pts, int C, const int *point_ranges,
+                        const int *pair_order, const float *pair_rows, float *dfeat);
+
 typedef float v16f __attribute__((ext_vector_type(16)));
 typedef float v4f __attribute__((ext_vector_type(4)));
 

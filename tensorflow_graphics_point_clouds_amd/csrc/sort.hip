@@ -106,13 +106,17 @@ __global__ void __launch_bounds__(kSortThreads) sort_scatter_kernel(
   }
 }
 
-__global__ void __launch_bounds__(256) sort_copy_kernel(int64_t n, const int64_t *__restrict__ keys,
-                                                        int64_t *__restrict__ keys_out,
-                                                        int *__restrict__ idx_out) {
-  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n;
-       i += (int64_t)gridDim.x * blockDim.x) {
-    keys_out[i] = keys[i];
-    idx_out[i] = (int)i;
+// keys[m] = num_pts - 1 - neighbour id (descending key order = ascending id), and
+// the number of pairs of each point.
+__global__ void __launch_bounds__(256) transpose_keys_kernel(int64_t m_total, int64_t num_pts,
+                                                             const int2 *__restrict__ nbrs,
+                                                             int64_t *__restrict__ keys,
+                                                             int *__restrict__ counts) {
+  for (int64_t m = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; m < m_total;
+       m += (int64_t)gridDim.x * blockDim.x) {
+    const int n = nbrs[m].x;
+    keys[m] = num_pts - 1 - n;
+    atomicAdd(&counts[n], 1);
   }
 }
 
@@ -203,4 +207,70 @@ extern "C" int mccnn_sort_keys_descending(mccnn_stream_t stream, int64_t num_pts
     iin = iout;
   }
   return MCCNN_OK;
+}
+
+// ------------------------------------------------- transposed pair lists ----
+
+namespace mccnn {
+struct TransposeWorkspace {
+  int64_t *keys;
+  int64_t *sorted_keys;
+  void *sort_ws;
+  size_t sort_ws_bytes;
+  int *scan_scratch;
+  int64_t *total;
+  size_t bytes;
+};
+
+static TransposeWorkspace carve_transpose_workspace(void *ws, int64_t m, int64_t n) {
+  char *p = (char *)ws;
+  TransposeWorkspace w;
+  size_t off = 0;
+  w.keys = (int64_t *)(p + off); off += align256(sizeof(int64_t) * (size_t)m);
+  w.sorted_keys = (int64_t *)(p + off); off += align256(sizeof(int64_t) * (size_t)m);
+  w.sort_ws = p + off;
+  w.sort_ws_bytes = carve_sort_workspace(nullptr, m).bytes;
+  off += align256(w.sort_ws_bytes);
+  w.scan_scratch = (int *)(p + off); off += align256(sizeof(int) * scan_scratch_ints(n));
+  w.total = (int64_t *)(p + off); off += 256;
+  w.bytes = off;
+  return w;
+}
+}  // namespace mccnn
+
+extern "C" size_t mccnn_transpose_neighbors_workspace_bytes(int64_t num_neighbors,
+                                                            int64_t num_pts) {
+  if (num_neighbors < 0) num_neighbors = 0;
+  if (num_pts < 0) num_pts = 0;
+  return carve_transpose_workspace(nullptr, num_neighbors, num_pts).bytes;
+}
+
+extern "C" int mccnn_transpose_neighbors(mccnn_stream_t stream, int64_t num_neighbors,
+                                         const int32_t *neighbors, int64_t num_pts,
+                                         void *workspace, size_t workspace_bytes,
+                                         int32_t *point_ranges_out, int32_t *pair_order_out) {
+  MCCNN_REQUIRE(num_neighbors >= 0 && num_neighbors < ((int64_t)1 << 31) && num_pts >= 0 &&
+                    num_pts < ((int64_t)1 << 31),
+                "transpose_neighbors expects sizes in [0, 2^31)");
+  hipStream_t s = as_stream(stream);
+  if (num_pts == 0) return MCCNN_OK;
+  MCCNN_REQUIRE(point_ranges_out, "transpose_neighbors received a null tensor");
+  int rc = fill_zero(s, point_ranges_out, sizeof(int32_t) * (size_t)num_pts);
+  if (rc != MCCNN_OK) return rc;
+  if (num_neighbors == 0) return MCCNN_OK;
+  MCCNN_REQUIRE(neighbors && workspace && pair_order_out,
+                "transpose_neighbors received a null tensor");
+  const TransposeWorkspace w = carve_transpose_workspace(workspace, num_neighbors, num_pts);
+  MCCNN_REQUIRE(workspace_bytes >= w.bytes, "transpose_neighbors workspace too small (%zu < %zu)",
+                workspace_bytes, w.bytes);
+  int64_t work = num_neighbors > ((int64_t)1 << 26) ? ((int64_t)1 << 26) : num_neighbors;
+  hipLaunchKernelGGL(transpose_keys_kernel, dim3(blocks_for(work, 256)), dim3(256), 0, s,
+                     num_neighbors, num_pts, (const int2 *)neighbors, w.keys, point_ranges_out);
+  MCCNN_LAUNCH_CHECK();
+  int bits = 1;
+  while (((int64_t)1 << bits) < num_pts) ++bits;
+  rc = mccnn_sort_keys_descending(stream, num_neighbors, bits, w.keys, w.sorted_keys,
+                                  pair_order_out, w.sort_ws, w.sort_ws_bytes);
+  if (rc != MCCNN_OK) return rc;
+  return inclusive_scan_i32(s, num_pts, point_ranges_out, w.scan_scratch, w.total);
 }

@@ -55,7 +55,7 @@ class _MCConvProject(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, weights, biases, features, points_in, points_out, neighbors, ranges,
-                inv_radii, pdf, act):
+                inv_radii, pdf, act, transposed):
         num_mlps, dims, hidden = weights.shape
         k = num_mlps * hidden
         out = torch.empty((ranges.shape[0], features.shape[1], k), dtype=_F32,
@@ -68,7 +68,7 @@ class _MCConvProject(torch.autograd.Function):
                   ptr(pdf, _F32), ptr(out))
         ctx.save_for_backward(weights, biases, features, points_in, points_out, neighbors,
                               ranges, inv_radii, pdf)
-        ctx.act = act
+        ctx.act, ctx.transposed = act, transposed
         return out
 
     @staticmethod
@@ -82,14 +82,19 @@ class _MCConvProject(torch.autograd.Function):
                             weights.device)
         dfeat = torch.empty_like(features)
         dw, db = torch.empty_like(weights), torch.empty_like(biases)
+        t_ranges = t_order = rows = None
+        if ctx.transposed is not None:
+            t_ranges, t_order = ctx.transposed
+            rows = torch.empty((neighbors.shape[0], features.shape[1]), dtype=_F32,
+                               device=features.device)
         _lib.call("mc_conv_project_grads", stream(), cint(dims), i64(features.shape[0]),
                   ptr(points_in, _F32), cint(features.shape[1]), ptr(features, _F32),
                   i64(ranges.shape[0]), ptr(points_out, _F32), i64(neighbors.shape[0]),
                   ptr(neighbors, _I32), ptr(ranges, _I32), ptr(inv_radii, _F32), cint(k),
                   cint(num_mlps), cint(ctx.act), ptr(weights, _F32), ptr(biases, _F32),
                   ptr(pdf, _F32), ptr(grad.contiguous(), _F32), ptr(ws), _lib.csize(ws.numel()),
-                  ptr(dfeat), ptr(dw), ptr(db))
-        return dw, db, dfeat, None, None, None, None, None, None, None
+                  ptr(t_ranges), ptr(t_order), ptr(rows), ptr(dfeat), ptr(dw), ptr(db))
+        return dw, db, dfeat, None, None, None, None, None, None, None, None
 
 
 def _truncated_normal(shape, std, generator, device):
@@ -105,7 +110,7 @@ class MCConv(torch.nn.Module):
 
     def __init__(self, num_features_in, num_features_out, num_dims, num_mlps=4, mlp_size=(8,),
                  non_linearity_type="leaky_relu", weights=None, biases=None,
-                 final_weights=None, device="cuda", seed=0, fused=True):
+                 final_weights=None, device="cuda", seed=0, fused=True, gathered_grads=True):
         super().__init__()
         if num_features_out % num_mlps != 0:
             raise ValueError("The number of output features must be divisible by the number"
@@ -132,6 +137,8 @@ class MCConv(torch.nn.Module):
         self.last_neighborhood = None
         # evaluate the kernel MLP inside the projection kernel when the shape allows
         self.fused = fused
+        # feature gradient by per-pair rows + ordered gather instead of float atomics
+        self.gathered_grads = gathered_grads
 
     def forward(self, features, point_cloud_in, point_cloud_out, radius, neighborhood=None,
                 bandwidth=0.2):
@@ -145,13 +152,17 @@ class MCConv(torch.nn.Module):
         pdf = neighborhood.get_pdf(bandwidth=bandwidth, mode=pc.KDEMode.constant)
         biases = self.biases.reshape(self._num_mlps, self._hidden)
         k = self._num_mlps * self._hidden
+        transposed = None
+        if self.gathered_grads and features.requires_grad and \
+                tfg_custom_ops.gathered_grads_supported(self._num_features_in, k):
+            transposed = neighborhood.transposed_pairs()
         if self.fused and _lib.lib().mccnn_mc_conv_supported(cint(d), cint(self._num_features_in),
                                                              cint(k)):
             proj = _MCConvProject.apply(self.weights, biases, features.contiguous(),
                                         point_cloud_in._points, point_cloud_out._points,
                                         neighborhood._original_neigh_ids,
                                         neighborhood._samples_neigh_ranges,
-                                        torch.reciprocal(radii), pdf, self._act)
+                                        torch.reciprocal(radii), pdf, self._act, transposed)
         else:
             basis = _MCBasis.apply(self.weights, biases, point_cloud_in._points,
                                    point_cloud_out._points, neighborhood._original_neigh_ids,
@@ -159,7 +170,7 @@ class MCConv(torch.nn.Module):
             proj = tfg_custom_ops.basis_proj(basis, features.contiguous(),
                                              neighborhood._original_neigh_ids,
                                              neighborhood._samples_neigh_ranges,
-                                             neighborhood._centre_order)
+                                             neighborhood._centre_order, transposed)
         n, c, l, h = proj.shape[0], self._num_features_in, self._num_mlps, self._hidden
         if l == 1:
             return proj.reshape(n, c * h) @ self.final_weights[0]
@@ -214,9 +225,13 @@ class KPConv(torch.nn.Module):
             cfloat(sigma), ptr(point_cloud_in._points, _F32), ptr(point_cloud_out._points, _F32),
             ptr(ids, _I32), ptr(torch.reciprocal(radii), _F32), ptr(self._kernel_points, _F32),
             ptr(None), ptr(basis), ptr(None))
+        transposed = None
+        if features.requires_grad and tfg_custom_ops.gathered_grads_supported(
+                self._num_features_in, k):
+            transposed = neighborhood.transposed_pairs()
         proj = tfg_custom_ops.basis_proj(basis, features.contiguous(), ids,
                                          neighborhood._samples_neigh_ranges,
-                                         neighborhood._centre_order)
+                                         neighborhood._centre_order, transposed)
         c = self._num_features_in
         if k == kp:
             return proj.reshape(-1, c * k) @ self.weights

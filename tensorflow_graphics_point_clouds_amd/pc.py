@@ -130,6 +130,15 @@ class Neighborhood:
         self._pdf_per_point = None
         # optional visiting order of the centres for the projection kernels
         self._centre_order = None
+        self._transposed_pairs = None
+
+    def transposed_pairs(self):
+        """(point_ranges, pair_order): the pairs grouped by neighbour point, used by
+        the atomic-free feature gradients; built on first use and kept."""
+        if self._transposed_pairs is None:
+            self._transposed_pairs = tfg_custom_ops.transpose_neighbors(
+                self._original_neigh_ids, self._grid._point_cloud._points.shape[0])
+        return self._transposed_pairs
 
     def compute_centre_order(self):
         """Rank the centres by their cell key in the grid (a scheduling hint for

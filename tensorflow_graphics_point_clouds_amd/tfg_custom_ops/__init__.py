@@ -15,7 +15,7 @@ from .._lib import InvalidArgumentError, cint, i64, ptr, stream, vptr
 
 __all__ = ["compute_keys", "build_grid_ds", "find_neighbors", "sampling",
            "compute_pdf_with_pt_grads", "compute_pdf_pt_grads", "basis_proj",
-           "basis_proj_grads", "InvalidArgumentError"]
+           "basis_proj_grads", "transpose_neighbors", "InvalidArgumentError"]
 
 _F32, _I32, _I64 = torch.float32, torch.int32, torch.int64
 
@@ -168,45 +168,78 @@ def _basis_proj_raw(basis, features, neighbors, ranges, centre_order=None):
     return out
 
 
+def gathered_grads_supported(num_features, num_basis):
+    """Shapes for which the atomic-free feature gradient exists."""
+    if num_basis == 16:
+        return num_features in (16, 32, 64, 128)
+    if num_basis == 32:
+        return num_features in (32, 64, 128)
+    return False
+
+
 def basis_proj_grads(basis_neighbors, pt_features, neighbors, sample_neigh_indices,
-                     in_gradients, centre_order=None):
+                     in_gradients, centre_order=None, transposed=None):
     """BasisProjGrads (basis_proj_ops.cpp:40-53) -> (basis_gradients [M, K],
-    feat_gradients [N_in, C])."""
+    feat_gradients [N_in, C]).  `transposed` = (point_ranges, pair_order) from
+    `transpose_neighbors` selects the atomic-free, bit-reproducible feature
+    gradient (needs an [M, C] scratch tensor)."""
     dbasis = torch.empty_like(basis_neighbors)
     dfeat = torch.empty_like(pt_features)
     g = in_gradients
-    _lib.call("basis_proj_grads_ordered", stream(), i64(basis_neighbors.shape[0]),
-              cint(_dim(basis_neighbors, 1)), ptr(basis_neighbors, _F32),
-              i64(pt_features.shape[0]), cint(_dim(pt_features, 1)), ptr(pt_features, _F32),
-              i64(neighbors.shape[0]), cint(neighbors.dim()), cint(_dim(neighbors, 1)),
-              ptr(neighbors, _I32), i64(sample_neigh_indices.shape[0]),
-              ptr(sample_neigh_indices, _I32),
-              ptr(centre_order, _I32 if centre_order is not None else None), cint(g.dim()),
-              i64(_dim(g, 0)), i64(_dim(g, 1)), i64(_dim(g, 2)), ptr(g, _F32), ptr(dbasis),
-              ptr(dfeat))
+    head = (stream(), i64(basis_neighbors.shape[0]), cint(_dim(basis_neighbors, 1)),
+            ptr(basis_neighbors, _F32), i64(pt_features.shape[0]), cint(_dim(pt_features, 1)),
+            ptr(pt_features, _F32), i64(neighbors.shape[0]), cint(neighbors.dim()),
+            cint(_dim(neighbors, 1)), ptr(neighbors, _I32), i64(sample_neigh_indices.shape[0]),
+            ptr(sample_neigh_indices, _I32))
+    gdims = (cint(g.dim()), i64(_dim(g, 0)), i64(_dim(g, 1)), i64(_dim(g, 2)), ptr(g, _F32))
+    if transposed is not None and gathered_grads_supported(_dim(pt_features, 1),
+                                                           _dim(basis_neighbors, 1)):
+        rows = torch.empty((neighbors.shape[0], pt_features.shape[1]), dtype=_F32,
+                           device=pt_features.device)
+        _lib.call("basis_proj_grads_gathered", *head, *gdims, ptr(transposed[0], _I32),
+                  ptr(transposed[1], _I32), ptr(rows), ptr(dbasis), ptr(dfeat))
+    else:
+        _lib.call("basis_proj_grads_ordered", *head,
+                  ptr(centre_order, _I32 if centre_order is not None else None), *gdims,
+                  ptr(dbasis), ptr(dfeat))
     return dbasis, dfeat
+
+
+def transpose_neighbors(neighbors, num_pts):
+    """Pair lists grouped by neighbour point: (point_ranges [num_pts] inclusive end
+    offsets, pair_order [M] pair indices sorted by neighbors[:, 0], stable)."""
+    L = _lib.lib()
+    L.mccnn_transpose_neighbors_workspace_bytes.restype = _lib.csize
+    m, dev = neighbors.shape[0], neighbors.device
+    ws = _lib.workspace(L.mccnn_transpose_neighbors_workspace_bytes(i64(m), i64(num_pts)), dev)
+    point_ranges = torch.empty(num_pts, dtype=_I32, device=dev)
+    pair_order = torch.empty(m, dtype=_I32, device=dev)
+    _lib.call("transpose_neighbors", stream(), i64(m), ptr(neighbors, _I32), i64(num_pts),
+              ptr(ws), _lib.csize(ws.numel()), ptr(point_ranges), ptr(pair_order))
+    return point_ranges, pair_order
 
 
 class _BasisProj(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, basis, features, neighbors, ranges, centre_order):
+    def forward(ctx, basis, features, neighbors, ranges, centre_order, transposed):
         ctx.save_for_backward(basis, features, neighbors, ranges)
-        ctx.centre_order = centre_order
+        ctx.centre_order, ctx.transposed = centre_order, transposed
         return _basis_proj_raw(basis, features, neighbors, ranges, centre_order)
 
     @staticmethod
     def backward(ctx, grad):
         basis, features, neighbors, ranges = ctx.saved_tensors
         dbasis, dfeat = basis_proj_grads(basis, features, neighbors, ranges, grad.contiguous(),
-                                         ctx.centre_order)
-        return dbasis, dfeat, None, None, None
+                                         ctx.centre_order, ctx.transposed)
+        return dbasis, dfeat, None, None, None, None
 
 
 def basis_proj(basis_neighbors, pt_features, neighbors, sample_neigh_indices,
-               centre_order=None):
+               centre_order=None, transposed=None):
     """BasisProj (basis_proj_ops.cpp:25-38): [N_out, C, K] sum over the pairs of
     each centre of feature (outer) basis; differentiable in basis and features.
-    `centre_order` (optional int32 permutation of the centres, e.g. their order by
-    grid cell) only changes the order in which centres are processed."""
+    `centre_order` (optional int32 permutation of the centres) only changes the
+    order in which centres are processed; `transposed` (optional, see
+    `basis_proj_grads`) selects the atomic-free backward."""
     return _BasisProj.apply(basis_neighbors, pt_features, neighbors, sample_neigh_indices,
-                            centre_order)
+                            centre_order, transposed)

@@ -394,3 +394,33 @@ def test_full_size_invariants(ops):
     lhs = float((up.double() * p1.double()).sum())
     assert abs(float((db.double() * basis.double()).sum()) - lhs) <= 1e-5 * abs(lhs) + 1e-3
     assert abs(float((df.double() * f1.double()).sum()) - lhs) <= 1e-5 * abs(lhs) + 1e-3
+
+
+@pytest.mark.parametrize("c,k", [(16, 16), (64, 16), (128, 16), (32, 32), (128, 32)])
+def test_gathered_feature_gradient(ops, oracle, c, k):
+    """Transposed pair lists equal a stable argsort by neighbour id, and the
+    atomic-free feature gradient matches the oracle and is bit-reproducible."""
+    rng = np.random.default_rng(c + k)
+    n = 3000
+    pts, bids = _cloud(rng, 2, n, 3)
+    g = oracle.Grid(pts, bids, 2, 0.12)
+    ctr, cb = _cloud(rng, 2, 900, 3)
+    nbh = oracle.Neighborhood(g, 0.12, ctr, cb)
+    ids = nbh.original_neigh_ids
+    t_ranges, t_order = ops.transpose_neighbors(dev(ids), n)
+    expect_order = np.argsort(ids[:, 0], kind="stable")
+    assert np.array_equal(t_order.cpu().numpy(), expect_order)
+    assert np.array_equal(t_ranges.cpu().numpy(), np.cumsum(np.bincount(ids[:, 0], minlength=n)))
+    basis = rng.random((len(ids), k)).astype(np.float32)
+    feat = rng.standard_normal((n, c)).astype(np.float32)
+    up = rng.standard_normal((900, c, k)).astype(np.float32)
+    args = (dev(basis), dev(feat), dev(ids), dev(nbh.ranges), dev(up))
+    db1, df1 = ops.basis_proj_grads(*args, transposed=(t_ranges, t_order))
+    db2, df2 = ops.basis_proj_grads(*args, transposed=(t_ranges, t_order))
+    assert torch.equal(df1, df2) and torch.equal(db1, db2)
+    edb, edf = oracle.basis_proj_grads(basis, feat, ids, nbh.ranges, up)
+    assert_normwise(db1.cpu().numpy(), edb)
+    assert_normwise(df1.cpu().numpy(), edf)
+    # points that are nobody's neighbour get an exact zero row
+    unused = np.setdiff1d(np.arange(n), ids[:, 0])
+    assert len(unused) > 0 and float(df1[dev(unused).long()].abs().sum()) == 0.0
