@@ -404,6 +404,44 @@ int mccnn_kp_basis(mccnn_stream_t stream, int64_t num_neighbors, int num_dims,
                    const float *kernel_points, const float *offsets,
                    float *basis_out, float *dist_out);
 
+/* Gradient of mccnn_kp_basis with respect to the per-centre kernel-point
+ * offsets (deformable KPConv, pylib/pc/layers/KPConv.py:193-198 differentiated):
+ * offsets_grads_out [num_samples, num_kernel_points, D] for upstream basis_grads
+ * [M, num_basis].  The pairs of a centre are summed in order, without atomics. */
+int mccnn_kp_basis_grads(mccnn_stream_t stream, int64_t num_neighbors,
+                         int num_dims, int num_kernel_points, int num_basis,
+                         int kind, float sigma, const float *points_in,
+                         const float *points_out, const int32_t *neighbors,
+                         int64_t num_samples, const int32_t *ranges,
+                         const float *inv_radii, const float *kernel_points,
+                         const float *offsets, const float *basis_grads,
+                         float *offsets_grads_out);
+
+/* Regularisation terms of deformable kernel points,
+ * pylib/pc/layers/KPConv.py:394-429: fit_out [num_samples, KP] = min over the
+ * pairs of the centre of (dist / sigma)^2 with the attaining pair in argmin_out
+ * (0 and -1 for a centre without pairs), repulsion_out [num_samples, KP] =
+ * sum over the other kernel points of the correlation weight of their distance.
+ * The loss is sum(fit) + sum(repulsion). */
+int mccnn_kp_regularization(mccnn_stream_t stream, int64_t num_neighbors,
+                            int num_dims, int num_kernel_points, int kind,
+                            float sigma, const float *points_in,
+                            const float *points_out, const int32_t *neighbors,
+                            int64_t num_samples, const int32_t *ranges,
+                            const float *inv_radii, const float *kernel_points,
+                            const float *offsets, float *fit_out,
+                            int32_t *argmin_out, float *repulsion_out);
+
+/* offsets_grads_out = loss_grad * d(sum(fit) + sum(repulsion)) / d(offsets). */
+int mccnn_kp_regularization_grads(mccnn_stream_t stream, int64_t num_neighbors,
+                                  int num_dims, int num_kernel_points, int kind,
+                                  float sigma, float loss_grad,
+                                  const float *points_in, const float *points_out,
+                                  const int32_t *neighbors, int64_t num_samples,
+                                  const float *inv_radii,
+                                  const float *kernel_points, const float *offsets,
+                                  const int32_t *argmin, float *offsets_grads_out);
+
 #ifdef __cplusplus
 }
 #endif

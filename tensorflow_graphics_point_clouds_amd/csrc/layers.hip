@@ -150,6 +150,169 @@ __global__ void __launch_bounds__(256) kp_basis_kernel(
   }
 }
 
+// d(weight)/d(distance) of the kernel-point correlation.
+__device__ __forceinline__ float kp_weight_slope(int kind, float sigma, float dist) {
+  if (kind == 0) return dist < sigma ? -1.0f / sigma : 0.0f;
+  const float s = sigma / 3.0f, q = dist / s;
+  return -2.0f * q / s * expf(-(q * q));
+}
+
+// Gradient of the kernel-point weights with respect to the per-centre offsets:
+//   doff[c, k, :] = sum over the pairs m of centre c of
+//                   dbasis[m, k] * w'(dist) * d(dist)/d(off),  d(dist)/d(off) = -diff / dist.
+// One thread per (centre, kernel point): the pairs of a centre are contiguous,
+// so the sum needs no atomics and has a fixed order.
+template <int D>
+__global__ void __launch_bounds__(256) kp_basis_grads_kernel(
+    int64_t n_out, int KP, int K, int kind, float sigma, const float *__restrict__ pin,
+    const float *__restrict__ pout, const int2 *__restrict__ nbrs, const int *__restrict__ ranges,
+    const float *__restrict__ inv_radii, const float *__restrict__ kpts,
+    const float *__restrict__ offsets, const float *__restrict__ dbasis,
+    float *__restrict__ doffsets) {
+  float ir[D];
+#pragma unroll
+  for (int d = 0; d < D; ++d) ir[d] = inv_radii[d];
+  const int64_t t = blockIdx.x * (int64_t)blockDim.x + threadIdx.x;
+  if (t >= n_out * KP) return;
+  const int64_t c = t / KP;
+  const int k = (int)(t - c * KP);
+  float kp[D], acc[D];
+#pragma unroll
+  for (int d = 0; d < D; ++d) {
+    kp[d] = kpts[k * D + d] + (offsets ? offsets[t * D + d] : 0.0f);
+    acc[d] = 0.0f;
+  }
+  const int a = c > 0 ? ranges[c - 1] : 0, b = ranges[c];
+  for (int m = a; m < b; ++m) {
+    const int2 pr = nbrs[m];
+    float diff[D], sq = 0.0f;
+#pragma unroll
+    for (int d = 0; d < D; ++d) {
+      diff[d] = (pin[(int64_t)pr.x * D + d] - pout[c * D + d]) * ir[d] - kp[d];
+      sq += diff[d] * diff[d];
+    }
+    const float dist = sqrtf(sq);
+    if (dist > 0.0f) {
+      const float g = dbasis[(int64_t)m * K + k] * kp_weight_slope(kind, sigma, dist) / dist;
+#pragma unroll
+      for (int d = 0; d < D; ++d) acc[d] -= g * diff[d];
+    }
+  }
+#pragma unroll
+  for (int d = 0; d < D; ++d) doffsets[t * D + d] = acc[d];
+}
+
+// Regularisation terms of the deformable kernel points (pylib/pc/layers/KPConv.py:394-429):
+//   fit[c, k]  = min over the pairs of centre c of (dist[m, k] / sigma)^2, with the pair that
+//                attains it in argmin[c, k] (-1 and 0 for a centre without pairs);
+//   rep[c]     = sum over k != k' of weight(|kp'_k - kp'_k'|), kp' = kernel point + offset.
+template <int D>
+__global__ void __launch_bounds__(256) kp_regularization_kernel(
+    int64_t n_out, int KP, int kind, float sigma, const float *__restrict__ pin,
+    const float *__restrict__ pout, const int2 *__restrict__ nbrs, const int *__restrict__ ranges,
+    const float *__restrict__ inv_radii, const float *__restrict__ kpts,
+    const float *__restrict__ offsets, float *__restrict__ fit, int *__restrict__ argmin,
+    float *__restrict__ rep) {
+  float ir[D];
+#pragma unroll
+  for (int d = 0; d < D; ++d) ir[d] = inv_radii[d];
+  const int64_t t = blockIdx.x * (int64_t)blockDim.x + threadIdx.x;
+  if (t >= n_out * KP) return;
+  const int64_t c = t / KP;
+  const int k = (int)(t - c * KP);
+  float kp[D];
+#pragma unroll
+  for (int d = 0; d < D; ++d) kp[d] = kpts[k * D + d] + offsets[t * D + d];
+  const int a = c > 0 ? ranges[c - 1] : 0, b = ranges[c];
+  float best = 0.0f;
+  int best_m = -1;
+  for (int m = a; m < b; ++m) {
+    const int2 pr = nbrs[m];
+    float sq = 0.0f;
+#pragma unroll
+    for (int d = 0; d < D; ++d) {
+      const float diff = (pin[(int64_t)pr.x * D + d] - pout[c * D + d]) * ir[d] - kp[d];
+      sq += diff * diff;
+    }
+    if (best_m < 0 || sq < best) {
+      best = sq;
+      best_m = m;
+    }
+  }
+  fit[t] = best / (sigma * sigma);
+  argmin[t] = best_m;
+  // repulsion of this kernel point against the others of the same centre
+  float r = 0.0f;
+  for (int k2 = 0; k2 < KP; ++k2) {
+    if (k2 == k) continue;
+    float sq = 0.0f;
+#pragma unroll
+    for (int d = 0; d < D; ++d) {
+      const float diff = kp[d] - (kpts[k2 * D + d] + offsets[(c * KP + k2) * D + d]);
+      sq += diff * diff;
+    }
+    const float dist = sqrtf(sq);
+    if (kind == 0) {
+      const float v = 1.0f - dist / sigma;
+      r += v > 0.0f ? v : 0.0f;
+    } else {
+      const float q = dist / (sigma / 3.0f);
+      r += expf(-(q * q));
+    }
+  }
+  rep[t] = r;
+}
+
+// d(scale * (sum fit + sum rep)) / d(offsets).
+template <int D>
+__global__ void __launch_bounds__(256) kp_regularization_grads_kernel(
+    int64_t n_out, int KP, int kind, float sigma, float scale, const float *__restrict__ pin,
+    const float *__restrict__ pout, const int2 *__restrict__ nbrs,
+    const float *__restrict__ inv_radii, const float *__restrict__ kpts,
+    const float *__restrict__ offsets, const int *__restrict__ argmin,
+    float *__restrict__ doffsets) {
+  float ir[D];
+#pragma unroll
+  for (int d = 0; d < D; ++d) ir[d] = inv_radii[d];
+  const int64_t t = blockIdx.x * (int64_t)blockDim.x + threadIdx.x;
+  if (t >= n_out * KP) return;
+  const int64_t c = t / KP;
+  const int k = (int)(t - c * KP);
+  float kp[D], g[D];
+#pragma unroll
+  for (int d = 0; d < D; ++d) {
+    kp[d] = kpts[k * D + d] + offsets[t * D + d];
+    g[d] = 0.0f;
+  }
+  const int m = argmin[t];
+  if (m >= 0) {       // fit: d/d(off) of |diff|^2 / sigma^2 = -2 diff / sigma^2
+    const int2 pr = nbrs[m];
+#pragma unroll
+    for (int d = 0; d < D; ++d) {
+      const float diff = (pin[(int64_t)pr.x * D + d] - pout[c * D + d]) * ir[d] - kp[d];
+      g[d] -= 2.0f * diff / (sigma * sigma);
+    }
+  }
+  // repulsion: the pair (k, k2) appears twice in the double sum
+  for (int k2 = 0; k2 < KP; ++k2) {
+    if (k2 == k) continue;
+    float diff[D], sq = 0.0f;
+#pragma unroll
+    for (int d = 0; d < D; ++d) {
+      diff[d] = kp[d] - (kpts[k2 * D + d] + offsets[(c * KP + k2) * D + d]);
+      sq += diff[d] * diff[d];
+    }
+    const float dist = sqrtf(sq);
+    if (dist > 0.0f) {
+      const float w = 2.0f * kp_weight_slope(kind, sigma, dist) / dist;
+#pragma unroll
+      for (int d = 0; d < D; ++d) g[d] += w * diff[d];
+    }
+  }
+#pragma unroll
+  for (int d = 0; d < D; ++d) doffsets[t * D + d] = scale * g[d];
+}
+
 static bool valid_basis_count(int k) { return k == 8 || k == 16 || k == 32 || k == 64; }
 
 }  // namespace mccnn
@@ -255,6 +418,96 @@ extern "C" int mccnn_kp_basis(mccnn_stream_t stream, int64_t num_neighbors, int 
                                                 points_in, points_out, (const int2 *)neighbors,
                                                 inv_radii, kernel_points, offsets, basis_out,
                                                 dist_out));
+  MCCNN_LAUNCH_CHECK();
+  return MCCNN_OK;
+}
+
+static int check_kp_args(const char *op, int num_dims, int num_kernel_points, int kind,
+                         float sigma, int64_t num_samples, int64_t num_neighbors) {
+  MCCNN_REQUIRE(valid_dims(num_dims), "%s expects a valid number of dimensions", op);
+  MCCNN_REQUIRE(num_kernel_points > 0 && num_kernel_points <= 64,
+                "%s expects between 1 and 64 kernel points", op);
+  MCCNN_REQUIRE(kind == 0 || kind == 1, "%s expects kind 0 (linear) or 1 (gaussian)", op);
+  MCCNN_REQUIRE(sigma > 0.0f, "%s expects a positive sigma", op);
+  MCCNN_REQUIRE(num_samples >= 0 && num_neighbors >= 0, "%s expects non-negative sizes", op);
+  return MCCNN_OK;
+}
+
+extern "C" int mccnn_kp_basis_grads(mccnn_stream_t stream, int64_t num_neighbors, int num_dims,
+                                    int num_kernel_points, int num_basis, int kind, float sigma,
+                                    const float *points_in, const float *points_out,
+                                    const int32_t *neighbors, int64_t num_samples,
+                                    const int32_t *ranges, const float *inv_radii,
+                                    const float *kernel_points, const float *offsets,
+                                    const float *basis_grads, float *offsets_grads_out) {
+  int rc = check_kp_args("kp_basis_grads", num_dims, num_kernel_points, kind, sigma, num_samples,
+                         num_neighbors);
+  if (rc != MCCNN_OK) return rc;
+  MCCNN_REQUIRE(valid_basis_count(num_basis) && num_kernel_points <= num_basis,
+                "kp_basis_grads expects 8, 16, 32 or 64 basis columns, at least one per kernel "
+                "point");
+  if (num_samples == 0) return MCCNN_OK;
+  MCCNN_REQUIRE(points_out && ranges && inv_radii && kernel_points && offsets_grads_out &&
+                    (num_neighbors == 0 || (points_in && neighbors && basis_grads)),
+                "kp_basis_grads received a null tensor");
+  const int64_t work = num_samples * num_kernel_points;
+  MCCNN_DIM_SWITCH(num_dims,
+                   hipLaunchKernelGGL(kp_basis_grads_kernel<D>, dim3(blocks_for(work, 256)),
+                                      dim3(256), 0, as_stream(stream), num_samples,
+                                      num_kernel_points, num_basis, kind, sigma, points_in,
+                                      points_out, (const int2 *)neighbors, ranges, inv_radii,
+                                      kernel_points, offsets, basis_grads, offsets_grads_out));
+  MCCNN_LAUNCH_CHECK();
+  return MCCNN_OK;
+}
+
+extern "C" int mccnn_kp_regularization(mccnn_stream_t stream, int64_t num_neighbors, int num_dims,
+                                       int num_kernel_points, int kind, float sigma,
+                                       const float *points_in, const float *points_out,
+                                       const int32_t *neighbors, int64_t num_samples,
+                                       const int32_t *ranges, const float *inv_radii,
+                                       const float *kernel_points, const float *offsets,
+                                       float *fit_out, int32_t *argmin_out, float *repulsion_out) {
+  int rc = check_kp_args("kp_regularization", num_dims, num_kernel_points, kind, sigma,
+                         num_samples, num_neighbors);
+  if (rc != MCCNN_OK) return rc;
+  if (num_samples == 0) return MCCNN_OK;
+  MCCNN_REQUIRE(points_out && ranges && inv_radii && kernel_points && offsets && fit_out &&
+                    argmin_out && repulsion_out && (num_neighbors == 0 || (points_in && neighbors)),
+                "kp_regularization received a null tensor");
+  const int64_t work = num_samples * num_kernel_points;
+  MCCNN_DIM_SWITCH(num_dims,
+                   hipLaunchKernelGGL(kp_regularization_kernel<D>, dim3(blocks_for(work, 256)),
+                                      dim3(256), 0, as_stream(stream), num_samples,
+                                      num_kernel_points, kind, sigma, points_in, points_out,
+                                      (const int2 *)neighbors, ranges, inv_radii, kernel_points,
+                                      offsets, fit_out, argmin_out, repulsion_out));
+  MCCNN_LAUNCH_CHECK();
+  return MCCNN_OK;
+}
+
+extern "C" int mccnn_kp_regularization_grads(mccnn_stream_t stream, int64_t num_neighbors,
+                                             int num_dims, int num_kernel_points, int kind,
+                                             float sigma, float loss_grad,
+                                             const float *points_in, const float *points_out,
+                                             const int32_t *neighbors, int64_t num_samples,
+                                             const float *inv_radii, const float *kernel_points,
+                                             const float *offsets, const int32_t *argmin,
+                                             float *offsets_grads_out) {
+  int rc = check_kp_args("kp_regularization_grads", num_dims, num_kernel_points, kind, sigma,
+                         num_samples, num_neighbors);
+  if (rc != MCCNN_OK) return rc;
+  if (num_samples == 0) return MCCNN_OK;
+  MCCNN_REQUIRE(points_out && inv_radii && kernel_points && offsets && argmin &&
+                    offsets_grads_out && (num_neighbors == 0 || (points_in && neighbors)),
+                "kp_regularization_grads received a null tensor");
+  const int64_t work = num_samples * num_kernel_points;
+  MCCNN_DIM_SWITCH(num_dims, hipLaunchKernelGGL(kp_regularization_grads_kernel<D>,
+                                                dim3(blocks_for(work, 256)), dim3(256), 0,
+                                                as_stream(stream), num_samples, num_kernel_points,
+                                                kind, sigma, loss_grad, points_in, points_out,
+                                                (const int2 *)neighbors, inv_radii, kernel_points,
+                                                offsets, argmin, offsets_grads_out));
   MCCNN_LAUNCH_CHECK();
   return MCCNN_OK;
 }

@@ -185,13 +185,85 @@ def _padded_basis_count(num_kernel_points):
     raise ValueError("at most 64 kernel points are supported")
 
 
+class _KPBasis(torch.autograd.Function):
+    """Kernel-point correlation weights per pair, zero-padded to `k` columns
+    (KPConv.py:29-57, 193-213); differentiable in the per-centre offsets."""
+
+    @staticmethod
+    def forward(ctx, offsets, points_in, points_out, neighbors, ranges, inv_radii,
+                kernel_points, k, kind, sigma):
+        kp, dims = kernel_points.shape
+        basis = torch.empty((neighbors.shape[0], k), dtype=_F32, device=points_in.device)
+        _lib.call("kp_basis", stream(), i64(neighbors.shape[0]), cint(dims), cint(kp), cint(k),
+                  cint(kind), cfloat(sigma), ptr(points_in, _F32), ptr(points_out, _F32),
+                  ptr(neighbors, _I32), ptr(inv_radii, _F32), ptr(kernel_points, _F32),
+                  ptr(offsets), ptr(basis), ptr(None))
+        ctx.save_for_backward(offsets, points_in, points_out, neighbors, ranges, inv_radii,
+                              kernel_points)
+        ctx.k, ctx.kind, ctx.sigma = k, kind, sigma
+        return basis
+
+    @staticmethod
+    def backward(ctx, grad):
+        (offsets, points_in, points_out, neighbors, ranges, inv_radii,
+         kernel_points) = ctx.saved_tensors
+        if offsets is None:
+            return (None,) * 10
+        kp, dims = kernel_points.shape
+        doff = torch.empty_like(offsets)
+        _lib.call("kp_basis_grads", stream(), i64(neighbors.shape[0]), cint(dims), cint(kp),
+                  cint(ctx.k), cint(ctx.kind), cfloat(ctx.sigma), ptr(points_in, _F32),
+                  ptr(points_out, _F32), ptr(neighbors, _I32), i64(ranges.shape[0]),
+                  ptr(ranges, _I32), ptr(inv_radii, _F32), ptr(kernel_points, _F32),
+                  ptr(offsets, _F32), ptr(grad.contiguous(), _F32), ptr(doff))
+        return (doff,) + (None,) * 9
+
+
+class _KPRegularization(torch.autograd.Function):
+    """sum(fit) + sum(repulsion) of the deformed kernel points (KPConv.py:394-429)."""
+
+    @staticmethod
+    def forward(ctx, offsets, points_in, points_out, neighbors, ranges, inv_radii,
+                kernel_points, kind, sigma):
+        kp, dims = kernel_points.shape
+        n_out = ranges.shape[0]
+        fit = torch.empty((n_out, kp), dtype=_F32, device=offsets.device)
+        rep = torch.empty((n_out, kp), dtype=_F32, device=offsets.device)
+        argmin = torch.empty((n_out, kp), dtype=_I32, device=offsets.device)
+        _lib.call("kp_regularization", stream(), i64(neighbors.shape[0]), cint(dims), cint(kp),
+                  cint(kind), cfloat(sigma), ptr(points_in, _F32), ptr(points_out, _F32),
+                  ptr(neighbors, _I32), i64(n_out), ptr(ranges, _I32), ptr(inv_radii, _F32),
+                  ptr(kernel_points, _F32), ptr(offsets, _F32), ptr(fit), ptr(argmin), ptr(rep))
+        ctx.save_for_backward(offsets, points_in, points_out, neighbors, inv_radii,
+                              kernel_points, argmin)
+        ctx.kind, ctx.sigma = kind, sigma
+        return fit.sum() + rep.sum()
+
+    @staticmethod
+    def backward(ctx, grad):
+        offsets, points_in, points_out, neighbors, inv_radii, kernel_points, argmin = \
+            ctx.saved_tensors
+        kp, dims = kernel_points.shape
+        doff = torch.empty_like(offsets)
+        _lib.call("kp_regularization_grads", stream(), i64(neighbors.shape[0]), cint(dims),
+                  cint(kp), cint(ctx.kind), cfloat(ctx.sigma), cfloat(1.0),
+                  ptr(points_in, _F32), ptr(points_out, _F32), ptr(neighbors, _I32),
+                  i64(offsets.shape[0]), ptr(inv_radii, _F32), ptr(kernel_points, _F32),
+                  ptr(offsets, _F32), ptr(argmin, _I32), ptr(doff))
+        return (doff * grad,) + (None,) * 8
+
+
 class KPConv(torch.nn.Module):
-    """Rigid kernel-point convolution (pylib/pc/layers/KPConv.py:60-315).  The
-    kernel points are scaled by 0.75 as in the reference (:131); `kernel_points`
-    is [K, D] in units of the convolution radius."""
+    """Kernel-point convolution, rigid or deformable
+    (pylib/pc/layers/KPConv.py:60-429).  The kernel points are scaled by 0.75 as
+    in the reference (:131); `kernel_points` is [K, D] in units of the convolution
+    radius.  With `deformable=True` a rigid kernel-point convolution predicts a
+    per-centre offset for every kernel point (:317-392) and
+    `regularization_loss()` returns the fitting + repulsive loss (:394-429)."""
 
     def __init__(self, num_features_in, num_features_out, kernel_points, num_dims=3,
-                 kernel_weighting="linear", weights=None, device="cuda", seed=0):
+                 kernel_weighting="linear", weights=None, deformable=False,
+                 offset_weights=None, device="cuda", seed=0):
         super().__init__()
         kp = torch.as_tensor(kernel_points, dtype=_F32).to(device) * 0.75
         self._kernel_points = kp.contiguous()
@@ -200,13 +272,30 @@ class KPConv(torch.nn.Module):
         self._kind = {"linear": 0, "gaussian": 1}[kernel_weighting]
         self._num_features_in, self._num_features_out = num_features_in, num_features_out
         self._num_dims = num_dims
-        if weights is None:      # Glorot normal as KPConv.py:133-160
-            gen = torch.Generator().manual_seed(seed)
-            fan_in, fan_out = self._num_kernel_points * num_features_in, num_features_out
-            weights = (torch.randn((fan_in, fan_out), generator=gen) *
-                       math.sqrt(2.0 / (fan_in + fan_out))).to(device)
+        gen = torch.Generator().manual_seed(seed)
+
+        def glorot(fan_in, fan_out):      # Glorot normal as KPConv.py:133-160
+            return (torch.randn((fan_in, fan_out), generator=gen) *
+                    math.sqrt(2.0 / (fan_in + fan_out))).to(device)
+
+        fan_in = self._num_kernel_points * num_features_in
+        if weights is None:
+            weights = glorot(fan_in, num_features_out)
         self.weights = torch.nn.Parameter(weights.to(_F32).contiguous())
+        self.deformable = deformable
+        if deformable:
+            if offset_weights is None:
+                offset_weights = glorot(fan_in, self._num_kernel_points * num_dims)
+            self.offset_weights = torch.nn.Parameter(offset_weights.to(_F32).contiguous())
         self.last_neighborhood = None
+        self._last = None
+
+    def _padded(self, w):
+        """[C*KP, F] -> [C*K, F] with zero rows for the padded basis columns."""
+        c, kp, k = self._num_features_in, self._num_kernel_points, self._num_basis
+        if k == kp:
+            return w
+        return torch.nn.functional.pad(w.reshape(c, kp, -1), (0, 0, 0, k - kp)).reshape(c * k, -1)
 
     def forward(self, features, point_cloud_in, point_cloud_out, conv_radius, neighborhood=None,
                 kernel_influence_dist=None):
@@ -218,26 +307,34 @@ class KPConv(torch.nn.Module):
             grid = pc.Grid(point_cloud_in, radii)
             neighborhood = pc.Neighborhood(grid, radii, point_cloud_out)
         self.last_neighborhood = neighborhood
-        ids = neighborhood._original_neigh_ids
-        kp, k = self._num_kernel_points, self._num_basis
-        basis = torch.empty((ids.shape[0], k), dtype=_F32, device=dev)
-        _lib.call("kp_basis", stream(), i64(ids.shape[0]), cint(d), cint(kp), cint(k), cint(self._kind),
-            cfloat(sigma), ptr(point_cloud_in._points, _F32), ptr(point_cloud_out._points, _F32),
-            ptr(ids, _I32), ptr(torch.reciprocal(radii), _F32), ptr(self._kernel_points, _F32),
-            ptr(None), ptr(basis), ptr(None))
+        ids, ranges = neighborhood._original_neigh_ids, neighborhood._samples_neigh_ranges
+        kp, k, c = self._num_kernel_points, self._num_basis, self._num_features_in
+        features = features.contiguous()
         transposed = None
-        if features.requires_grad and tfg_custom_ops.gathered_grads_supported(
-                self._num_features_in, k):
+        if features.requires_grad and tfg_custom_ops.gathered_grads_supported(c, k):
             transposed = neighborhood.transposed_pairs()
-        proj = tfg_custom_ops.basis_proj(basis, features.contiguous(), ids,
-                                         neighborhood._samples_neigh_ranges,
-                                         neighborhood._centre_order, transposed)
-        c = self._num_features_in
-        if k == kp:
-            return proj.reshape(-1, c * k) @ self.weights
-        # zero rows for the padded basis columns instead of slicing the projection
-        w = torch.nn.functional.pad(self.weights.reshape(c, kp, -1), (0, 0, 0, k - kp))
-        return proj.reshape(-1, c * k) @ w.reshape(c * k, -1)
+        geometry = (point_cloud_in._points, point_cloud_out._points, ids, ranges,
+                    torch.reciprocal(radii), self._kernel_points)
+
+        def project(basis):
+            return tfg_custom_ops.basis_proj(basis, features, ids, ranges,
+                                             neighborhood._centre_order, transposed)
+
+        offsets = None
+        if self.deformable:       # KPConv.py:317-392: offsets from a rigid convolution
+            rigid = _KPBasis.apply(None, *geometry, k, self._kind, sigma)
+            offsets = (project(rigid).reshape(-1, c * k) @ self._padded(self.offset_weights))
+            offsets = offsets.reshape(-1, kp, d).contiguous()
+        self._last = (offsets, geometry, sigma)
+        basis = _KPBasis.apply(offsets, *geometry, k, self._kind, sigma)
+        return project(basis).reshape(-1, c * k) @ self._padded(self.weights)
+
+    def regularization_loss(self):
+        """Fitting + repulsive loss of the last deformable call (KPConv.py:394-429)."""
+        if not self.deformable or self._last is None:
+            raise RuntimeError("regularization_loss needs a preceding deformable forward pass")
+        offsets, geometry, sigma = self._last
+        return _KPRegularization.apply(offsets, *geometry, self._kind, sigma)
 
 
 class _LocalPool(torch.autograd.Function):
