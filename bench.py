@@ -246,6 +246,8 @@ def main():
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--scale", type=float, default=1.0, help="shrink the point counts (tests)")
+    ap.add_argument("--fuse-final", action="store_true",
+                    help="run the product with the final weights inside the projection kernel")
     ap.add_argument("--no-cpu", action="store_true", help="skip the host-CPU baseline")
     ap.add_argument("--no-isolated", action="store_true", help="skip the isolated basis_proj case")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -282,7 +284,7 @@ def main():
     log("scene: %d points, %d pairs (mean %.1f per point), build %s" % (N, M, M / N, build_ms))
 
     conv = layers.MCConv(C, CO, D, num_mlps=1, mlp_size=[K], non_linearity_type="leaky_relu",
-                         seed=3)
+                         seed=3, fuse_final=args.fuse_final)
     gen = torch.Generator(device="cuda").manual_seed(3)
     feats = torch.randn((N, C), device="cuda", generator=gen).requires_grad_(True)
     up = torch.randn((N, CO), device="cuda", generator=gen)
@@ -308,12 +310,13 @@ def main():
 
     ops = {}
     for name, vals in per_op.items():
-        ms = sum(vals) / len(vals)
+        ms = sum(vals) / args.steps            # per step, over all calls of the op
+        calls = len(vals) / args.steps
         by = op_bytes(name, M, N, N, C, K, D)
-        ops[name] = {"ms": round(ms, 4)}
+        ops[name] = {"ms": round(ms, 4), "calls_per_step": calls}
         if by:
-            ops[name].update(GBps=round(by / ms / 1e6, 1),
-                             frac_hbm_peak=round(by / ms / 1e6 / HBM_PEAK_GBS, 4),
+            ops[name].update(GBps=round(by * calls / ms / 1e6, 1),
+                             frac_hbm_peak=round(by * calls / ms / 1e6 / HBM_PEAK_GBS, 4),
                              algorithmic_bytes=by)
     kernel_ms = sum(v["ms"] for v in ops.values())
     ops["dense_gemms_and_glue"] = {"ms": round(ms_per_step - kernel_ms, 4),

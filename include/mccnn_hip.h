@@ -242,6 +242,20 @@ int mccnn_transpose_neighbors(mccnn_stream_t stream, int64_t num_neighbors,
                               void *workspace, size_t workspace_bytes,
                               int32_t *point_ranges_out, int32_t *pair_order_out);
 
+/* The pair table regrouped for another order of the centres: slot q of the
+ * outputs holds the pairs of centre centre_order[q] (centre_order is a
+ * permutation of 0..num_samples-1), in their original order, with the centre
+ * column rewritten to q; ranges_out are the inclusive end offsets per slot.
+ * With centre_order = the centres sorted by grid cell this gives the table in
+ * which neighbouring slots share their neighbours, the layout the layer kernels
+ * run on.  No counterpart in the reference. */
+size_t mccnn_reorder_neighbors_workspace_bytes(int64_t num_samples);
+int mccnn_reorder_neighbors(mccnn_stream_t stream, int64_t num_samples,
+                            const int32_t *ranges, int64_t num_neighbors,
+                            const int32_t *neighbors, const int32_t *centre_order,
+                            void *workspace, size_t workspace_bytes,
+                            int32_t *ranges_out, int32_t *neighbors_out);
+
 /* BasisProjGrads without atomics: the feature gradient of each pair is written
  * to pair_rows_workspace [M, C] and then summed per point over the lists of
  * mccnn_transpose_neighbors, in a fixed order (bit-reproducible, unlike the
@@ -367,7 +381,11 @@ int mccnn_mc_basis_grads(mccnn_stream_t stream, int64_t num_neighbors,
  * is covered (D in {2,3}, K = 16, C in {16,32,64,128}); other shapes return
  * MCCNN_INVALID_ARGUMENT and must use the separate entry points.  The last three
  * inputs of the backward select the atomic-free feature gradient of
- * mccnn_basis_proj_grads_gathered (all NULL = atomics).  No
+ * mccnn_basis_proj_grads_gathered (all NULL = atomics); a NULL
+ * feature_grads_out skips the feature gradient (a layer obtains it without any
+ * scatter as the projection of its output gradient over the transposed pair
+ * table: mccnn_mc_conv_project with the roles of the two point sets swapped and
+ * negated inv_radii, followed by a product with the re-indexed weights).  No
  * counterpart among the reference's ops, which materialise the basis in
  * TensorFlow. */
 int mccnn_mc_conv_supported(int num_dims, int num_features, int num_basis);
@@ -390,6 +408,32 @@ int mccnn_mc_conv_project_grads(
     const int32_t *point_ranges, const int32_t *pair_order,
     float *pair_rows_workspace, float *feature_grads_out,
     float *weight_grads_out, float *bias_grads_out);
+
+/* The whole Monte-Carlo convolution (MCConv.py:137-194) in one kernel:
+ *   out[i, f] = sum_{c,k} proj[i, c, k] * final_weights[c*K + k, f]
+ * with proj as produced by mccnn_mc_conv_project; the projection is handed from
+ * the matrix-core accumulators to the final product through LDS and reaches HBM
+ * only when proj_out [N_out, C, K] is not NULL.  final_weights is the dense
+ * [C*K, F] matrix (several kernel MLPs: their [C*H, F/L] blocks placed on the
+ * block diagonal).  workspace holds the weights re-ordered for the kernel
+ * (mccnn_mc_conv_layer_workspace_bytes).  Covered shapes
+ * (mccnn_mc_conv_layer_supported): D in {2,3}, K = 16, C and F in
+ * {16,32,64,128}.  No counterpart among the reference's ops, which run the
+ * projection and tf.matmul separately. */
+int mccnn_mc_conv_layer_supported(int num_dims, int num_features, int num_basis,
+                                  int num_out_features);
+size_t mccnn_mc_conv_layer_workspace_bytes(int num_features, int num_basis,
+                                           int num_out_features);
+int mccnn_mc_conv_layer(mccnn_stream_t stream, int num_dims, int64_t num_pts,
+                        const float *points_in, int num_features,
+                        const float *features, int64_t num_samples,
+                        const float *points_out, int64_t num_neighbors,
+                        const int32_t *neighbors, const int32_t *ranges,
+                        const float *inv_radii, int num_basis, int num_mlps,
+                        int activation, const float *weights, const float *biases,
+                        const float *pdf, int num_out_features,
+                        const float *final_weights, void *workspace,
+                        size_t workspace_bytes, float *proj_out, float *out);
 
 /* Per-pair kernel-point weights, pylib/pc/layers/KPConv.py:29-57,193-213:
  *   d[m,k] = || delta_m - (kernel_points[k] + offsets[ctr_m,k]) ||

@@ -1,0 +1,96 @@
+// Kernel-MLP parameters shared by the fused Monte-Carlo convolution kernels.
+#pragma once
+#include "common.h"
+#include "mfma.h"
+
+namespace mccnn {
+
+constexpr int kFusedUnroll = 4;
+constexpr int kFusedK = 16;
+
+template <int D>
+struct McParams {
+  const float *pin;        // [N_in, D]
+  const float *pout;       // [N_out, D]
+  const float *inv_radii;  // [D]
+  const float *weights;    // [L, D, H]
+  const float *biases;     // [L*H]
+  const float *pdf;        // [M]
+  int hidden;              // H
+  int act;
+};
+
+// Weight column j of the flattened [D, L*H] kernel matrix.
+template <int D>
+__device__ __forceinline__ void load_weight_column(const McParams<D> &p, int j, float *w,
+                                                   float *bias) {
+  const int l = j / p.hidden, h = j - l * p.hidden;
+#pragma unroll
+  for (int d = 0; d < D; ++d) w[d] = p.weights[(l * D + d) * p.hidden + h];
+  *bias = p.biases[j];
+}
+
+// Per-wavefront LDS staging of one chunk of 64 pairs: lane n prepares pair n once
+// (offset to the neighbour, 1/pdf, neighbour feature row), and every matrix-core
+// step then fetches the four pairs it needs with two broadcast LDS reads instead
+// of recomputing them in each of the 16 lanes of a quarter.
+struct PairStage {
+  float4 geo[kWave];      // delta * inv_radii in x, y, z (z = 0 for D = 2), 1 / pdf in w
+  unsigned row[kWave];    // byte offset of the neighbour's feature row
+};
+
+// acc[j] += projection of the pairs [a, b) of one centre for the channels
+// col*kCPL + j of the 16*kCPL-channel chunk starting at feat_base.  Rows are
+// row_bytes apart; every byte offset fits 32 bits (checked by the host).
+template <int kCPL, int D>
+__device__ __forceinline__ void project_pairs(const char *__restrict__ feat_base,
+                                              unsigned row_bytes, const int2 *__restrict__ nbrs,
+                                              int a, int b, const McParams<D> &p,
+                                              const float *ctr, PairStage *stage, v4f *acc) {
+  const int lane = lane_id(), quarter = lane >> 4, col = lane & 15;
+  float wcol[3] = {0.0f, 0.0f, 0.0f}, ir[D], bcol;
+  load_weight_column<D>(p, col, wcol, &bcol);
+#pragma unroll
+  for (int d = 0; d < D; ++d) ir[d] = p.inv_radii[d];
+  const unsigned lane_off = col * kCPL * 4;
+  for (int m0 = a; m0 < b; m0 += kWave) {
+    const int cnt = b - m0 < kWave ? b - m0 : kWave;
+    float4 g = {0.0f, 0.0f, 0.0f, 0.0f};
+    unsigned row = 0;
+    if (lane < cnt) {
+      const int idx = nbrs[m0 + lane].x;
+      float dl[3] = {0.0f, 0.0f, 0.0f};
+#pragma unroll
+      for (int d = 0; d < D; ++d) dl[d] = (p.pin[(int64_t)idx * D + d] - ctr[d]) * ir[d];
+      g = make_float4(dl[0], dl[1], dl[2], 1.0f / p.pdf[m0 + lane]);
+      row = (unsigned)idx * row_bytes;
+    }
+    // unused slots of the last step point at the first pair's row with weight 0
+    const unsigned row0 = __builtin_amdgcn_readfirstlane(row);
+    stage->geo[lane] = g;
+    stage->row[lane] = lane < cnt ? row : row0;
+    const int steps = (cnt + 3) >> 2;
+    for (int t = 0; t < steps; t += kFusedUnroll) {
+      FVec<kCPL> f[kFusedUnroll];
+      float w[kFusedUnroll];
+#pragma unroll
+      for (int u = 0; u < kFusedUnroll; ++u) {
+        const int n = (4 * (t + u) + quarter) & (kWave - 1);
+        const float4 gn = stage->geo[n];
+        const unsigned rn = stage->row[n];
+        f[u] = load_vec<kCPL>(reinterpret_cast<const float *>(feat_base + rn + lane_off), true);
+        const float z = bcol + gn.x * wcol[0] + gn.y * wcol[1] + gn.z * wcol[2];
+        w[u] = act_fwd(p.act, z) * gn.w;
+      }
+#pragma unroll
+      for (int u = 0; u < kFusedUnroll; ++u)
+        if (t + u < steps) {
+#pragma unroll
+          for (int j = 0; j < kCPL; ++j)
+            acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(w[u], f[u].v[j], acc[j], 0, 0, 0);
+        }
+    }
+  }
+}
+
+}  // namespace mccnn

@@ -11,33 +11,9 @@
 #include "common.h"
 #include "fill.h"
 #include "mfma.h"
+#include "mc_conv.h"
 
 namespace mccnn {
-
-constexpr int kFusedUnroll = 4;
-constexpr int kFusedK = 16;
-
-template <int D>
-struct McParams {
-  const float *pin;        // [N_in, D]
-  const float *pout;       // [N_out, D]
-  const float *inv_radii;  // [D]
-  const float *weights;    // [L, D, H]
-  const float *biases;     // [L*H]
-  const float *pdf;        // [M]
-  int hidden;              // H
-  int act;
-};
-
-// Weight column j of the flattened [D, L*H] kernel matrix.
-template <int D>
-__device__ __forceinline__ void load_weight_column(const McParams<D> &p, int j, float *w,
-                                                   float *bias) {
-  const int l = j / p.hidden, h = j - l * p.hidden;
-#pragma unroll
-  for (int d = 0; d < D; ++d) w[d] = p.weights[(l * D + d) * p.hidden + h];
-  *bias = p.biases[j];
-}
 
 template <int kCPL, int D>
 __global__ void __launch_bounds__(256) mc_conv_project16_kernel(
@@ -53,49 +29,17 @@ __global__ void __launch_bounds__(256) mc_conv_project16_kernel(
   const int chunk = (int)(wid - centre * chunks);
   const int quarter = lane >> 4, col = lane & 15;
   const int a = centre > 0 ? ranges[centre - 1] : 0, b = ranges[centre];
-  const float *fbase = feat + chunk * kCW + col * kCPL;
-  float wcol[D], ctr[D], ir[D], bcol;
-  load_weight_column<D>(p, col, wcol, &bcol);
+  __shared__ PairStage stages[kWavesPerBlock];
+  float ctr[D];
 #pragma unroll
-  for (int d = 0; d < D; ++d) {
-    ctr[d] = p.pout[centre * D + d];
-    ir[d] = p.inv_radii[d];
-  }
+  for (int d = 0; d < D; ++d) ctr[d] = p.pout[centre * D + d];
   v4f acc[kCPL];
 #pragma unroll
   for (int j = 0; j < kCPL; ++j)
 #pragma unroll
     for (int r = 0; r < 4; ++r) acc[j][r] = 0.0f;
-
-  for (int m0 = a; m0 < b; m0 += kWave) {
-    const int cnt = b - m0 < kWave ? b - m0 : kWave;
-    const int myidx = nbrs[m0 + (lane < cnt ? lane : 0)].x;
-    const int steps = (cnt + 3) >> 2;
-    for (int t = 0; t < steps; t += kFusedUnroll) {
-      FVec<kCPL> f[kFusedUnroll];
-      float w[kFusedUnroll];
-#pragma unroll
-      for (int u = 0; u < kFusedUnroll; ++u) {
-        const int n = 4 * (t + u) + quarter;
-        const bool valid = n < cnt;
-        const int idx = __shfl(myidx, n & (kWave - 1), kWave);
-        f[u] = load_vec<kCPL>(fbase + (int64_t)idx * C, valid);
-        w[u] = 0.0f;
-        if (valid) {
-          float z = bcol;
-#pragma unroll
-          for (int d = 0; d < D; ++d)
-            z += (p.pin[(int64_t)idx * D + d] - ctr[d]) * ir[d] * wcol[d];
-          w[u] = act_fwd(p.act, z) / p.pdf[m0 + n];
-        }
-      }
-#pragma unroll
-      for (int u = 0; u < kFusedUnroll; ++u)
-#pragma unroll
-        for (int j = 0; j < kCPL; ++j)
-          acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(w[u], f[u].v[j], acc[j], 0, 0, 0);
-    }
-  }
+  project_pairs<kCPL, D>(reinterpret_cast<const char *>(feat + chunk * kCW), (unsigned)C * 4, nbrs,
+                         a, b, p, ctr, &stages[threadIdx.x / kWave], acc);
   float *o = out + centre * (int64_t)C * K + (int64_t)chunk * kCW * K + 4 * quarter;
 #pragma unroll
   for (int j = 0; j < kCPL; ++j)
@@ -314,7 +258,8 @@ extern "C" int mccnn_mc_conv_project(mccnn_stream_t stream, int num_dims, int64_
   int rc = check_fused_args("mc_conv_project", num_dims, num_features, num_basis, num_mlps,
                             activation, num_neighbors, num_samples);
   if (rc != MCCNN_OK) return rc;
-  MCCNN_REQUIRE(num_pts >= 0, "mc_conv_project expects a non-negative size");
+  MCCNN_REQUIRE(num_pts >= 0 && num_pts * num_features < ((int64_t)1 << 30),
+                "mc_conv_project expects a feature table of fewer than 2^30 elements");
   if (num_samples == 0) return MCCNN_OK;
   MCCNN_REQUIRE(ranges && out && points_out && inv_radii && weights && biases &&
                     (num_neighbors == 0 || (points_in && features && neighbors && pdf)),
@@ -377,8 +322,11 @@ extern "C" int mccnn_mc_conv_project_grads(
                     mccnn_mc_conv_project_grads_workspace_bytes(num_dims, num_basis),
                 "mc_conv_project_grads workspace too small");
   hipStream_t s = as_stream(stream);
-  if (num_pts > 0 && (!gathered || num_samples == 0 || num_neighbors == 0)) {
-    MCCNN_REQUIRE(feature_grads_out, "mc_conv_project_grads received a null tensor");
+  // A null feature_grads_out asks for the kernel-MLP gradients only.
+  const bool want_dfeat = feature_grads_out != nullptr;
+  MCCNN_REQUIRE(want_dfeat || !gathered,
+                "mc_conv_project_grads received a pair-row workspace but no feature gradient");
+  if (want_dfeat && num_pts > 0 && (!gathered || num_samples == 0 || num_neighbors == 0)) {
     rc = fill_zero(s, feature_grads_out, sizeof(float) * (size_t)num_pts * num_features);
     if (rc != MCCNN_OK) return rc;
   }
@@ -399,9 +347,10 @@ extern "C" int mccnn_mc_conv_project_grads(
     hipLaunchKernelGGL((mc_conv_project_grads16_kernel<C_, D_, true, false>), grid, block, 0,  \
                        s, num_samples, features, nb, ranges, prm, in_grads, feature_grads_out, \
                        pair_rows, (float *)workspace);                                         \
-    hipLaunchKernelGGL((mc_conv_project_grads16_kernel<C_, D_, false, true>), grid2, block, 0, \
-                       s, num_samples, features, nb, ranges, prm, in_grads, feature_grads_out, \
-                       pair_rows, (float *)workspace);                                         \
+    if (want_dfeat)                                                                            \
+      hipLaunchKernelGGL((mc_conv_project_grads16_kernel<C_, D_, false, true>), grid2, block,  \
+                         0, s, num_samples, features, nb, ranges, prm, in_grads,               \
+                         feature_grads_out, pair_rows, (float *)workspace);                    \
   }
 #define MCCNN_FUSED_BWD_D(C_) \
   if (num_dims == 3) MCCNN_FUSED_BWD(C_, 3) else MCCNN_FUSED_BWD(C_, 2)

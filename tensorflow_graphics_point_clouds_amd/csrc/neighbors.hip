@@ -185,6 +185,32 @@ static NbrWorkspace carve_nbr_workspace(void *ws, int d, int64_t ns) {
   return w;
 }
 
+// Pair table regrouped for another order of the centres: slot q takes the
+// segment of centre order[q].  counts pass, then (after the scan) a copy pass
+// with 16 lanes per slot; the centre column is rewritten to the slot.
+__global__ void __launch_bounds__(256) segment_counts_kernel(int64_t n, const int *__restrict__ ranges,
+                                                             const int *__restrict__ order,
+                                                             int *__restrict__ counts) {
+  const int64_t q = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (q >= n) return;
+  const int i = order[q];
+  counts[q] = ranges[i] - (i > 0 ? ranges[i - 1] : 0);
+}
+
+__global__ void __launch_bounds__(256) segment_copy_kernel(int64_t n, const int *__restrict__ ranges,
+                                                           const int *__restrict__ order,
+                                                           const int2 *__restrict__ pairs,
+                                                           const int *__restrict__ ranges_out,
+                                                           int2 *__restrict__ pairs_out) {
+  const int64_t q = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 4;
+  if (q >= n) return;
+  const int sub = threadIdx.x & 15;
+  const int i = order[q];
+  const int src = i > 0 ? ranges[i - 1] : 0, cnt = ranges[i] - src;
+  const int dst = ranges_out[q] - cnt;
+  for (int t = sub; t < cnt; t += 16) pairs_out[dst + t] = make_int2(pairs[src + t].x, (int)q);
+}
+
 }  // namespace mccnn
 
 using namespace mccnn;
@@ -291,6 +317,41 @@ extern "C" int mccnn_find_neighbors_fill(
                                                 num_samples, samples, points,
                                                 (const int2 *)w.ranges, inv_radii, max_neighs,
                                                 (int *)nullptr, ranges, (int2 *)neighbors_out));
+  MCCNN_LAUNCH_CHECK();
+  return MCCNN_OK;
+}
+
+extern "C" size_t mccnn_reorder_neighbors_workspace_bytes(int64_t num_samples) {
+  if (num_samples < 0) return 0;
+  return align256(sizeof(int) * scan_scratch_ints(num_samples)) + align256(sizeof(int64_t));
+}
+
+extern "C" int mccnn_reorder_neighbors(mccnn_stream_t stream, int64_t num_samples,
+                                       const int32_t *ranges, int64_t num_neighbors,
+                                       const int32_t *neighbors, const int32_t *centre_order,
+                                       void *workspace, size_t workspace_bytes,
+                                       int32_t *ranges_out, int32_t *neighbors_out) {
+  MCCNN_REQUIRE(num_samples >= 0 && num_neighbors >= 0 && num_neighbors < ((int64_t)1 << 31),
+                "reorder_neighbors expects sizes in [0, 2^31)");
+  if (num_samples == 0) return MCCNN_OK;
+  MCCNN_REQUIRE(ranges && centre_order && ranges_out && workspace &&
+                    (num_neighbors == 0 || (neighbors && neighbors_out)),
+                "reorder_neighbors received a null tensor");
+  MCCNN_REQUIRE(workspace_bytes >= mccnn_reorder_neighbors_workspace_bytes(num_samples),
+                "reorder_neighbors workspace too small");
+  hipStream_t s = as_stream(stream);
+  int *scratch = (int *)workspace;
+  int64_t *total = (int64_t *)((char *)workspace +
+                               align256(sizeof(int) * scan_scratch_ints(num_samples)));
+  hipLaunchKernelGGL(segment_counts_kernel, dim3(blocks_for(num_samples, 256)), dim3(256), 0, s,
+                     num_samples, ranges, centre_order, ranges_out);
+  MCCNN_LAUNCH_CHECK();
+  int rc = inclusive_scan_i32(s, num_samples, ranges_out, scratch, total);
+  if (rc != MCCNN_OK) return rc;
+  if (num_neighbors == 0) return MCCNN_OK;
+  hipLaunchKernelGGL(segment_copy_kernel, dim3(blocks_for(num_samples * 16, 256)), dim3(256), 0, s,
+                     num_samples, ranges, centre_order, (const int2 *)neighbors, ranges_out,
+                     (int2 *)neighbors_out);
   MCCNN_LAUNCH_CHECK();
   return MCCNN_OK;
 }

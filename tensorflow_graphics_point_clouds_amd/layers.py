@@ -97,6 +97,142 @@ class _MCConvProject(torch.autograd.Function):
         return dw, db, dfeat, None, None, None, None, None, None, None, None
 
 
+def _mc_project(weights, biases, features, points_in, points_out, neighbors, ranges, inv_radii,
+                pdf, act):
+    num_mlps, dims, hidden = weights.shape
+    k = num_mlps * hidden
+    out = torch.empty((ranges.shape[0], features.shape[1], k), dtype=_F32,
+                      device=features.device)
+    _lib.call("mc_conv_project", stream(), cint(dims), i64(features.shape[0]),
+              ptr(points_in, _F32), cint(features.shape[1]), ptr(features, _F32),
+              i64(ranges.shape[0]), ptr(points_out, _F32), i64(neighbors.shape[0]),
+              ptr(neighbors, _I32), ptr(ranges, _I32), ptr(inv_radii, _F32), cint(k),
+              cint(num_mlps), cint(act), ptr(weights, _F32), ptr(biases, _F32),
+              ptr(pdf, _F32), ptr(out))
+    return out
+
+
+def _mc_layer(weights, biases, features, points_in, points_out, neighbors, ranges, inv_radii,
+              pdf, act, dense_weights, want_proj=False):
+    """Fused projection + product with the dense [C*K, F] final weights."""
+    num_mlps, dims, hidden = weights.shape
+    k, c, f = num_mlps * hidden, features.shape[1], dense_weights.shape[1]
+    L = _lib.lib()
+    L.mccnn_mc_conv_layer_workspace_bytes.restype = _lib.csize
+    ws = _lib.workspace(L.mccnn_mc_conv_layer_workspace_bytes(cint(c), cint(k), cint(f)),
+                        features.device)
+    out = torch.empty((ranges.shape[0], f), dtype=_F32, device=features.device)
+    proj = None
+    if want_proj:
+        proj = torch.empty((ranges.shape[0], c, k), dtype=_F32, device=features.device)
+    _lib.call("mc_conv_layer", stream(), cint(dims), i64(features.shape[0]),
+              ptr(points_in, _F32), cint(c), ptr(features, _F32), i64(ranges.shape[0]),
+              ptr(points_out, _F32), i64(neighbors.shape[0]), ptr(neighbors, _I32),
+              ptr(ranges, _I32), ptr(inv_radii, _F32), cint(k), cint(num_mlps), cint(act),
+              ptr(weights, _F32), ptr(biases, _F32), ptr(pdf, _F32), cint(f),
+              ptr(dense_weights.contiguous(), _F32), ptr(ws), _lib.csize(ws.numel()), ptr(proj),
+              ptr(out))
+    return out, proj
+
+
+def _dense_final_weights(final_weights, c):
+    """[L, C*H, G] per-MLP blocks -> dense [C*(L*H), L*G] with zero off-diagonal blocks."""
+    l, ch, g = final_weights.shape
+    if l == 1:
+        return final_weights[0]
+    h = ch // c
+    dense = torch.zeros((c, l, h, l, g), dtype=_F32, device=final_weights.device)
+    blocks = final_weights.reshape(l, c, h, g)
+    for i in range(l):
+        dense[:, i, :, i, :] = blocks[i]
+    return dense.reshape(c * l * h, l * g)
+
+
+class _MCConvLayer(torch.autograd.Function):
+    """The whole Monte-Carlo convolution (MCConv.py:137-194), run on the
+    neighbourhood's grid-ordered view (features and output gradients are permuted
+    into grid order once per pass so that the gathers of neighbouring centres hit
+    in L2).  Forward: fused basis + projection, product with the final weights
+    (inside the same kernel with `fuse_final`).  Backward: the feature gradient
+    is the same convolution run from the centres back to the points over the
+    transposed pair table (no scatter):
+        Q[j, f, k]  = sum_{i in T(j)} basis[ij, k] dout[i, f]
+        dfeat[j, c] = sum_{f,k} Q[j, f, k] W[c, k, f]
+        dW[c, k, f] = sum_j feat[j, c] Q[j, f, k]
+    and the kernel-MLP gradients come from dproj = dout W^T through the weight
+    half of the fused projection backward."""
+
+    @staticmethod
+    def forward(ctx, weights, biases, final_weights, features, neighborhood, inv_radii, act,
+                fuse_final):
+        view = neighborhood.sorted_view()
+        pdf, _ = view.pair_pdf(neighborhood)
+        feats = features.index_select(0, view.point_order)
+        dense = _dense_final_weights(final_weights, features.shape[1])
+        if fuse_final:
+            out, _ = _mc_layer(weights, biases, feats, view.points_in, view.points_out,
+                               view.table, view.ranges, inv_radii, pdf, act, dense)
+        else:
+            proj = _mc_project(weights, biases, feats, view.points_in, view.points_out,
+                               view.table, view.ranges, inv_radii, pdf, act)
+            out = proj.reshape(proj.shape[0], -1) @ dense
+        if view.centre_order is not None:
+            out = torch.empty_like(out).index_copy_(0, view.centre_order, out)
+        ctx.save_for_backward(weights, biases, final_weights, feats, inv_radii)
+        ctx.neighborhood, ctx.act, ctx.fuse_final = neighborhood, act, fuse_final
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        weights, biases, final_weights, feats, inv_radii = ctx.saved_tensors
+        nbh = ctx.neighborhood
+        view = nbh.sorted_view()
+        pdf, pdf_t = view.pair_pdf(nbh)
+        l, dims, h = weights.shape
+        k, n, c = l * h, view.ranges.shape[0], feats.shape[1]
+        g = final_weights.shape[2]
+        f = g * l
+        if view.centre_order is not None:
+            dout = dout.index_select(0, view.centre_order)
+        else:
+            dout = dout.contiguous()
+        dense = _dense_final_weights(final_weights, c)               # [C*K, F]
+        # kernel-MLP gradients
+        dproj = dout @ dense.t()
+        L = _lib.lib()
+        ws = _lib.workspace(L.mccnn_mc_conv_project_grads_workspace_bytes(cint(dims), cint(k)),
+                            weights.device)
+        dw, db = torch.empty_like(weights), torch.empty_like(biases)
+        _lib.call("mc_conv_project_grads", stream(), cint(dims), i64(feats.shape[0]),
+                  ptr(view.points_in, _F32), cint(c), ptr(feats, _F32), i64(n),
+                  ptr(view.points_out, _F32), i64(view.table.shape[0]), ptr(view.table, _I32),
+                  ptr(view.ranges, _I32), ptr(inv_radii, _F32), cint(k), cint(l), cint(ctx.act),
+                  ptr(weights, _F32), ptr(biases, _F32), ptr(pdf, _F32), ptr(dproj, _F32),
+                  ptr(ws), _lib.csize(ws.numel()), ptr(None), ptr(None), ptr(None), ptr(None),
+                  ptr(dw), ptr(db))
+        del dproj
+        # feature and final-weight gradients from the transposed convolution
+        w2 = dense.reshape(c, k, f).permute(2, 1, 0).reshape(f * k, c)
+        neg = -inv_radii
+        if ctx.fuse_final:
+            dfeat, q = _mc_layer(weights, biases, dout, view.points_out, view.points_in,
+                                 view.table_t, view.ranges_t, neg, pdf_t, ctx.act, w2,
+                                 want_proj=True)
+        else:
+            q = _mc_project(weights, biases, dout, view.points_out, view.points_in,
+                            view.table_t, view.ranges_t, neg, pdf_t, ctx.act)
+            dfeat = q.reshape(q.shape[0], f * k) @ w2
+        ddense = (feats.t() @ q.reshape(feats.shape[0], f * k)).reshape(c, f, k)
+        ddense = ddense.permute(0, 2, 1)                              # [C, K, F]
+        if l == 1:
+            dfinal = ddense.reshape(1, c * k, f)
+        else:
+            blocks = ddense.reshape(c, l, h, l, g)
+            dfinal = torch.stack([blocks[:, i, :, i, :].reshape(c * h, g) for i in range(l)])
+        dfeat = torch.empty_like(dfeat).index_copy_(0, view.point_order, dfeat)
+        return dw, db, dfinal, dfeat, None, None, None, None
+
+
 def _truncated_normal(shape, std, generator, device):
     t = torch.empty(shape, dtype=_F32)
     torch.nn.init.trunc_normal_(t, mean=0.0, std=std, a=-2 * std, b=2 * std,
@@ -110,7 +246,8 @@ class MCConv(torch.nn.Module):
 
     def __init__(self, num_features_in, num_features_out, num_dims, num_mlps=4, mlp_size=(8,),
                  non_linearity_type="leaky_relu", weights=None, biases=None,
-                 final_weights=None, device="cuda", seed=0, fused=True, gathered_grads=True):
+                 final_weights=None, device="cuda", seed=0, fused=True, gathered_grads=True,
+                 transposed_grads=True, fuse_final=False):
         super().__init__()
         if num_features_out % num_mlps != 0:
             raise ValueError("The number of output features must be divisible by the number"
@@ -139,6 +276,10 @@ class MCConv(torch.nn.Module):
         self.fused = fused
         # feature gradient by per-pair rows + ordered gather instead of float atomics
         self.gathered_grads = gathered_grads
+        # feature gradient as a convolution over the transposed pair table (fused path)
+        self.transposed_grads = transposed_grads
+        # product with the final weights inside the projection kernel (out of LDS)
+        self.fuse_final = fuse_final
 
     def forward(self, features, point_cloud_in, point_cloud_out, radius, neighborhood=None,
                 bandwidth=0.2):
@@ -152,12 +293,18 @@ class MCConv(torch.nn.Module):
         pdf = neighborhood.get_pdf(bandwidth=bandwidth, mode=pc.KDEMode.constant)
         biases = self.biases.reshape(self._num_mlps, self._hidden)
         k = self._num_mlps * self._hidden
+        fused = self.fused and _lib.lib().mccnn_mc_conv_supported(
+            cint(d), cint(self._num_features_in), cint(k))
+        if fused and self.transposed_grads and _lib.lib().mccnn_mc_conv_layer_supported(
+                cint(d), cint(self._num_features_in), cint(k), cint(self._num_features_out)):
+            return _MCConvLayer.apply(self.weights, biases, self.final_weights, features,
+                                      neighborhood, torch.reciprocal(radii), self._act,
+                                      self.fuse_final)
         transposed = None
         if self.gathered_grads and features.requires_grad and \
                 tfg_custom_ops.gathered_grads_supported(self._num_features_in, k):
             transposed = neighborhood.transposed_pairs()
-        if self.fused and _lib.lib().mccnn_mc_conv_supported(cint(d), cint(self._num_features_in),
-                                                             cint(k)):
+        if fused:
             proj = _MCConvProject.apply(self.weights, biases, features.contiguous(),
                                         point_cloud_in._points, point_cloud_out._points,
                                         neighborhood._original_neigh_ids,

@@ -99,6 +99,69 @@ class Grid:
         return self._fast_DS
 
 
+class _SortedView:
+    """A neighbourhood with input points and centres both numbered in grid-cell
+    order, the layout the layer kernels run on: consecutive centres then share
+    their neighbours and every neighbour list is a few contiguous index runs, so
+    the feature gathers hit in L2 instead of walking the whole table at random.
+
+    points_in / points_out   coordinates in that order
+    point_order [N_in]       position -> original point id (the grid's sort)
+    centre_order [N_out]     slot -> original centre id, None if the centres
+                             already are the grid's sorted points
+    table [M,2], ranges      pairs (point position, centre slot) grouped by slot
+    table_t [M,2], ranges_t  pairs (centre slot, point position) grouped by point
+    """
+
+    def __init__(self, nbh):
+        grid, samples = nbh._grid, nbh._point_cloud_sampled
+        self.points_in = grid._sorted_points
+        self.point_order = grid._sorted_indices.long()
+        n_out = samples._points.shape[0]
+        if nbh._equal_samples:
+            self.centre_order = None
+            self.points_out = grid._sorted_points
+            self.table, self.ranges = nbh._neighbors, nbh._samples_neigh_ranges
+        else:
+            if samples is grid._point_cloud:
+                order = grid._sorted_indices
+                self.points_out = grid._sorted_points
+            else:
+                order = nbh.compute_centre_order()
+                self.points_out = samples._points[order.long()].contiguous()
+            self.centre_order = order.long()
+            L = _lib.lib()
+            L.mccnn_reorder_neighbors_workspace_bytes.restype = _lib.csize
+            dev = nbh._neighbors.device
+            ws = _lib.workspace(L.mccnn_reorder_neighbors_workspace_bytes(i64(n_out)), dev)
+            self.ranges = torch.empty_like(nbh._samples_neigh_ranges)
+            self.table = torch.empty_like(nbh._neighbors)
+            _lib.call("reorder_neighbors", stream(), i64(n_out),
+                      ptr(nbh._samples_neigh_ranges, _I32), i64(nbh._neighbors.shape[0]),
+                      ptr(nbh._neighbors, _I32), ptr(order, _I32), ptr(ws),
+                      _lib.csize(ws.numel()), ptr(self.ranges), ptr(self.table))
+        self.ranges_t, pair_order = tfg_custom_ops.transpose_neighbors(
+            self.table, self.points_in.shape[0])
+        sel = pair_order.long()
+        self.table_t = torch.stack((self.table[sel, 1], self.table[sel, 0]), dim=1).contiguous()
+        self._pdf_key, self.pdf, self.pdf_t = None, None, None
+
+    def pair_pdf(self, nbh):
+        """Per-pair densities of `table` and `table_t` (the neighbour point's)."""
+        per_point = nbh._pdf_per_point
+        key = None if per_point is None else (per_point.data_ptr(), per_point._version)
+        if self.pdf is None or key != self._pdf_key:
+            m, dev = self.table.shape[0], self.table.device
+            if per_point is None:
+                self.pdf = self.pdf_t = torch.ones(m, dtype=_F32, device=dev)
+            else:
+                per_point = per_point.detach()
+                self.pdf = per_point[self.table[:, 0].long()].contiguous()
+                self.pdf_t = per_point[self.table_t[:, 1].long()].contiguous()
+            self._pdf_key = key
+        return self.pdf, self.pdf_t
+
+
 class Neighborhood:
     """Neighbour pairs of the centres `point_cloud_sample` (default: the grid's
     own sorted points) inside `grid` (pylib/pc/Neighborhood.py:218-311)."""
@@ -131,6 +194,9 @@ class Neighborhood:
         # optional visiting order of the centres for the projection kernels
         self._centre_order = None
         self._transposed_pairs = None
+        self._transposed_table = None
+        self._transposed_pdf = None
+        self._sorted_view = None
 
     def transposed_pairs(self):
         """(point_ranges, pair_order): the pairs grouped by neighbour point, used by
@@ -139,6 +205,33 @@ class Neighborhood:
             self._transposed_pairs = tfg_custom_ops.transpose_neighbors(
                 self._original_neigh_ids, self._grid._point_cloud._points.shape[0])
         return self._transposed_pairs
+
+    def transposed_table(self, pdf=None):
+        """The pair table seen from the neighbour points: rows (centre, point) sorted
+        by point with inclusive end offsets per point, and `pdf` (per pair) in the same
+        order.  A convolution over this table carries values from the centres back
+        to the points (Neighborhood.py:313-329 builds the same view); the layers use
+        it for their feature gradients.  Built on first use and kept."""
+        point_ranges, pair_order = self.transposed_pairs()
+        if self._transposed_table is None:
+            order = pair_order.long()
+            ids = self._original_neigh_ids
+            self._transposed_table = torch.stack((ids[order, 1], ids[order, 0]),
+                                                 dim=1).contiguous()
+        pdf_t = None
+        if pdf is not None:
+            key = (pdf.data_ptr(), pdf._version)
+            if self._transposed_pdf is None or self._transposed_pdf[0] != key:
+                self._transposed_pdf = (key, pdf[pair_order.long()].contiguous())
+            pdf_t = self._transposed_pdf[1]
+        return self._transposed_table, point_ranges, pdf_t
+
+    def sorted_view(self):
+        """The neighbourhood re-expressed in grid order on both sides (built on
+        first use and kept): see `_SortedView`."""
+        if self._sorted_view is None:
+            self._sorted_view = _SortedView(self)
+        return self._sorted_view
 
     def compute_centre_order(self):
         """Rank the centres by their cell key in the grid (a scheduling hint for

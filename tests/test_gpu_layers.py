@@ -34,14 +34,17 @@ _T_ACT = {"relu": torch.relu, "leaky_relu": lambda x: torch.nn.functional.leaky_
           "elu": torch.nn.functional.elu}
 
 
-@pytest.mark.parametrize("fused,gathered", [(True, True), (True, False), (False, True),
-                                            (False, False)])
+@pytest.mark.parametrize("fused,gathered,transposed,fuse_final",
+                         [(True, True, True, True), (True, True, True, False),
+                          (True, True, False, False), (True, False, False, False),
+                          (False, True, False, False), (False, False, False, False)])
 @pytest.mark.parametrize("c_in,c_out,hidden,num_mlps,act",
                          [(8, 16, 16, 1, "relu"), (3, 8, 8, 1, "leaky_relu"),
                           (16, 32, 8, 4, "elu"), (64, 64, 16, 1, "leaky_relu"),
                           (32, 16, 8, 2, "relu"), (16, 8, 16, 1, "elu"),
                           (128, 32, 16, 1, "leaky_relu")])
-def test_mcconv_forward_backward(oracle, c_in, c_out, hidden, num_mlps, act, fused, gathered):
+def test_mcconv_forward_backward(oracle, c_in, c_out, hidden, num_mlps, act, fused, gathered,
+                                 transposed, fuse_final):
     from tensorflow_graphics_point_clouds_amd import layers, pc, synthetic
     rng = np.random.default_rng(c_in + hidden)
     batch, radius = 2, 0.15
@@ -55,7 +58,8 @@ def test_mcconv_forward_backward(oracle, c_in, c_out, hidden, num_mlps, act, fus
 
     conv = layers.MCConv(c_in, c_out, 3, num_mlps=num_mlps, mlp_size=[hidden],
                          non_linearity_type=act, weights=dev(w), biases=dev(b),
-                         final_weights=dev(wo), fused=fused, gathered_grads=gathered)
+                         final_weights=dev(wo), fused=fused, gathered_grads=gathered,
+                         transposed_grads=transposed, fuse_final=fuse_final)
     tfeat = dev(feat).requires_grad_(True)
     out = conv(tfeat, pc.PointCloud(dev(pts), dev(bids), batch),
                pc.PointCloud(dev(ctr), dev(cb), batch), radius, bandwidth=0.2)
