@@ -39,10 +39,20 @@ struct PairStage {
   unsigned row[kWave];    // byte offset of the neighbour's feature row
 };
 
+// The activation is a template parameter of the fused kernels: with a run-time
+// selector the compiler evaluates all three (including the exponential of ELU)
+// for every pair and selects afterwards.
+#define MCCNN_ACT_SWITCH(act_, ...)                                   \
+  switch (act_) {                                                     \
+    case MCCNN_ACT_RELU: { constexpr int ACT = MCCNN_ACT_RELU; __VA_ARGS__; } break;             \
+    case MCCNN_ACT_LEAKY_RELU: { constexpr int ACT = MCCNN_ACT_LEAKY_RELU; __VA_ARGS__; } break; \
+    default: { constexpr int ACT = MCCNN_ACT_ELU; __VA_ARGS__; } break;                          \
+  }
+
 // acc[j] += projection of the pairs [a, b) of one centre for the channels
 // col*kCPL + j of the 16*kCPL-channel chunk starting at feat_base.  Rows are
 // row_bytes apart; every byte offset fits 32 bits (checked by the host).
-template <int kCPL, int D>
+template <int kCPL, int D, int kAct>
 __device__ __forceinline__ void project_pairs(const char *__restrict__ feat_base,
                                               unsigned row_bytes, const int2 *__restrict__ nbrs,
                                               int a, int b, const McParams<D> &p,
@@ -80,7 +90,7 @@ __device__ __forceinline__ void project_pairs(const char *__restrict__ feat_base
         const unsigned rn = stage->row[n];
         f[u] = load_vec<kCPL>(reinterpret_cast<const float *>(feat_base + rn + lane_off), true);
         const float z = bcol + gn.x * wcol[0] + gn.y * wcol[1] + gn.z * wcol[2];
-        w[u] = act_fwd(p.act, z) * gn.w;
+        w[u] = act_fwd(kAct, z) * gn.w;
       }
 #pragma unroll
       for (int u = 0; u < kFusedUnroll; ++u)

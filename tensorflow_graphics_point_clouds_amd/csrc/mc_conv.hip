@@ -15,7 +15,7 @@
 
 namespace mccnn {
 
-template <int kCPL, int D>
+template <int kCPL, int D, int kAct>
 __global__ void __launch_bounds__(256) mc_conv_project16_kernel(
     int64_t n_out, int C, int chunks, const float *__restrict__ feat,
     const int2 *__restrict__ nbrs, const int *__restrict__ ranges, McParams<D> p,
@@ -38,7 +38,7 @@ __global__ void __launch_bounds__(256) mc_conv_project16_kernel(
   for (int j = 0; j < kCPL; ++j)
 #pragma unroll
     for (int r = 0; r < 4; ++r) acc[j][r] = 0.0f;
-  project_pairs<kCPL, D>(reinterpret_cast<const char *>(feat + chunk * kCW), (unsigned)C * 4, nbrs,
+  project_pairs<kCPL, D, kAct>(reinterpret_cast<const char *>(feat + chunk * kCW), (unsigned)C * 4, nbrs,
                          a, b, p, ctr, &stages[threadIdx.x / kWave], acc);
   float *o = out + centre * (int64_t)C * K + (int64_t)chunk * kCW * K + 4 * quarter;
 #pragma unroll
@@ -61,7 +61,7 @@ constexpr int kFusedGradBlocks = 2048;
 // kDB / kDF select the two halves (weight-gradient half, feature-gradient half);
 // launching them as two kernels keeps each under ~90 registers, which more than
 // pays for reading the upstream gradient twice.
-template <int C, int D, bool kDB, bool kDF>
+template <int C, int D, int kAct, bool kDB, bool kDF>
 __global__ void __launch_bounds__(256) mc_conv_project_grads16_kernel(
     int64_t n_out, const float *__restrict__ feat, const int2 *__restrict__ nbrs,
     const int *__restrict__ ranges, McParams<D> p, const float *__restrict__ in_grad,
@@ -124,8 +124,8 @@ __global__ void __launch_bounds__(256) mc_conv_project_grads16_kernel(
         float z = wr[D];
 #pragma unroll
         for (int d = 0; d < D; ++d) z += delta[d] * wr[d];
-        basis4[r] = valid ? act_fwd(p.act, z) * inv_pdf : 0.0f;
-        dact4[r] = act_bwd(p.act, z) * inv_pdf;
+        basis4[r] = valid ? act_fwd(kAct, z) * inv_pdf : 0.0f;
+        dact4[r] = act_bwd(kAct, z) * inv_pdf;
       }
       if (kDB) {
         v4f acc = {0.0f, 0.0f, 0.0f, 0.0f};
@@ -200,6 +200,127 @@ __global__ void __launch_bounds__(256) mc_conv_project_grads16_kernel(
   }
 }
 
+// Kernel-MLP gradients alone (the layer obtains its feature gradient from the
+// transposed convolution).  Persistent wavefronts, as many as fit on the device,
+// stride over the centres.  Per centre the upstream tile G [C x 16] sits in
+// registers as the A operand; per chunk of 64 pairs lane n stages pair n in LDS
+// (offset, 1/pdf, feature row), then every tile of 16 pairs takes 16*C/64 matrix
+// steps for dbasis^T [k x pair] while the feature rows of the next tile are
+// already in flight, and the result is folded in registers into
+//   dW[d][k] += delta_d * dz,  db[k] += dz,  dz = dbasis * act'(z) / pdf.
+template <int C, int D, int kAct>
+__global__ void __launch_bounds__(256) mc_conv_weight_grads16_kernel(
+    int64_t n_out, const float *__restrict__ feat, const int2 *__restrict__ nbrs,
+    const int *__restrict__ ranges, McParams<D> p, const float *__restrict__ in_grad,
+    float *__restrict__ partials) {
+  constexpr int K = kFusedK;
+  constexpr int kQuarterC = C / 4;
+  __shared__ float red[kWavesPerBlock][(D + 1) * K];
+  __shared__ float4 wlds[K];               // column j: weights (z = 0 for D = 2), bias in w
+  __shared__ PairStage stages[kWavesPerBlock];
+  const int lane = lane_id(), wave = threadIdx.x / kWave;
+  const int quarter = lane >> 4, col = lane & 15;
+  if (threadIdx.x < K) {
+    float w[3] = {0.0f, 0.0f, 0.0f}, bias;
+    load_weight_column<D>(p, threadIdx.x, w, &bias);
+    wlds[threadIdx.x] = make_float4(w[0], w[1], w[2], bias);
+  }
+  __syncthreads();
+  PairStage *stage = &stages[wave];
+  float ir[D];
+#pragma unroll
+  for (int d = 0; d < D; ++d) ir[d] = p.inv_radii[d];
+  float dw[4][3], db[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    db[r] = 0.0f;
+#pragma unroll
+    for (int d = 0; d < 3; ++d) dw[r][d] = 0.0f;
+  }
+  const char *feat_lane = reinterpret_cast<const char *>(feat + quarter * kQuarterC);
+  const int64_t total_waves = (int64_t)gridDim.x * kWavesPerBlock;
+  for (int64_t centre = wave_slot(); centre < n_out; centre += total_waves) {
+    const int a = centre > 0 ? ranges[centre - 1] : 0, b = ranges[centre];
+    if (b <= a) continue;
+    const float *gi = in_grad + centre * (int64_t)C * K;
+    float gk[kQuarterC];
+#pragma unroll
+    for (int s = 0; s < kQuarterC; ++s) gk[s] = gi[(quarter * kQuarterC + s) * K + col];
+    float ctr[D];
+#pragma unroll
+    for (int d = 0; d < D; ++d) ctr[d] = p.pout[centre * D + d];
+
+    for (int m0 = a; m0 < b; m0 += kWave) {
+      const int cnt = b - m0 < kWave ? b - m0 : kWave;
+      float4 g = {0.0f, 0.0f, 0.0f, 0.0f};
+      unsigned row = 0;
+      if (lane < cnt) {
+        const int idx = nbrs[m0 + lane].x;
+        float dl[3] = {0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int d = 0; d < D; ++d) dl[d] = (p.pin[(int64_t)idx * D + d] - ctr[d]) * ir[d];
+        g = make_float4(dl[0], dl[1], dl[2], 1.0f / p.pdf[m0 + lane]);
+        row = (unsigned)idx * (unsigned)(C * 4);
+      }
+      const unsigned row0 = __builtin_amdgcn_readfirstlane(row);
+      stage->geo[lane] = g;
+      stage->row[lane] = lane < cnt ? row : row0;
+      const int tiles = (cnt + 15) >> 4;
+      FVec<kQuarterC> f = load_vec<kQuarterC>(
+          reinterpret_cast<const float *>(feat_lane + stage->row[col]), true);
+      for (int t = 0; t < tiles; ++t) {
+        FVec<kQuarterC> fn = f;
+        if (t + 1 < tiles)
+          fn = load_vec<kQuarterC>(
+              reinterpret_cast<const float *>(feat_lane + stage->row[16 * (t + 1) + col]), true);
+        const float4 geo = stage->geo[16 * t + col];
+        v4f acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int s = 0; s < kQuarterC; ++s)
+          acc = __builtin_amdgcn_mfma_f32_16x16x4f32(gk[s], f.v[s], acc, 0, 0, 0);
+        // acc[r] = dbasis[pair col][k = 4*quarter + r]
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const float4 wr = wlds[4 * quarter + r];
+          const float z = wr.w + geo.x * wr.x + geo.y * wr.y + geo.z * wr.z;
+          const float dz = acc[r] * act_bwd(kAct, z) * geo.w;
+          db[r] += dz;
+          dw[r][0] += geo.x * dz;
+          dw[r][1] += geo.y * dz;
+          if (D > 2) dw[r][2] += geo.z * dz;
+        }
+        f = fn;
+      }
+    }
+  }
+  // reduce over the 16 pair-lanes of each quarter
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+#pragma unroll
+    for (int off = 8; off > 0; off >>= 1) {
+      db[r] += __shfl_xor(db[r], off, kWave);
+#pragma unroll
+      for (int d = 0; d < D; ++d) dw[r][d] += __shfl_xor(dw[r][d], off, kWave);
+    }
+  }
+  if (col == 0) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int k = 4 * quarter + r;
+#pragma unroll
+      for (int d = 0; d < D; ++d) red[wave][d * K + k] = dw[r][d];
+      red[wave][D * K + k] = db[r];
+    }
+  }
+  __syncthreads();
+  if (threadIdx.x < (D + 1) * K) {
+    float s = 0.0f;
+#pragma unroll
+    for (int w = 0; w < kWavesPerBlock; ++w) s += red[w][threadIdx.x];
+    partials[(int64_t)blockIdx.x * (D + 1) * K + threadIdx.x] = s;
+  }
+}
+
 // weight_grads [L, D, H], bias_grads [L*H] from partials [blocks][(D+1)][K]: one
 // wavefront per output, lanes stride over the blocks, fixed summation order.
 __global__ void __launch_bounds__(256) mc_conv_reduce_kernel(int blocks, int D, int K, int H,
@@ -216,6 +337,30 @@ __global__ void __launch_bounds__(256) mc_conv_reduce_kernel(int blocks, int D, 
   const int l = j / H, h = j - l * H;
   if (q < D) dweights[(l * D + q) * H + h] = s;
   else dbiases[j] = s;
+}
+
+// Weight-gradient kernel on as many persistent blocks as the device holds at
+// once (*blocks is lowered to that number; the partial sums of that many blocks
+// are reduced afterwards), then, if asked for, the feature-gradient half.
+template <int C, int D, int ACT>
+static int launch_fused_backward(hipStream_t s, int64_t num_samples, const float *features,
+                                 const int2 *nb, const int *ranges, const McParams<D> &prm,
+                                 const float *in_grads, float *feature_grads_out,
+                                 float *pair_rows, float *workspace, bool want_dfeat,
+                                 int *blocks) {
+  auto wkernel = mc_conv_weight_grads16_kernel<C, D, ACT>;
+  int per_cu = 0, dev = 0, cus = 0;
+  MCCNN_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, wkernel, 256, 0));
+  MCCNN_HIP_CHECK(hipGetDevice(&dev));
+  MCCNN_HIP_CHECK(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+  if (per_cu * cus >= 1 && per_cu * cus < *blocks) *blocks = per_cu * cus;
+  hipLaunchKernelGGL(wkernel, dim3(*blocks), dim3(256), 0, s, num_samples, features, nb, ranges,
+                     prm, in_grads, workspace);
+  if (want_dfeat)        // the feature half keeps no running sums: one wavefront per centre
+    hipLaunchKernelGGL((mc_conv_project_grads16_kernel<C, D, ACT, false, true>),
+                       dim3(wave_grid(num_samples)), dim3(256), 0, s, num_samples, features, nb,
+                       ranges, prm, in_grads, feature_grads_out, pair_rows, workspace);
+  return MCCNN_OK;
 }
 
 static bool fused_supported(int D, int C, int K) {
@@ -275,8 +420,10 @@ extern "C" int mccnn_mc_conv_project(mccnn_stream_t stream, int num_dims, int64_
   {                                                                                            \
     McParams<D_> prm{points_in, points_out, inv_radii, weights, biases, pdf,                   \
                      num_basis / num_mlps, activation};                                        \
-    hipLaunchKernelGGL((mc_conv_project16_kernel<CPL_, D_>), grid, block, 0, s, num_samples,   \
-                       num_features, chunks, features, nb, ranges, prm, out);                  \
+    MCCNN_ACT_SWITCH(activation,                                                               \
+                     hipLaunchKernelGGL((mc_conv_project16_kernel<CPL_, D_, ACT>), grid, block, \
+                                        0, s, num_samples, num_features, chunks, features, nb, \
+                                        ranges, prm, out));                                    \
   }
 #define MCCNN_FUSED_FWD_D(CPL_) \
   if (num_dims == 3) MCCNN_FUSED_FWD(CPL_, 3) else MCCNN_FUSED_FWD(CPL_, 2)
@@ -314,7 +461,8 @@ extern "C" int mccnn_mc_conv_project_grads(
   int rc = check_fused_args("mc_conv_project_grads", num_dims, num_features, num_basis, num_mlps,
                             activation, num_neighbors, num_samples);
   if (rc != MCCNN_OK) return rc;
-  MCCNN_REQUIRE(num_pts >= 0, "mc_conv_project_grads expects a non-negative size");
+  MCCNN_REQUIRE(num_pts >= 0 && num_pts * num_features < ((int64_t)1 << 30),
+                "mc_conv_project_grads expects a feature table of fewer than 2^30 elements");
   MCCNN_REQUIRE(workspace && weight_grads_out && bias_grads_out && weights && biases &&
                     inv_radii,
                 "mc_conv_project_grads received a null tensor");
@@ -337,20 +485,16 @@ extern "C" int mccnn_mc_conv_project_grads(
   int64_t blocks64 = (num_samples + kWavesPerBlock - 1) / kWavesPerBlock;
   int blocks = (int)(blocks64 > kFusedGradBlocks ? kFusedGradBlocks : blocks64);
   if (blocks < 1) blocks = 1;
-  const dim3 grid(blocks), block(256);
-  const dim3 grid2(wave_grid(num_samples));      // the feature half keeps no running sums
   const int2 *nb = (const int2 *)neighbors;
 #define MCCNN_FUSED_BWD(C_, D_)                                                                \
   {                                                                                            \
     McParams<D_> prm{points_in, points_out, inv_radii, weights, biases, pdf,                   \
                      num_basis / num_mlps, activation};                                        \
-    hipLaunchKernelGGL((mc_conv_project_grads16_kernel<C_, D_, true, false>), grid, block, 0,  \
-                       s, num_samples, features, nb, ranges, prm, in_grads, feature_grads_out, \
-                       pair_rows, (float *)workspace);                                         \
-    if (want_dfeat)                                                                            \
-      hipLaunchKernelGGL((mc_conv_project_grads16_kernel<C_, D_, false, true>), grid2, block,  \
-                         0, s, num_samples, features, nb, ranges, prm, in_grads,               \
-                         feature_grads_out, pair_rows, (float *)workspace);                    \
+    MCCNN_ACT_SWITCH(activation,                                                               \
+                     rc = (launch_fused_backward<C_, D_, ACT>(                                 \
+                         s, num_samples, features, nb, ranges, prm, in_grads,                  \
+                         feature_grads_out, pair_rows, (float *)workspace, want_dfeat,         \
+                         &blocks)));                                                           \
   }
 #define MCCNN_FUSED_BWD_D(C_) \
   if (num_dims == 3) MCCNN_FUSED_BWD(C_, 3) else MCCNN_FUSED_BWD(C_, 2)
@@ -362,6 +506,7 @@ extern "C" int mccnn_mc_conv_project_grads(
   }
 #undef MCCNN_FUSED_BWD_D
 #undef MCCNN_FUSED_BWD
+  if (rc != MCCNN_OK) return rc;
   MCCNN_LAUNCH_CHECK();
   const int outs = (num_dims + 1) * num_basis;
   hipLaunchKernelGGL(mc_conv_reduce_kernel, dim3(blocks_for(outs, 256 / kWave)), dim3(256), 0, s,

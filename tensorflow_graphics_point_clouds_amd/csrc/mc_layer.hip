@@ -52,7 +52,7 @@ __global__ void __launch_bounds__(256) pack_final_weights_kernel(int C, int F,
   packed[t] = w[(int64_t)tile_row_to_weight_row(row, cpl) * F + ct * 16 + (lane & 15)];
 }
 
-template <int kCPL, int D>
+template <int kCPL, int D, int kAct>
 __global__ void __launch_bounds__(1024) mc_conv_layer16_kernel(
     int64_t n_out, int F, const float *__restrict__ feat, const int2 *__restrict__ nbrs,
     const int *__restrict__ ranges, McParams<D> p, const float4 *__restrict__ packed_w,
@@ -80,7 +80,7 @@ __global__ void __launch_bounds__(1024) mc_conv_layer16_kernel(
     float ctr[D];
 #pragma unroll
     for (int d = 0; d < D; ++d) ctr[d] = p.pout[centre * D + d];
-    project_pairs<kCPL, D>(reinterpret_cast<const char *>(feat), (unsigned)C * 4, nbrs, a, b, p,
+    project_pairs<kCPL, D, kAct>(reinterpret_cast<const char *>(feat), (unsigned)C * 4, nbrs, a, b, p,
                            ctr, reinterpret_cast<PairStage *>(tile) + wave, acc);
     if (proj_out) {
       float *o = proj_out + centre * (int64_t)C * K + 4 * quarter;
@@ -126,6 +126,19 @@ __global__ void __launch_bounds__(1024) mc_conv_layer16_kernel(
     for (int q = 0; q < split; ++q) s += tile[q * 16 * F + t];
     if (centre0 + ce < n_out) out[(centre0 + ce) * F + (t - ce * F)] = s;
   }
+}
+
+template <int kCPL, int D, int ACT>
+static int launch_layer(hipStream_t s, dim3 grid, dim3 block, size_t lds, int64_t num_samples,
+                        int F, const float *features, const int2 *nb, const int *ranges,
+                        const McParams<D> &prm, const float4 *packed, float *proj_out,
+                        float *out) {
+  auto kernel = mc_conv_layer16_kernel<kCPL, D, ACT>;
+  MCCNN_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+  hipLaunchKernelGGL(kernel, grid, block, lds, s, num_samples, F, features, nb, ranges, prm,
+                     packed, proj_out, out);
+  return MCCNN_OK;
 }
 
 }  // namespace mccnn
@@ -184,15 +197,16 @@ extern "C" int mccnn_mc_conv_layer(mccnn_stream_t stream, int num_dims, int64_t 
   if (lds < sizeof(PairStage) * kLayerWaves) lds = sizeof(PairStage) * kLayerWaves;
   const dim3 grid(blocks_for(num_samples, kLayerWaves)), block(kLayerWaves * kWave);
   const int2 *nb = (const int2 *)neighbors;
+  int rc = MCCNN_OK;
 #define MCCNN_LAYER(CPL_, D_)                                                                  \
   {                                                                                            \
     McParams<D_> prm{points_in, points_out, inv_radii, weights, biases, pdf,                   \
                      num_basis / num_mlps, activation};                                        \
-    auto kernel = mc_conv_layer16_kernel<CPL_, D_>;                                            \
-    MCCNN_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),                \
-                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)); \
-    hipLaunchKernelGGL(kernel, grid, block, lds, s, num_samples, F, features, nb, ranges, prm, \
-                       (const float4 *)workspace, proj_out, out);                              \
+    MCCNN_ACT_SWITCH(activation,                                                               \
+                     rc = (launch_layer<CPL_, D_, ACT>(s, grid, block, lds, num_samples, F,    \
+                                                       features, nb, ranges, prm,              \
+                                                       (const float4 *)workspace, proj_out,    \
+                                                       out)));                                 \
   }
 #define MCCNN_LAYER_D(CPL_) \
   if (num_dims == 3) MCCNN_LAYER(CPL_, 3) else MCCNN_LAYER(CPL_, 2)
@@ -204,6 +218,7 @@ extern "C" int mccnn_mc_conv_layer(mccnn_stream_t stream, int num_dims, int64_t 
   }
 #undef MCCNN_LAYER_D
 #undef MCCNN_LAYER
+  if (rc != MCCNN_OK) return rc;
   MCCNN_LAUNCH_CHECK();
   return MCCNN_OK;
 }
