@@ -243,7 +243,7 @@ __global__ void __launch_bounds__(256) basis_proj_mfma16_kernel(
 #pragma unroll
   for (int j = 0; j < kCPL; ++j) {
     float *dst = o + (col * kCPL + j) * K;
-    __builtin_nontemporal_store(acc[j], reinterpret_cast<v4f *>(dst));
+    *reinterpret_cast<v4f *>(dst) = acc[j];
   }
 }
 
@@ -300,7 +300,7 @@ __global__ void __launch_bounds__(256) basis_proj_grads_mfma32_kernel(
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
           v4f v = {acc[4 * q], acc[4 * q + 1], acc[4 * q + 2], acc[4 * q + 3]};
-          __builtin_nontemporal_store(v, reinterpret_cast<v4f *>(dst + 8 * q));
+          *reinterpret_cast<v4f *>(dst + 8 * q) = v;
         }
       }
     }

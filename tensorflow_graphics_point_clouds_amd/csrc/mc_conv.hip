@@ -43,7 +43,7 @@ __global__ void __launch_bounds__(256) mc_conv_project16_kernel(
   float *o = out + centre * (int64_t)C * K + (int64_t)chunk * kCW * K + 4 * quarter;
 #pragma unroll
   for (int j = 0; j < kCPL; ++j)
-    __builtin_nontemporal_store(acc[j], reinterpret_cast<v4f *>(o + (col * kCPL + j) * K));
+    *reinterpret_cast<v4f *>(o + (col * kCPL + j) * K) = acc[j];
 }
 
 constexpr int kFusedGradBlocks = 2048;
@@ -153,9 +153,8 @@ __global__ void __launch_bounds__(256) mc_conv_project_grads16_kernel(
           for (int s = 0; s < 4; ++s)
             acc = __builtin_amdgcn_mfma_f32_16x16x4f32(gt.v[s], basis4[s], acc, 0, 0, 0);
           if (valid)
-            __builtin_nontemporal_store(
-                acc, reinterpret_cast<v4f *>(pair_rows + (int64_t)(m0 + col) * C + 16 * t +
-                                             4 * quarter));
+            *reinterpret_cast<v4f *>(pair_rows + (int64_t)(m0 + col) * C + 16 * t +
+                                     4 * quarter) = acc;
         } else {
           // rows = pairs, columns = channels: 64 consecutive bytes per row and atomic
 #pragma unroll

@@ -86,7 +86,7 @@ __global__ void __launch_bounds__(1024) mc_conv_layer16_kernel(
       float *o = proj_out + centre * (int64_t)C * K + 4 * quarter;
 #pragma unroll
       for (int j = 0; j < kCPL; ++j)
-        __builtin_nontemporal_store(acc[j], reinterpret_cast<v4f *>(o + (col * kCPL + j) * K));
+        *reinterpret_cast<v4f *>(o + (col * kCPL + j) * K) = acc[j];
     }
   }
   __syncthreads();
