@@ -167,7 +167,8 @@ class _MCConvLayer(torch.autograd.Function):
                 fuse_final):
         view = neighborhood.sorted_view()
         pdf, _ = view.pair_pdf(neighborhood)
-        feats = features.index_select(0, view.point_order)
+        with _lib.region("permute_rows"):
+            feats = features.index_select(0, view.point_order)
         dense = _dense_final_weights(final_weights, features.shape[1])
         if fuse_final:
             out, _ = _mc_layer(weights, biases, feats, view.points_in, view.points_out,
@@ -175,9 +176,11 @@ class _MCConvLayer(torch.autograd.Function):
         else:
             proj = _mc_project(weights, biases, feats, view.points_in, view.points_out,
                                view.table, view.ranges, inv_radii, pdf, act)
-            out = proj.reshape(proj.shape[0], -1) @ dense
+            with _lib.region("gemm_out"):
+                out = proj.reshape(proj.shape[0], -1) @ dense
         if view.centre_order is not None:
-            out = torch.empty_like(out).index_copy_(0, view.centre_order, out)
+            with _lib.region("permute_rows"):
+                out = torch.empty_like(out).index_copy_(0, view.centre_order, out)
         ctx.save_for_backward(weights, biases, final_weights, feats, inv_radii)
         ctx.neighborhood, ctx.act, ctx.fuse_final = neighborhood, act, fuse_final
         return out
@@ -193,12 +196,14 @@ class _MCConvLayer(torch.autograd.Function):
         g = final_weights.shape[2]
         f = g * l
         if view.centre_order is not None:
-            dout = dout.index_select(0, view.centre_order)
+            with _lib.region("permute_rows"):
+                dout = dout.index_select(0, view.centre_order)
         else:
             dout = dout.contiguous()
         dense = _dense_final_weights(final_weights, c)               # [C*K, F]
         # kernel-MLP gradients
-        dproj = dout @ dense.t()
+        with _lib.region("gemm_dproj"):
+            dproj = dout @ dense.t()
         L = _lib.lib()
         ws = _lib.workspace(L.mccnn_mc_conv_project_grads_workspace_bytes(cint(dims), cint(k)),
                             weights.device)
@@ -221,15 +226,18 @@ class _MCConvLayer(torch.autograd.Function):
         else:
             q = _mc_project(weights, biases, dout, view.points_out, view.points_in,
                             view.table_t, view.ranges_t, neg, pdf_t, ctx.act)
-            dfeat = q.reshape(q.shape[0], f * k) @ w2
-        ddense = (feats.t() @ q.reshape(feats.shape[0], f * k)).reshape(c, f, k)
+            with _lib.region("gemm_dfeat"):
+                dfeat = q.reshape(q.shape[0], f * k) @ w2
+        with _lib.region("gemm_dfinal"):
+            ddense = (feats.t() @ q.reshape(feats.shape[0], f * k)).reshape(c, f, k)
         ddense = ddense.permute(0, 2, 1)                              # [C, K, F]
         if l == 1:
             dfinal = ddense.reshape(1, c * k, f)
         else:
             blocks = ddense.reshape(c, l, h, l, g)
             dfinal = torch.stack([blocks[:, i, :, i, :].reshape(c * h, g) for i in range(l)])
-        dfeat = torch.empty_like(dfeat).index_copy_(0, view.point_order, dfeat)
+        with _lib.region("permute_rows"):
+            dfeat = torch.empty_like(dfeat).index_copy_(0, view.point_order, dfeat)
         return dw, db, dfinal, dfeat, None, None, None, None
 
 
