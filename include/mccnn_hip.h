@@ -379,7 +379,10 @@ int mccnn_mc_basis_grads(mccnn_stream_t stream, int64_t num_neighbors,
  * separate entry points up to fp32 summation order; the [M, K] basis and its
  * gradient are never written.  mccnn_mc_conv_supported() tells whether a shape
  * is covered (D in {2,3}, K = 16, C in {16,32,64,128}); other shapes return
- * MCCNN_INVALID_ARGUMENT and must use the separate entry points.  The last three
+ * MCCNN_INVALID_ARGUMENT and must use the separate entry points.  out_rows
+ * (optional permutation of 0..N_out-1) makes the forward write the projection of
+ * centre i to row out_rows[i] of out, so that a caller working on re-ordered
+ * centres gets its result back in the original order for free.  The last three
  * inputs of the backward select the atomic-free feature gradient of
  * mccnn_basis_proj_grads_gathered (all NULL = atomics); a NULL
  * feature_grads_out skips the feature gradient (a layer obtains it without any
@@ -396,7 +399,8 @@ int mccnn_mc_conv_project(mccnn_stream_t stream, int num_dims, int64_t num_pts,
                           const int32_t *neighbors, const int32_t *ranges,
                           const float *inv_radii, int num_basis, int num_mlps,
                           int activation, const float *weights,
-                          const float *biases, const float *pdf, float *out);
+                          const float *biases, const float *pdf,
+                          const int32_t *out_rows, float *out);
 size_t mccnn_mc_conv_project_grads_workspace_bytes(int num_dims, int num_basis);
 int mccnn_mc_conv_project_grads(
     mccnn_stream_t stream, int num_dims, int64_t num_pts, const float *points_in,
@@ -434,6 +438,20 @@ int mccnn_mc_conv_layer(mccnn_stream_t stream, int num_dims, int64_t num_pts,
                         const float *pdf, int num_out_features,
                         const float *final_weights, void *workspace,
                         size_t workspace_bytes, float *proj_out, float *out);
+
+/* out[c, r] = sum_n x[n, c] * y[n, r]: the gradient of a layer's final weights
+ * (the backward of the tf.matmul of MCConv.py:187 / KPConv.py:226-230), a product
+ * with a reduction over all points and a small [C, R] output.  y is read from
+ * HBM exactly once; per-slice partial sums in the workspace are added in a fixed
+ * order (bit-reproducible).  Supported: C in {16,32,64,128}, R a multiple of 256
+ * up to 4096.  No counterpart among the reference's ops (TensorFlow's matmul
+ * gradient). */
+int mccnn_weight_grad_product_supported(int num_rows_out, int num_cols_out);
+size_t mccnn_weight_grad_product_workspace_bytes(int num_rows_out, int num_cols_out);
+int mccnn_weight_grad_product(mccnn_stream_t stream, int64_t num_pts,
+                              int num_rows_out, const float *x, int num_cols_out,
+                              const float *y, void *workspace,
+                              size_t workspace_bytes, float *out);
 
 /* Per-pair kernel-point weights, pylib/pc/layers/KPConv.py:29-57,193-213:
  *   d[m,k] = || delta_m - (kernel_points[k] + offsets[ctr_m,k]) ||

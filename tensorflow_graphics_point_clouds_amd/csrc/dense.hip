@@ -1,0 +1,138 @@
+// Gradient of the final weights of a convolution layer (pylib/pc/layers/MCConv.py:187,
+// KPConv.py:226-230): out[c, r] = sum_n x[n, c] * y[n, r] with a reduction over all
+// N points and a small output (C <= 128 rows, R = C_out * K columns).  A library
+// GEMM re-reads the long operand for every tile of the small output; here y
+// streams from HBM exactly once: the points are cut into slices, a block owns
+// (slice, 256 columns), each wavefront 64 of them with all C rows as 16x16
+// matrix-core accumulators, and the per-slice partial sums are added up
+// afterwards in a fixed order.
+#include "common.h"
+#include "fill.h"
+#include "mfma.h"
+
+namespace mccnn {
+
+static int tn_slices(int R) {
+  const int groups = R / 256;
+  int s = 1024 / groups;
+  return s < 1 ? 1 : s;
+}
+
+template <int kRT>
+__global__ void __launch_bounds__(256) tn_product_kernel(int64_t n, int R,
+                                                         const float *__restrict__ x,
+                                                         const float *__restrict__ y,
+                                                         int slices, float *__restrict__ partials) {
+  constexpr int C = 16 * kRT;
+  const int lane = lane_id(), wave = threadIdx.x / kWave;
+  const int quarter = lane >> 4, c16 = lane & 15;
+  const int groups = R >> 8;
+  const int grp = blockIdx.x % groups, slice = blockIdx.x / groups;
+  const int col0 = grp * 256 + wave * 64;
+  const int64_t steps_total = (n + 3) >> 2;                 // 4 points per matrix step
+  const int64_t per = (steps_total + slices - 1) / slices;
+  const int64_t s0 = slice * per;
+  const int64_t s1 = s0 + per < steps_total ? s0 + per : steps_total;
+  v4f acc[kRT][4];
+#pragma unroll
+  for (int i = 0; i < kRT; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.0f;
+  // lane (quarter, c16): point 4 s + quarter, channels kRT*c16 + i, columns col0 + 4*c16 + j
+  const float *xl = x + kRT * c16;
+  const float *yl = y + col0 + 4 * c16;
+  auto load_a = [&](int64_t s) {
+    const int64_t pt = 4 * s + quarter;
+    return load_vec<kRT>(xl + pt * C, s < s1 && pt < n);
+  };
+  auto load_b = [&](int64_t s) {
+    const int64_t pt = 4 * s + quarter;
+    return load_vec<4>(yl + pt * R, s < s1 && pt < n);
+  };
+  FVec<kRT> a0 = load_a(s0), a1 = load_a(s0 + 1);
+  FVec<4> b0 = load_b(s0), b1 = load_b(s0 + 1);
+  for (int64_t s = s0; s < s1; s += 2) {
+    const FVec<kRT> a2 = load_a(s + 2), a3 = load_a(s + 3);
+    const FVec<4> b2 = load_b(s + 2), b3 = load_b(s + 3);
+#pragma unroll
+    for (int i = 0; i < kRT; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a0.v[i], b0.v[j], acc[i][j], 0, 0, 0);
+#pragma unroll
+    for (int i = 0; i < kRT; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a1.v[i], b1.v[j], acc[i][j], 0, 0, 0);
+    a0 = a2; a1 = a3; b0 = b2; b1 = b3;
+  }
+  // accumulator (i, j), register r: channel kRT*(4*quarter + r) + i, column col0 + 4*c16 + j
+  float *o = partials + (int64_t)slice * C * R + col0 + 4 * c16;
+#pragma unroll
+  for (int i = 0; i < kRT; ++i)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const v4f v = {acc[i][0][r], acc[i][1][r], acc[i][2][r], acc[i][3][r]};
+      *reinterpret_cast<v4f *>(o + (int64_t)(kRT * (4 * quarter + r) + i) * R) = v;
+    }
+}
+
+__global__ void __launch_bounds__(256) tn_reduce_kernel(int64_t elems, int slices,
+                                                        const float *__restrict__ partials,
+                                                        float *__restrict__ out) {
+  const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= elems) return;
+  float s = 0.0f;
+  for (int k = 0; k < slices; ++k) s += partials[(int64_t)k * elems + e];
+  out[e] = s;
+}
+
+static bool tn_supported(int C, int R) {
+  return (C == 16 || C == 32 || C == 64 || C == 128) && R >= 256 && R % 256 == 0 && R <= 4096;
+}
+
+}  // namespace mccnn
+
+using namespace mccnn;
+
+extern "C" int mccnn_weight_grad_product_supported(int num_rows_out, int num_cols_out) {
+  return tn_supported(num_rows_out, num_cols_out) ? 1 : 0;
+}
+
+extern "C" size_t mccnn_weight_grad_product_workspace_bytes(int num_rows_out, int num_cols_out) {
+  if (!tn_supported(num_rows_out, num_cols_out)) return 0;
+  return align256(sizeof(float) * (size_t)tn_slices(num_cols_out) * num_rows_out * num_cols_out);
+}
+
+extern "C" int mccnn_weight_grad_product(mccnn_stream_t stream, int64_t num_pts, int num_rows_out,
+                                         const float *x, int num_cols_out, const float *y,
+                                         void *workspace, size_t workspace_bytes, float *out) {
+  MCCNN_REQUIRE(tn_supported(num_rows_out, num_cols_out),
+                "weight_grad_product supports 16/32/64/128 output rows and a multiple of 256 "
+                "(at most 4096) output columns (got %d x %d)", num_rows_out, num_cols_out);
+  MCCNN_REQUIRE(num_pts >= 0 && num_pts < ((int64_t)1 << 31),
+                "weight_grad_product expects a size in [0, 2^31)");
+  MCCNN_REQUIRE(out && workspace && (num_pts == 0 || (x && y)),
+                "weight_grad_product received a null tensor");
+  MCCNN_REQUIRE(workspace_bytes >=
+                    mccnn_weight_grad_product_workspace_bytes(num_rows_out, num_cols_out),
+                "weight_grad_product workspace too small");
+  hipStream_t s = as_stream(stream);
+  const int C = num_rows_out, R = num_cols_out, slices = tn_slices(R);
+  const dim3 grid((R / 256) * slices), block(256);
+  float *partials = (float *)workspace;
+  switch (C / 16) {
+    case 8: hipLaunchKernelGGL(tn_product_kernel<8>, grid, block, 0, s, num_pts, R, x, y, slices, partials); break;
+    case 4: hipLaunchKernelGGL(tn_product_kernel<4>, grid, block, 0, s, num_pts, R, x, y, slices, partials); break;
+    case 2: hipLaunchKernelGGL(tn_product_kernel<2>, grid, block, 0, s, num_pts, R, x, y, slices, partials); break;
+    default: hipLaunchKernelGGL(tn_product_kernel<1>, grid, block, 0, s, num_pts, R, x, y, slices, partials); break;
+  }
+  MCCNN_LAUNCH_CHECK();
+  const int64_t elems = (int64_t)C * R;
+  hipLaunchKernelGGL(tn_reduce_kernel, dim3(blocks_for(elems, 256)), dim3(256), 0, s, elems,
+                     slices, partials, out);
+  MCCNN_LAUNCH_CHECK();
+  return MCCNN_OK;
+}

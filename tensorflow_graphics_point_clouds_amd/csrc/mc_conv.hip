@@ -19,7 +19,7 @@ template <int kCPL, int D, int kAct>
 __global__ void __launch_bounds__(256) mc_conv_project16_kernel(
     int64_t n_out, int C, int chunks, const float *__restrict__ feat,
     const int2 *__restrict__ nbrs, const int *__restrict__ ranges, McParams<D> p,
-    float *__restrict__ out) {
+    const int *__restrict__ out_rows, float *__restrict__ out) {
   constexpr int K = kFusedK;
   constexpr int kCW = 16 * kCPL;
   const int lane = lane_id();
@@ -40,7 +40,8 @@ __global__ void __launch_bounds__(256) mc_conv_project16_kernel(
     for (int r = 0; r < 4; ++r) acc[j][r] = 0.0f;
   project_pairs<kCPL, D, kAct>(reinterpret_cast<const char *>(feat + chunk * kCW), (unsigned)C * 4, nbrs,
                          a, b, p, ctr, &stages[threadIdx.x / kWave], acc);
-  float *o = out + centre * (int64_t)C * K + (int64_t)chunk * kCW * K + 4 * quarter;
+  const int64_t row = out_rows ? (int64_t)__builtin_amdgcn_readfirstlane(out_rows[centre]) : centre;
+  float *o = out + row * (int64_t)C * K + (int64_t)chunk * kCW * K + 4 * quarter;
 #pragma unroll
   for (int j = 0; j < kCPL; ++j)
     *reinterpret_cast<v4f *>(o + (col * kCPL + j) * K) = acc[j];
@@ -398,7 +399,7 @@ extern "C" int mccnn_mc_conv_project(mccnn_stream_t stream, int num_dims, int64_
                                      const int32_t *neighbors, const int32_t *ranges,
                                      const float *inv_radii, int num_basis, int num_mlps,
                                      int activation, const float *weights, const float *biases,
-                                     const float *pdf, float *out) {
+                                     const float *pdf, const int32_t *out_rows, float *out) {
   int rc = check_fused_args("mc_conv_project", num_dims, num_features, num_basis, num_mlps,
                             activation, num_neighbors, num_samples);
   if (rc != MCCNN_OK) return rc;
@@ -422,7 +423,7 @@ extern "C" int mccnn_mc_conv_project(mccnn_stream_t stream, int num_dims, int64_
     MCCNN_ACT_SWITCH(activation,                                                               \
                      hipLaunchKernelGGL((mc_conv_project16_kernel<CPL_, D_, ACT>), grid, block, \
                                         0, s, num_samples, num_features, chunks, features, nb, \
-                                        ranges, prm, out));                                    \
+                                        ranges, prm, out_rows, out));                          \
   }
 #define MCCNN_FUSED_FWD_D(CPL_) \
   if (num_dims == 3) MCCNN_FUSED_FWD(CPL_, 3) else MCCNN_FUSED_FWD(CPL_, 2)

@@ -65,7 +65,7 @@ class _MCConvProject(torch.autograd.Function):
                   i64(ranges.shape[0]), ptr(points_out, _F32), i64(neighbors.shape[0]),
                   ptr(neighbors, _I32), ptr(ranges, _I32), ptr(inv_radii, _F32), cint(k),
                   cint(num_mlps), cint(act), ptr(weights, _F32), ptr(biases, _F32),
-                  ptr(pdf, _F32), ptr(out))
+                  ptr(pdf, _F32), ptr(None), ptr(out))
         ctx.save_for_backward(weights, biases, features, points_in, points_out, neighbors,
                               ranges, inv_radii, pdf)
         ctx.act, ctx.transposed = act, transposed
@@ -98,7 +98,7 @@ class _MCConvProject(torch.autograd.Function):
 
 
 def _mc_project(weights, biases, features, points_in, points_out, neighbors, ranges, inv_radii,
-                pdf, act):
+                pdf, act, out_rows=None):
     num_mlps, dims, hidden = weights.shape
     k = num_mlps * hidden
     out = torch.empty((ranges.shape[0], features.shape[1], k), dtype=_F32,
@@ -108,7 +108,7 @@ def _mc_project(weights, biases, features, points_in, points_out, neighbors, ran
               i64(ranges.shape[0]), ptr(points_out, _F32), i64(neighbors.shape[0]),
               ptr(neighbors, _I32), ptr(ranges, _I32), ptr(inv_radii, _F32), cint(k),
               cint(num_mlps), cint(act), ptr(weights, _F32), ptr(biases, _F32),
-              ptr(pdf, _F32), ptr(out))
+              ptr(pdf, _F32), ptr(out_rows), ptr(out))
     return out
 
 
@@ -133,6 +133,21 @@ def _mc_layer(weights, biases, features, points_in, points_out, neighbors, range
               ptr(dense_weights.contiguous(), _F32), ptr(ws), _lib.csize(ws.numel()), ptr(proj),
               ptr(out))
     return out, proj
+
+
+def _weight_grad_product(x, y):
+    """x^T y for [N, C] and [N, R] operands with the long reduction over N."""
+    c, r = x.shape[1], y.shape[1]
+    L = _lib.lib()
+    if not L.mccnn_weight_grad_product_supported(cint(c), cint(r)):
+        with _lib.region("gemm_dfinal"):
+            return x.t() @ y
+    L.mccnn_weight_grad_product_workspace_bytes.restype = _lib.csize
+    ws = _lib.workspace(L.mccnn_weight_grad_product_workspace_bytes(cint(c), cint(r)), x.device)
+    out = torch.empty((c, r), dtype=_F32, device=x.device)
+    _lib.call("weight_grad_product", stream(), i64(x.shape[0]), cint(c), ptr(x, _F32), cint(r),
+              ptr(y, _F32), ptr(ws), _lib.csize(ws.numel()), ptr(out))
+    return out
 
 
 def _dense_final_weights(final_weights, c):
@@ -173,21 +188,23 @@ class _MCConvLayer(torch.autograd.Function):
         if fuse_final:
             out, _ = _mc_layer(weights, biases, feats, view.points_in, view.points_out,
                                view.table, view.ranges, inv_radii, pdf, act, dense)
+            if view.centre_order is not None:
+                with _lib.region("permute_rows"):
+                    out = torch.empty_like(out).index_copy_(0, view.centre_order, out)
         else:
+            # rows of the projection go straight to the centres' original positions
             proj = _mc_project(weights, biases, feats, view.points_in, view.points_out,
-                               view.table, view.ranges, inv_radii, pdf, act)
+                               view.table, view.ranges, inv_radii, pdf, act,
+                               view.centre_rows)
             with _lib.region("gemm_out"):
                 out = proj.reshape(proj.shape[0], -1) @ dense
-        if view.centre_order is not None:
-            with _lib.region("permute_rows"):
-                out = torch.empty_like(out).index_copy_(0, view.centre_order, out)
-        ctx.save_for_backward(weights, biases, final_weights, feats, inv_radii)
+        ctx.save_for_backward(weights, biases, final_weights, feats, features, inv_radii)
         ctx.neighborhood, ctx.act, ctx.fuse_final = neighborhood, act, fuse_final
         return out
 
     @staticmethod
     def backward(ctx, dout):
-        weights, biases, final_weights, feats, inv_radii = ctx.saved_tensors
+        weights, biases, final_weights, feats, features, inv_radii = ctx.saved_tensors
         nbh = ctx.neighborhood
         view = nbh.sorted_view()
         pdf, pdf_t = view.pair_pdf(nbh)
@@ -223,21 +240,22 @@ class _MCConvLayer(torch.autograd.Function):
             dfeat, q = _mc_layer(weights, biases, dout, view.points_out, view.points_in,
                                  view.table_t, view.ranges_t, neg, pdf_t, ctx.act, w2,
                                  want_proj=True)
+            with _lib.region("permute_rows"):
+                dfeat = torch.empty_like(dfeat).index_copy_(0, view.point_order, dfeat)
+            ddense = _weight_grad_product(feats, q.reshape(feats.shape[0], f * k))
         else:
+            # rows of Q (and so of dfeat) go straight to the points' original positions
             q = _mc_project(weights, biases, dout, view.points_out, view.points_in,
-                            view.table_t, view.ranges_t, neg, pdf_t, ctx.act)
+                            view.table_t, view.ranges_t, neg, pdf_t, ctx.act, view.point_rows)
             with _lib.region("gemm_dfeat"):
                 dfeat = q.reshape(q.shape[0], f * k) @ w2
-        with _lib.region("gemm_dfinal"):
-            ddense = (feats.t() @ q.reshape(feats.shape[0], f * k)).reshape(c, f, k)
-        ddense = ddense.permute(0, 2, 1)                              # [C, K, F]
+            ddense = _weight_grad_product(features, q.reshape(features.shape[0], f * k))
+        ddense = ddense.reshape(c, f, k).permute(0, 2, 1)            # [C, K, F]
         if l == 1:
             dfinal = ddense.reshape(1, c * k, f)
         else:
             blocks = ddense.reshape(c, l, h, l, g)
             dfinal = torch.stack([blocks[:, i, :, i, :].reshape(c * h, g) for i in range(l)])
-        with _lib.region("permute_rows"):
-            dfeat = torch.empty_like(dfeat).index_copy_(0, view.point_order, dfeat)
         return dw, db, dfinal, dfeat, None, None, None, None
 
 

@@ -116,10 +116,11 @@ class _SortedView:
     def __init__(self, nbh):
         grid, samples = nbh._grid, nbh._point_cloud_sampled
         self.points_in = grid._sorted_points
+        self.point_rows = grid._sorted_indices           # int32, for kernels
         self.point_order = grid._sorted_indices.long()
         n_out = samples._points.shape[0]
         if nbh._equal_samples:
-            self.centre_order = None
+            self.centre_order = self.centre_rows = None
             self.points_out = grid._sorted_points
             self.table, self.ranges = nbh._neighbors, nbh._samples_neigh_ranges
         else:
@@ -129,6 +130,7 @@ class _SortedView:
             else:
                 order = nbh.compute_centre_order()
                 self.points_out = samples._points[order.long()].contiguous()
+            self.centre_rows = order
             self.centre_order = order.long()
             L = _lib.lib()
             L.mccnn_reorder_neighbors_workspace_bytes.restype = _lib.csize

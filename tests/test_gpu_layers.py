@@ -243,3 +243,18 @@ def test_local_and_global_pooling(oracle, c):
         else:
             gexp = np.where(feat == expect.astype(np.float32)[bids], up[bids], 0.0)
         normwise(t.grad.cpu().numpy(), gexp)
+
+
+@pytest.mark.parametrize("n,c,r", [(1, 16, 256), (4099, 64, 1024), (20000, 128, 512),
+                                   (777, 32, 2048), (0, 64, 256)])
+def test_weight_grad_product_matches_float64(n, c, r):
+    """x^T y with the long reduction over the points against float64 matmul
+    (tolerance 1e-5 of the largest entry)."""
+    from tensorflow_graphics_point_clouds_amd import layers
+    gen = torch.Generator(device="cuda").manual_seed(n + c)
+    x = torch.randn((n, c), device="cuda", generator=gen)
+    y = torch.randn((n, r), device="cuda", generator=gen)
+    got = layers._weight_grad_product(x, y).cpu().numpy().astype(np.float64)
+    expect = (x.double().t() @ y.double()).cpu().numpy()
+    assert got.shape == (c, r)
+    assert np.abs(got - expect).max() <= 1e-5 * max(1.0, np.abs(expect).max())
