@@ -453,6 +453,16 @@ int mccnn_weight_grad_product(mccnn_stream_t stream, int64_t num_pts,
                               const float *y, void *workspace,
                               size_t workspace_bytes, float *out);
 
+/* out[n, r] = sum_f x[n, f] * w[r, f]: the gradient of the projection entering a
+ * layer's final product (x = output gradient [N, F], w = final weights [R, F],
+ * out [N, R]); write-bound, each wavefront keeps its slice of w in registers.
+ * Supported: F in {16,32,64}, R a multiple of 256.  No counterpart among the
+ * reference's ops (TensorFlow's matmul gradient). */
+int mccnn_projection_grad_product_supported(int num_cols_in, int num_cols_out);
+int mccnn_projection_grad_product(mccnn_stream_t stream, int64_t num_pts,
+                                  int num_cols_in, const float *x,
+                                  int num_cols_out, const float *w, float *out);
+
 /* Per-pair kernel-point weights, pylib/pc/layers/KPConv.py:29-57,193-213:
  *   d[m,k] = || delta_m - (kernel_points[k] + offsets[ctr_m,k]) ||
  *   kind 0: max(1 - d/sigma, 0);  kind 1: exp(-(d/(sigma/3))^2)

@@ -89,6 +89,68 @@ __global__ void __launch_bounds__(256) tn_reduce_kernel(int64_t elems, int slice
   out[e] = s;
 }
 
+// out[n, r] = sum_f x[n, f] * w[r, f]: the gradient of the projection that enters
+// a layer's final product (x = output gradient [N, F], w = dense final weights
+// [R, F], R = C * K).  Write-bound: 4 R bytes per point leave, 4 F arrive.  A
+// wavefront keeps its 64 x F slice of w in registers for its whole life and
+// streams tiles of 16 points through the matrix cores; a lane owns 4 consecutive
+// output columns so that every row of a tile leaves as 256 contiguous bytes.
+template <int F>
+__global__ void __launch_bounds__(256) nt_product_kernel(int64_t n, int R,
+                                                         const float *__restrict__ x,
+                                                         const float *__restrict__ w,
+                                                         int slices, float *__restrict__ out) {
+  constexpr int kSteps = F / 4;            // reduction steps; lane (kk, row) owns f = kk*kSteps + s
+  const int lane = lane_id(), wave = threadIdx.x / kWave;
+  const int kk = lane >> 4, c16 = lane & 15;
+  const int groups = R >> 8;
+  const int grp = blockIdx.x % groups, slice = blockIdx.x / groups;
+  const int col0 = grp * 256 + wave * 64;
+  // B operand of step s, column tile j: w[col0 + 4*c16 + j][kk*kSteps + s]
+  float b[4][kSteps];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const FVec<kSteps> t = load_vec<kSteps>(w + (int64_t)(col0 + 4 * c16 + j) * F + kk * kSteps,
+                                            true);
+#pragma unroll
+    for (int s = 0; s < kSteps; ++s) b[j][s] = t.v[s];
+  }
+  const int64_t tiles_total = (n + 15) >> 4;
+  const int64_t per = (tiles_total + slices - 1) / slices;
+  const int64_t t0 = slice * per;
+  const int64_t t1 = t0 + per < tiles_total ? t0 + per : tiles_total;
+  auto load_a = [&](int64_t t) {
+    const int64_t pt = 16 * t + c16;
+    return load_vec<kSteps>(x + pt * F + kk * kSteps, t < t1 && pt < n);
+  };
+  FVec<kSteps> a = load_a(t0);
+  for (int64_t t = t0; t < t1; ++t) {
+    const FVec<kSteps> an = load_a(t + 1);
+    v4f acc[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[j] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int s = 0; s < kSteps; ++s)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.v[s], b[j][s], acc[j], 0, 0, 0);
+    // acc[j][r]: point 16 t + 4*kk + r, column col0 + 4*c16 + j
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int64_t pt = 16 * t + 4 * kk + r;
+      if (pt < n) {
+        const v4f v = {acc[0][r], acc[1][r], acc[2][r], acc[3][r]};
+        *reinterpret_cast<v4f *>(out + pt * R + col0 + 4 * c16) = v;
+      }
+    }
+    a = an;
+  }
+}
+
+static bool nt_supported(int F, int R) {
+  return (F == 16 || F == 32 || F == 64) && R >= 256 && R % 256 == 0;
+}
+
 static bool tn_supported(int C, int R) {
   return (C == 16 || C == 32 || C == 64 || C == 128) && R >= 256 && R % 256 == 0 && R <= 4096;
 }
@@ -133,6 +195,35 @@ extern "C" int mccnn_weight_grad_product(mccnn_stream_t stream, int64_t num_pts,
   const int64_t elems = (int64_t)C * R;
   hipLaunchKernelGGL(tn_reduce_kernel, dim3(blocks_for(elems, 256)), dim3(256), 0, s, elems,
                      slices, partials, out);
+  MCCNN_LAUNCH_CHECK();
+  return MCCNN_OK;
+}
+
+extern "C" int mccnn_projection_grad_product_supported(int num_cols_in, int num_cols_out) {
+  return nt_supported(num_cols_in, num_cols_out) ? 1 : 0;
+}
+
+extern "C" int mccnn_projection_grad_product(mccnn_stream_t stream, int64_t num_pts,
+                                             int num_cols_in, const float *x, int num_cols_out,
+                                             const float *w, float *out) {
+  MCCNN_REQUIRE(nt_supported(num_cols_in, num_cols_out),
+                "projection_grad_product supports 16/32/64 input columns and a multiple of 256 "
+                "output columns (got %d -> %d)", num_cols_in, num_cols_out);
+  MCCNN_REQUIRE(num_pts >= 0 && num_pts < ((int64_t)1 << 31),
+                "projection_grad_product expects a size in [0, 2^31)");
+  if (num_pts == 0) return MCCNN_OK;
+  MCCNN_REQUIRE(x && w && out, "projection_grad_product received a null tensor");
+  hipStream_t s = as_stream(stream);
+  const int F = num_cols_in, R = num_cols_out, groups = R / 256;
+  int slices = 2048 / groups;
+  const int64_t tiles = (num_pts + 15) / 16;
+  if (slices > tiles) slices = (int)tiles;
+  const dim3 grid(groups * slices), block(256);
+  switch (F) {
+    case 64: hipLaunchKernelGGL(nt_product_kernel<64>, grid, block, 0, s, num_pts, R, x, w, slices, out); break;
+    case 32: hipLaunchKernelGGL(nt_product_kernel<32>, grid, block, 0, s, num_pts, R, x, w, slices, out); break;
+    default: hipLaunchKernelGGL(nt_product_kernel<16>, grid, block, 0, s, num_pts, R, x, w, slices, out); break;
+  }
   MCCNN_LAUNCH_CHECK();
   return MCCNN_OK;
 }

@@ -150,6 +150,18 @@ def _weight_grad_product(x, y):
     return out
 
 
+def _projection_grad_product(x, w):
+    """x w^T for x [N, F] and w [R, F]."""
+    f, r = x.shape[1], w.shape[0]
+    if not _lib.lib().mccnn_projection_grad_product_supported(cint(f), cint(r)):
+        with _lib.region("gemm_dproj"):
+            return x @ w.t()
+    out = torch.empty((x.shape[0], r), dtype=_F32, device=x.device)
+    _lib.call("projection_grad_product", stream(), i64(x.shape[0]), cint(f), ptr(x, _F32),
+              cint(r), ptr(w.contiguous(), _F32), ptr(out))
+    return out
+
+
 def _dense_final_weights(final_weights, c):
     """[L, C*H, G] per-MLP blocks -> dense [C*(L*H), L*G] with zero off-diagonal blocks."""
     l, ch, g = final_weights.shape
@@ -219,8 +231,7 @@ class _MCConvLayer(torch.autograd.Function):
             dout = dout.contiguous()
         dense = _dense_final_weights(final_weights, c)               # [C*K, F]
         # kernel-MLP gradients
-        with _lib.region("gemm_dproj"):
-            dproj = dout @ dense.t()
+        dproj = _projection_grad_product(dout, dense)
         L = _lib.lib()
         ws = _lib.workspace(L.mccnn_mc_conv_project_grads_workspace_bytes(cint(dims), cint(k)),
                             weights.device)
