@@ -401,7 +401,8 @@ int mccnn_mc_conv_project(mccnn_stream_t stream, int num_dims, int64_t num_pts,
                           int activation, const float *weights,
                           const float *biases, const float *pdf,
                           const int32_t *out_rows, float *out);
-size_t mccnn_mc_conv_project_grads_workspace_bytes(int num_dims, int num_basis);
+size_t mccnn_mc_conv_project_grads_workspace_bytes(int num_dims, int num_basis,
+                                                   int64_t num_samples);
 int mccnn_mc_conv_project_grads(
     mccnn_stream_t stream, int num_dims, int64_t num_pts, const float *points_in,
     int num_features, const float *features, int64_t num_samples,

@@ -42,10 +42,15 @@ def lib():
                 "`make -C %s` or __graft_entry__.build()" % (LIB_PATH, CSRC_DIR))
         handle = ctypes.CDLL(LIB_PATH)
         handle.mccnn_last_error.restype = ctypes.c_char_p
-        for name in ("mccnn_sort_keys_workspace_bytes",
-                     "mccnn_find_neighbors_workspace_bytes",
+        for name in ("mccnn_find_neighbors_workspace_bytes",
+                     "mccnn_mc_basis_grads_workspace_bytes",
+                     "mccnn_mc_conv_layer_workspace_bytes",
+                     "mccnn_mc_conv_project_grads_workspace_bytes",
+                     "mccnn_reorder_neighbors_workspace_bytes",
                      "mccnn_sampling_workspace_bytes",
-                     "mccnn_mc_basis_grads_workspace_bytes"):
+                     "mccnn_sort_keys_workspace_bytes",
+                     "mccnn_transpose_neighbors_workspace_bytes",
+                     "mccnn_weight_grad_product_workspace_bytes"):
             getattr(handle, name).restype = csize
         _lib = handle
     return _lib

@@ -47,7 +47,6 @@ __global__ void __launch_bounds__(256) mc_conv_project16_kernel(
     *reinterpret_cast<v4f *>(o + (col * kCPL + j) * K) = acc[j];
 }
 
-constexpr int kFusedGradBlocks = 2048;
 
 // Persistent wavefronts stride over the centres.  Per tile of 16 pairs:
 //   dbasis^T [k x pair] by MFMA (reduction over channels), turned in registers
@@ -201,13 +200,20 @@ __global__ void __launch_bounds__(256) mc_conv_project_grads16_kernel(
 }
 
 // Kernel-MLP gradients alone (the layer obtains its feature gradient from the
-// transposed convolution).  Persistent wavefronts, as many as fit on the device,
-// stride over the centres.  Per centre the upstream tile G [C x 16] sits in
+// transposed convolution).  Per centre the upstream tile G [C x 16] sits in
 // registers as the A operand; per chunk of 64 pairs lane n stages pair n in LDS
 // (offset, 1/pdf, feature row), then every tile of 16 pairs takes 16*C/64 matrix
 // steps for dbasis^T [k x pair] while the feature rows of the next tile are
 // already in flight, and the result is folded in registers into
 //   dW[d][k] += delta_d * dz,  db[k] += dz,  dz = dbasis * act'(z) / pdf.
+constexpr int kGradRun = 8;
+
+static int64_t grad_blocks(int64_t num_samples) {
+  const int64_t per_block = (int64_t)kWavesPerBlock * kGradRun;
+  const int64_t b = (num_samples + per_block - 1) / per_block;
+  return b < 1 ? 1 : b;
+}
+
 template <int C, int D, int kAct>
 __global__ void __launch_bounds__(256) mc_conv_weight_grads16_kernel(
     int64_t n_out, const float *__restrict__ feat, const int2 *__restrict__ nbrs,
@@ -238,8 +244,12 @@ __global__ void __launch_bounds__(256) mc_conv_weight_grads16_kernel(
     for (int d = 0; d < 3; ++d) dw[r][d] = 0.0f;
   }
   const char *feat_lane = reinterpret_cast<const char *>(feat + quarter * kQuarterC);
-  const int64_t total_waves = (int64_t)gridDim.x * kWavesPerBlock;
-  for (int64_t centre = wave_slot(); centre < n_out; centre += total_waves) {
+  // A wavefront takes kGradRun consecutive centres and blocks are dispatched in
+  // index order, so at any moment the device works on one compact window of the
+  // (grid-ordered) centres and the feature rows of that window stay in L2.
+  const int64_t first = wave_slot() * kGradRun;
+  const int64_t last = first + kGradRun < n_out ? first + kGradRun : n_out;
+  for (int64_t centre = first; centre < last; ++centre) {
     const int a = centre > 0 ? ranges[centre - 1] : 0, b = ranges[centre];
     if (b <= a) continue;
     const float *gi = in_grad + centre * (int64_t)C * K;
@@ -322,40 +332,38 @@ __global__ void __launch_bounds__(256) mc_conv_weight_grads16_kernel(
 }
 
 // weight_grads [L, D, H], bias_grads [L*H] from partials [blocks][(D+1)][K]: one
-// wavefront per output, lanes stride over the blocks, fixed summation order.
-__global__ void __launch_bounds__(256) mc_conv_reduce_kernel(int blocks, int D, int K, int H,
+// block per output, threads stride over the partials, fixed summation order.
+__global__ void __launch_bounds__(256) mc_conv_reduce_kernel(int64_t blocks, int D, int K, int H,
                                                              const float *__restrict__ partials,
                                                              float *__restrict__ dweights,
                                                              float *__restrict__ dbiases) {
-  const int t = blockIdx.x * (256 / kWave) + threadIdx.x / kWave;
-  if (t >= (D + 1) * K) return;
+  __shared__ float red[256 / kWave];
+  const int t = blockIdx.x;
   const int q = t / K, j = t - q * K;
   float s = 0.0f;
-  for (int b = lane_id(); b < blocks; b += kWave) s += partials[(int64_t)b * (D + 1) * K + t];
+  for (int64_t b = threadIdx.x; b < blocks; b += 256) s += partials[b * (D + 1) * K + t];
   s = wave_sum(s);
-  if (lane_id() != 0) return;
+  if (lane_id() == 0) red[threadIdx.x / kWave] = s;
+  __syncthreads();
+  if (threadIdx.x != 0) return;
+  s = 0.0f;
+#pragma unroll
+  for (int w = 0; w < 256 / kWave; ++w) s += red[w];
   const int l = j / H, h = j - l * H;
   if (q < D) dweights[(l * D + q) * H + h] = s;
   else dbiases[j] = s;
 }
 
-// Weight-gradient kernel on as many persistent blocks as the device holds at
-// once (*blocks is lowered to that number; the partial sums of that many blocks
-// are reduced afterwards), then, if asked for, the feature-gradient half.
+// Weight-gradient kernel (one partial sum per block, reduced afterwards), then, if
+// asked for, the feature-gradient half.
 template <int C, int D, int ACT>
 static int launch_fused_backward(hipStream_t s, int64_t num_samples, const float *features,
                                  const int2 *nb, const int *ranges, const McParams<D> &prm,
                                  const float *in_grads, float *feature_grads_out,
-                                 float *pair_rows, float *workspace, bool want_dfeat,
-                                 int *blocks) {
-  auto wkernel = mc_conv_weight_grads16_kernel<C, D, ACT>;
-  int per_cu = 0, dev = 0, cus = 0;
-  MCCNN_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, wkernel, 256, 0));
-  MCCNN_HIP_CHECK(hipGetDevice(&dev));
-  MCCNN_HIP_CHECK(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
-  if (per_cu * cus >= 1 && per_cu * cus < *blocks) *blocks = per_cu * cus;
-  hipLaunchKernelGGL(wkernel, dim3(*blocks), dim3(256), 0, s, num_samples, features, nb, ranges,
-                     prm, in_grads, workspace);
+                                 float *pair_rows, float *workspace, bool want_dfeat) {
+  hipLaunchKernelGGL((mc_conv_weight_grads16_kernel<C, D, ACT>),
+                     dim3((unsigned)grad_blocks(num_samples)), dim3(256), 0, s, num_samples,
+                     features, nb, ranges, prm, in_grads, workspace);
   if (want_dfeat)        // the feature half keeps no running sums: one wavefront per centre
     hipLaunchKernelGGL((mc_conv_project_grads16_kernel<C, D, ACT, false, true>),
                        dim3(wave_grid(num_samples)), dim3(256), 0, s, num_samples, features, nb,
@@ -439,9 +447,10 @@ extern "C" int mccnn_mc_conv_project(mccnn_stream_t stream, int num_dims, int64_
   return MCCNN_OK;
 }
 
-extern "C" size_t mccnn_mc_conv_project_grads_workspace_bytes(int num_dims, int num_basis) {
-  if (!valid_dims(num_dims) || num_basis <= 0) return 0;
-  return align256(sizeof(float) * (size_t)kFusedGradBlocks * (num_dims + 1) * num_basis);
+extern "C" size_t mccnn_mc_conv_project_grads_workspace_bytes(int num_dims, int num_basis,
+                                                              int64_t num_samples) {
+  if (!valid_dims(num_dims) || num_basis <= 0 || num_samples < 0) return 0;
+  return align256(sizeof(float) * (size_t)grad_blocks(num_samples) * (num_dims + 1) * num_basis);
 }
 
 extern "C" int mccnn_mc_conv_project_grads(
@@ -467,7 +476,7 @@ extern "C" int mccnn_mc_conv_project_grads(
                     inv_radii,
                 "mc_conv_project_grads received a null tensor");
   MCCNN_REQUIRE(workspace_bytes >=
-                    mccnn_mc_conv_project_grads_workspace_bytes(num_dims, num_basis),
+                    mccnn_mc_conv_project_grads_workspace_bytes(num_dims, num_basis, num_samples),
                 "mc_conv_project_grads workspace too small");
   hipStream_t s = as_stream(stream);
   // A null feature_grads_out asks for the kernel-MLP gradients only.
@@ -482,9 +491,6 @@ extern "C" int mccnn_mc_conv_project_grads(
                     (points_in && points_out && features && neighbors && ranges && pdf &&
                      in_grads),
                 "mc_conv_project_grads received a null tensor");
-  int64_t blocks64 = (num_samples + kWavesPerBlock - 1) / kWavesPerBlock;
-  int blocks = (int)(blocks64 > kFusedGradBlocks ? kFusedGradBlocks : blocks64);
-  if (blocks < 1) blocks = 1;
   const int2 *nb = (const int2 *)neighbors;
 #define MCCNN_FUSED_BWD(C_, D_)                                                                \
   {                                                                                            \
@@ -493,8 +499,7 @@ extern "C" int mccnn_mc_conv_project_grads(
     MCCNN_ACT_SWITCH(activation,                                                               \
                      rc = (launch_fused_backward<C_, D_, ACT>(                                 \
                          s, num_samples, features, nb, ranges, prm, in_grads,                  \
-                         feature_grads_out, pair_rows, (float *)workspace, want_dfeat,         \
-                         &blocks)));                                                           \
+                         feature_grads_out, pair_rows, (float *)workspace, want_dfeat)));      \
   }
 #define MCCNN_FUSED_BWD_D(C_) \
   if (num_dims == 3) MCCNN_FUSED_BWD(C_, 3) else MCCNN_FUSED_BWD(C_, 2)
@@ -509,9 +514,8 @@ extern "C" int mccnn_mc_conv_project_grads(
   if (rc != MCCNN_OK) return rc;
   MCCNN_LAUNCH_CHECK();
   const int outs = (num_dims + 1) * num_basis;
-  hipLaunchKernelGGL(mc_conv_reduce_kernel, dim3(blocks_for(outs, 256 / kWave)), dim3(256), 0, s,
-                     blocks,
-                     num_dims, num_basis, num_basis / num_mlps, (const float *)workspace,
+  hipLaunchKernelGGL(mc_conv_reduce_kernel, dim3(outs), dim3(256), 0, s,
+                     grad_blocks(num_samples), num_dims, num_basis, num_basis / num_mlps, (const float *)workspace,
                      weight_grads_out, bias_grads_out);
   MCCNN_LAUNCH_CHECK();
   if (gathered && num_samples > 0 && num_neighbors > 0)

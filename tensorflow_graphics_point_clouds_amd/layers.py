@@ -78,8 +78,8 @@ class _MCConvProject(torch.autograd.Function):
         num_mlps, dims, hidden = weights.shape
         k = num_mlps * hidden
         L = _lib.lib()
-        ws = _lib.workspace(L.mccnn_mc_conv_project_grads_workspace_bytes(cint(dims), cint(k)),
-                            weights.device)
+        ws = _lib.workspace(L.mccnn_mc_conv_project_grads_workspace_bytes(
+            cint(dims), cint(k), i64(ranges.shape[0])), weights.device)
         dfeat = torch.empty_like(features)
         dw, db = torch.empty_like(weights), torch.empty_like(biases)
         t_ranges = t_order = rows = None
@@ -233,8 +233,8 @@ class _MCConvLayer(torch.autograd.Function):
         # kernel-MLP gradients
         dproj = _projection_grad_product(dout, dense)
         L = _lib.lib()
-        ws = _lib.workspace(L.mccnn_mc_conv_project_grads_workspace_bytes(cint(dims), cint(k)),
-                            weights.device)
+        ws = _lib.workspace(L.mccnn_mc_conv_project_grads_workspace_bytes(
+            cint(dims), cint(k), i64(n)), weights.device)
         dw, db = torch.empty_like(weights), torch.empty_like(biases)
         _lib.call("mc_conv_project_grads", stream(), cint(dims), i64(feats.shape[0]),
                   ptr(view.points_in, _F32), cint(c), ptr(feats, _F32), i64(n),
