@@ -181,6 +181,9 @@ def per_op_times(torch, pc, layers, synthetic, _lib, radius=0.04, reps=5):
         from tensorflow_graphics_point_clouds_amd import tfg_custom_ops as tfg
         tfg.compute_pdf_pt_grads(pts, nbh._neighbors, nbh._samples_neigh_ranges,
                                  torch.full((3,), 5.0, device="cuda"), nbh._inv_radii, g, 0)
+        tfg.compute_pdf_pt_grads(pts, nbh._neighbors, nbh._samples_neigh_ranges,
+                                 torch.full((3,), 5.0, device="cuda"), nbh._inv_radii, g, 0,
+                                 symmetric=True)
         pc.sample(nbh, "poisson")
         pc.sample(nbh, "average")
         layers.MaxPooling()(feats, cloud, None, radius, neighborhood=nbh)
@@ -206,6 +209,7 @@ def per_op_times(torch, pc, layers, synthetic, _lib, radius=0.04, reps=5):
         "find_neighbors_fill": N * (4 * D) + N * (4 * D) + 8 * M,
         "compute_pdf": N * 4 * D + 8 * M + 4 * N + M * 4 * D + 4 * N,
         "compute_pdf_pt_grads": N * 4 * D + 8 * M + 8 * N + M * 4 * D + 2 * N * 4 * D,
+        "compute_pdf_pt_grads_symmetric": N * 4 * D + 8 * M + 8 * N + M * (4 * D + 4) + N * 4 * D,
         "local_pool": 4 * M * 64 + 8 * M + 4 * N * 64,
     }
     out = {"workload": "4x200k uniform, r=%.2f, self neighbourhood, %d pairs; pooling C=64"

@@ -181,6 +181,21 @@ int mccnn_compute_pdf_pt_grads(mccnn_stream_t stream, int64_t num_pts,
                                int64_t pdf_grads_len, const float *pdf_grads,
                                int mode, float *pt_grads_out);
 
+/* ComputePdfPtGrads for a symmetric pair table (j in N(c) <=> c in N(j)), which
+ * an untruncated self-neighbourhood is: the same gradient as a pure gather,
+ *   grad[c] = sum_{j in N(c)} (pdf_grads_c + pdf_grads_j) * d k_cj / d x_c,
+ * without atomics and in a fixed summation order.  The caller vouches for the
+ * symmetry; same arguments as mccnn_compute_pdf_pt_grads.  No counterpart in
+ * the reference, whose kernel scatters with atomics
+ * (compute_pdf_kernels.cu.cc:193-199). */
+int mccnn_compute_pdf_pt_grads_symmetric(
+    mccnn_stream_t stream, int64_t num_pts, int num_dims, const float *points,
+    int64_t num_neighbors, int neighbors_rank, int neighbors_cols,
+    const int32_t *neighbors, int64_t num_samples, const int32_t *ranges,
+    int inv_bandwidth_len, const float *inv_bandwidth, int inv_radii_len,
+    const float *inv_radii, int64_t pdf_grads_len, const float *pdf_grads,
+    int mode, float *pt_grads_out);
+
 /* ----------------------------------------------------------- basis_proj --- */
 
 /* BasisProj: basis_proj/cc/ops/basis_proj_ops.cpp:25-131.

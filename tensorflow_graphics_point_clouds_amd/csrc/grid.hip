@@ -116,41 +116,76 @@ __global__ void aabb_init_kernel(int count, unsigned *mn, unsigned *mx) {
   }
 }
 
-// One atomic per wave and dimension when the wave's points belong to one cloud
-// (the usual layout: clouds stored one after another), else one per lane.
+// A wavefront walks a run of kAabbRun points.  While the 64 points of an
+// iteration belong to one cloud (the usual layout: clouds stored one after
+// another) the lanes keep running minima / maxima in registers; they are reduced
+// over the wavefront and sent as one atomic per dimension when the cloud changes
+// or the run ends.  Iterations that straddle two clouds use one atomic per lane.
+constexpr int kAabbRun = 1024;
+
+template <int D>
+__device__ __forceinline__ void aabb_flush(int b, float *lo, float *hi, unsigned *mn,
+                                           unsigned *mx) {
+#pragma unroll
+  for (int d = 0; d < D; ++d) {
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) {
+      lo[d] = fminf(lo[d], __shfl_xor(lo[d], off, kWave));
+      hi[d] = fmaxf(hi[d], __shfl_xor(hi[d], off, kWave));
+    }
+    if (lane_id() == 0) {
+      atomicMin(&mn[(int64_t)b * D + d], enc_float(lo[d]));
+      atomicMax(&mx[(int64_t)b * D + d], enc_float(hi[d]));
+    }
+    lo[d] = FLT_MAX;
+    hi[d] = -FLT_MAX;
+  }
+}
+
 template <int D>
 __global__ void __launch_bounds__(256) aabb_reduce_kernel(
     int64_t n, const float *__restrict__ pts, const int *__restrict__ bids,
     unsigned *mn, unsigned *mx) {
-  const int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x;
-  const bool live = i < n;
-  const int b = live ? bids[i] : -1;
-  float p[D];
+  const int64_t wave = blockIdx.x * (int64_t)(blockDim.x / kWave) + threadIdx.x / kWave;
+  const int64_t first = wave * kAabbRun;
+  const int64_t last = first + kAabbRun < n ? first + kAabbRun : n;
+  float lo[D], hi[D];
 #pragma unroll
-  for (int d = 0; d < D; ++d) p[d] = live ? pts[i * D + d] : 0.f;
-  const int b0 = __shfl(b, 0, kWave);
-  const bool uniform = __all(b == b0 || !live) && b0 >= 0;
-  if (uniform) {
+  for (int d = 0; d < D; ++d) {
+    lo[d] = FLT_MAX;
+    hi[d] = -FLT_MAX;
+  }
+  int cur = -1;                     // cloud of the running minima / maxima (wave-uniform)
+  for (int64_t base = first; base < last; base += kWave) {
+    const int64_t i = base + lane_id();
+    const bool live = i < last;
+    const int b = live ? bids[i] : -1;
+    float p[D];
 #pragma unroll
-    for (int d = 0; d < D; ++d) {
-      float lo = live ? p[d] : FLT_MAX, hi = live ? p[d] : -FLT_MAX;
-#pragma unroll
-      for (int off = kWave / 2; off > 0; off >>= 1) {
-        lo = fminf(lo, __shfl_xor(lo, off, kWave));
-        hi = fmaxf(hi, __shfl_xor(hi, off, kWave));
+    for (int d = 0; d < D; ++d) p[d] = live ? pts[i * D + d] : 0.f;
+    const int b0 = __shfl(b, 0, kWave);
+    const bool uniform = __all(b == b0 || !live) && b0 >= 0;
+    if (uniform) {
+      if (b0 != cur) {
+        if (cur >= 0) aabb_flush<D>(cur, lo, hi, mn, mx);
+        cur = b0;
       }
-      if (lane_id() == 0) {
-        atomicMin(&mn[(int64_t)b0 * D + d], enc_float(lo));
-        atomicMax(&mx[(int64_t)b0 * D + d], enc_float(hi));
-      }
-    }
-  } else if (live) {
+      if (live) {
 #pragma unroll
-    for (int d = 0; d < D; ++d) {
-      atomicMin(&mn[(int64_t)b * D + d], enc_float(p[d]));
-      atomicMax(&mx[(int64_t)b * D + d], enc_float(p[d]));
+        for (int d = 0; d < D; ++d) {
+          lo[d] = fminf(lo[d], p[d]);
+          hi[d] = fmaxf(hi[d], p[d]);
+        }
+      }
+    } else if (live) {
+#pragma unroll
+      for (int d = 0; d < D; ++d) {
+        atomicMin(&mn[(int64_t)b * D + d], enc_float(p[d]));
+        atomicMax(&mx[(int64_t)b * D + d], enc_float(p[d]));
+      }
     }
   }
+  if (cur >= 0) aabb_flush<D>(cur, lo, hi, mn, mx);
 }
 
 // min - 1e-9f, max + 1e-9f, grid shape, scaled minimum and reciprocal cell size,
@@ -279,7 +314,8 @@ extern "C" int mccnn_grid_setup(mccnn_stream_t stream, int64_t num_pts, int num_
   if (num_pts > 0) {
     MCCNN_REQUIRE(points && batch_ids, "grid_setup received a null tensor");
     MCCNN_DIM_SWITCH(num_dims, hipLaunchKernelGGL(aabb_reduce_kernel<D>,
-                                                  dim3(blocks_for(num_pts, 256)), dim3(256), 0,
+                                                  dim3(blocks_for(num_pts, 4 * kAabbRun)),
+                                                  dim3(256), 0,
                                                   as_stream(stream), num_pts, points, batch_ids,
                                                   (unsigned *)aabb_min_out,
                                                   (unsigned *)aabb_max_out));

@@ -112,6 +112,51 @@ __global__ void __launch_bounds__(kPdfThreads) compute_pdf_grads_kernel(
   }
 }
 
+// The same gradient when the pair table is symmetric (j in N(c) <=> c in N(j), as
+// in an untruncated self-neighbourhood: the distance test is exact under
+// negation).  The term centre j adds to grad[c] through its pair (c, j) equals
+// pdf_grad_j * k_cj * u_cj * s, so
+//   grad[c] = sum_{j in N(c)} (pdf_grad_c + pdf_grad_j) * k_cj * u_cj * s
+// is a pure gather: no atomics, no zero fill, fixed summation order.
+template <int D>
+__global__ void __launch_bounds__(kPdfThreads) compute_pdf_grads_symmetric_kernel(
+    int64_t n, const float *__restrict__ pts, const int2 *__restrict__ nbrs,
+    const int *__restrict__ ranges, const float *__restrict__ inv_bw,
+    const float *__restrict__ inv_r, const float *__restrict__ pdf_grads, int mode,
+    float *__restrict__ grads) {
+  const PdfScale<D> sc = load_pdf_scale<D>(inv_bw, inv_r, mode, n);
+  const int sub = threadIdx.x & (kPdfGroup - 1);
+  const int64_t c = (int64_t)blockIdx.x * kPdfCentresPerBlock + threadIdx.x / kPdfGroup;
+  if (c >= n) return;
+  float p[D], own[D];
+#pragma unroll
+  for (int d = 0; d < D; ++d) {
+    p[d] = pts[c * D + d];
+    own[d] = 0.0f;
+  }
+  const float up = pdf_grads[c];
+  const int64_t a = c > 0 ? ranges[c - 1] : 0, b = ranges[c];
+  for (int64_t m = a + sub; m < b; m += kPdfGroup) {
+    const int64_t j = nbrs[m].x;
+    float u[D], e = 0.0f;
+#pragma unroll
+    for (int d = 0; d < D; ++d) {
+      u[d] = (pts[j * D + d] - p[d]) * sc.s[d];
+      e += u[d] * u[d];
+    }
+    const float local = (up + pdf_grads[j]) * sc.norm * expf(-0.5f * e);
+#pragma unroll
+    for (int d = 0; d < D; ++d) own[d] += u[d] * sc.s[d] * local;
+  }
+#pragma unroll
+  for (int d = 0; d < D; ++d) {
+    float v = own[d];
+#pragma unroll
+    for (int off = kPdfGroup / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+    if (sub == 0) grads[c * D + d] = v;
+  }
+}
+
 static int check_pdf_args(const char *op, int64_t num_pts, int num_dims, int neighbors_rank,
                           int neighbors_cols, int64_t num_samples, int inv_bandwidth_len,
                           int inv_radii_len, int mode) {
@@ -157,15 +202,14 @@ extern "C" int mccnn_compute_pdf(mccnn_stream_t stream, int64_t num_pts, int num
   return MCCNN_OK;
 }
 
-extern "C" int mccnn_compute_pdf_pt_grads(mccnn_stream_t stream, int64_t num_pts, int num_dims,
-                                          const float *points, int64_t num_neighbors,
-                                          int neighbors_rank, int neighbors_cols,
-                                          const int32_t *neighbors, int64_t num_samples,
-                                          const int32_t *ranges, int inv_bandwidth_len,
-                                          const float *inv_bandwidth, int inv_radii_len,
-                                          const float *inv_radii, int64_t pdf_grads_len,
-                                          const float *pdf_grads, int mode,
-                                          float *pt_grads_out) {
+static int pdf_pt_grads_impl(mccnn_stream_t stream, int64_t num_pts, int num_dims,
+                             const float *points, int64_t num_neighbors, int neighbors_rank,
+                             int neighbors_cols, const int32_t *neighbors, int64_t num_samples,
+                             const int32_t *ranges, int inv_bandwidth_len,
+                             const float *inv_bandwidth, int inv_radii_len,
+                             const float *inv_radii, int64_t pdf_grads_len,
+                             const float *pdf_grads, int mode, bool symmetric,
+                             float *pt_grads_out) {
   int rc = check_pdf_args("ComputePdfPtGrads", num_pts, num_dims, neighbors_rank, neighbors_cols,
                           num_samples, inv_bandwidth_len, inv_radii_len, mode);
   if (rc != MCCNN_OK) return rc;
@@ -178,13 +222,49 @@ extern "C" int mccnn_compute_pdf_pt_grads(mccnn_stream_t stream, int64_t num_pts
                     (neighbors || num_neighbors == 0),
                 "ComputePdfPtGrads received a null tensor");
   hipStream_t s = as_stream(stream);
+  const unsigned grid = blocks_for(num_pts, kPdfCentresPerBlock);
+  if (symmetric) {
+    MCCNN_DIM_SWITCH(num_dims,
+                     hipLaunchKernelGGL(compute_pdf_grads_symmetric_kernel<D>, dim3(grid),
+                                        dim3(kPdfThreads), 0, s, num_pts, points,
+                                        (const int2 *)neighbors, ranges, inv_bandwidth, inv_radii,
+                                        pdf_grads, mode, pt_grads_out));
+    MCCNN_LAUNCH_CHECK();
+    return MCCNN_OK;
+  }
   rc = fill_zero(s, pt_grads_out, sizeof(float) * (size_t)num_pts * num_dims);
   if (rc != MCCNN_OK) return rc;
-  const unsigned grid = blocks_for(num_pts, kPdfCentresPerBlock);
   MCCNN_DIM_SWITCH(num_dims, hipLaunchKernelGGL(compute_pdf_grads_kernel<D>, dim3(grid),
                                                 dim3(kPdfThreads), 0, s, num_pts, points,
                                                 (const int2 *)neighbors, ranges, inv_bandwidth,
                                                 inv_radii, pdf_grads, mode, pt_grads_out));
   MCCNN_LAUNCH_CHECK();
   return MCCNN_OK;
+}
+
+extern "C" int mccnn_compute_pdf_pt_grads(mccnn_stream_t stream, int64_t num_pts, int num_dims,
+                                          const float *points, int64_t num_neighbors,
+                                          int neighbors_rank, int neighbors_cols,
+                                          const int32_t *neighbors, int64_t num_samples,
+                                          const int32_t *ranges, int inv_bandwidth_len,
+                                          const float *inv_bandwidth, int inv_radii_len,
+                                          const float *inv_radii, int64_t pdf_grads_len,
+                                          const float *pdf_grads, int mode,
+                                          float *pt_grads_out) {
+  return pdf_pt_grads_impl(stream, num_pts, num_dims, points, num_neighbors, neighbors_rank,
+                           neighbors_cols, neighbors, num_samples, ranges, inv_bandwidth_len,
+                           inv_bandwidth, inv_radii_len, inv_radii, pdf_grads_len, pdf_grads, mode,
+                           false, pt_grads_out);
+}
+
+extern "C" int mccnn_compute_pdf_pt_grads_symmetric(
+    mccnn_stream_t stream, int64_t num_pts, int num_dims, const float *points,
+    int64_t num_neighbors, int neighbors_rank, int neighbors_cols, const int32_t *neighbors,
+    int64_t num_samples, const int32_t *ranges, int inv_bandwidth_len,
+    const float *inv_bandwidth, int inv_radii_len, const float *inv_radii,
+    int64_t pdf_grads_len, const float *pdf_grads, int mode, float *pt_grads_out) {
+  return pdf_pt_grads_impl(stream, num_pts, num_dims, points, num_neighbors, neighbors_rank,
+                           neighbors_cols, neighbors, num_samples, ranges, inv_bandwidth_len,
+                           inv_bandwidth, inv_radii_len, inv_radii, pdf_grads_len, pdf_grads, mode,
+                           true, pt_grads_out);
 }

@@ -33,6 +33,62 @@ __global__ void __launch_bounds__(kPoolThreads) local_pool_kernel(
   }
 }
 
+// One wavefront per centre for C = 4 * 2^q <= 256 channels: a feature row is read
+// by C/4 lanes with 16-byte loads, so one load instruction fetches 256/C rows; the
+// neighbour indices are read 64 at a time and passed around by lane shuffle, four
+// row loads are in flight per lane.  The partial results of the lane groups are
+// combined by butterfly shuffles at the end.
+template <bool kMax>
+__global__ void __launch_bounds__(kPoolThreads) local_pool_rows_kernel(
+    int64_t n_out, int C, int lpr_log2, const float *__restrict__ feat,
+    const int2 *__restrict__ nbrs, const int *__restrict__ ranges, float *__restrict__ out) {
+  const int64_t centre = (int64_t)blockIdx.x * (kPoolThreads / kWave) + threadIdx.x / kWave;
+  if (centre >= n_out) return;
+  const int lane = lane_id();
+  const int lpr = 1 << lpr_log2;                 // lanes per row
+  const int slot = lane >> lpr_log2, colv = lane & (lpr - 1);
+  const int slots = kWave >> lpr_log2;           // rows per load instruction
+  const int a = centre > 0 ? ranges[centre - 1] : 0, b = ranges[centre];
+  const float init = kMax ? -FLT_MAX : 0.0f;
+  float4 acc = make_float4(init, init, init, init);
+  const float *fl = feat + 4 * colv;
+  for (int m0 = a; m0 < b; m0 += kWave) {
+    const int cnt = b - m0 < kWave ? b - m0 : kWave;
+    const int myidx = nbrs[m0 + (lane < cnt ? lane : 0)].x;
+    for (int t0 = 0; t0 < cnt; t0 += 4 * slots) {      // uniform trip count: shuffles inside
+      float4 v[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int n = t0 + slot + u * slots;
+        const int idx = __shfl(myidx, n < cnt ? n : 0, kWave);   // past the end: repeat pair 0
+        v[u] = *reinterpret_cast<const float4 *>(fl + (int64_t)idx * C);
+        if (!kMax && n >= cnt) v[u] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        acc.x = kMax ? fmaxf(acc.x, v[u].x) : acc.x + v[u].x;
+        acc.y = kMax ? fmaxf(acc.y, v[u].y) : acc.y + v[u].y;
+        acc.z = kMax ? fmaxf(acc.z, v[u].z) : acc.z + v[u].z;
+        acc.w = kMax ? fmaxf(acc.w, v[u].w) : acc.w + v[u].w;
+      }
+    }
+  }
+  for (int off = lpr; off < kWave; off <<= 1) {
+    const float x = __shfl_xor(acc.x, off, kWave), y = __shfl_xor(acc.y, off, kWave);
+    const float z = __shfl_xor(acc.z, off, kWave), w = __shfl_xor(acc.w, off, kWave);
+    acc.x = kMax ? fmaxf(acc.x, x) : acc.x + x;
+    acc.y = kMax ? fmaxf(acc.y, y) : acc.y + y;
+    acc.z = kMax ? fmaxf(acc.z, z) : acc.z + z;
+    acc.w = kMax ? fmaxf(acc.w, w) : acc.w + w;
+  }
+  if (slot != 0) return;
+  if (!kMax) {
+    const float inv = 1.0f / (float)(b - a > 0 ? b - a : 1);
+    acc.x *= inv; acc.y *= inv; acc.z *= inv; acc.w *= inv;
+  }
+  *reinterpret_cast<float4 *>(out + centre * C + 4 * colv) = acc;
+}
+
 template <bool kMax>
 __global__ void __launch_bounds__(kPoolThreads) local_pool_grads_kernel(
     int64_t n_out, int C, int lanes, const float *__restrict__ feat,
@@ -179,6 +235,23 @@ extern "C" int mccnn_local_pool(mccnn_stream_t stream, int kind, int64_t num_pts
   if (num_samples == 0) return MCCNN_OK;
   MCCNN_REQUIRE(ranges && out && (num_neighbors == 0 || (features && neighbors)),
                 "local_pool received a null tensor");
+  // C = 4 * 2^q <= 256: row-vectorised kernel, one wavefront per centre
+  int lpr_log2 = -1;
+  for (int q = 0; q <= 6; ++q)
+    if (num_features == (4 << q)) lpr_log2 = q;
+  if (lpr_log2 >= 0) {
+    const unsigned wgrid = blocks_for(num_samples, kPoolThreads / kWave);
+    if (kind == 0)
+      hipLaunchKernelGGL(local_pool_rows_kernel<true>, dim3(wgrid), dim3(kPoolThreads), 0,
+                         as_stream(stream), num_samples, num_features, lpr_log2, features,
+                         (const int2 *)neighbors, ranges, out);
+    else
+      hipLaunchKernelGGL(local_pool_rows_kernel<false>, dim3(wgrid), dim3(kPoolThreads), 0,
+                         as_stream(stream), num_samples, num_features, lpr_log2, features,
+                         (const int2 *)neighbors, ranges, out);
+    MCCNN_LAUNCH_CHECK();
+    return MCCNN_OK;
+  }
   const int lanes = lanes_for(num_features);
   const unsigned grid = blocks_for(num_samples, kPoolThreads / lanes);
   if (kind == 0)

@@ -255,7 +255,8 @@ class Neighborhood:
             bw = _as_vector(bandwidth, d, dev)
             self._pdf_per_point = tfg_custom_ops.compute_pdf_with_pt_grads(
                 self._grid._sorted_points, nbh._neighbors, nbh._samples_neigh_ranges,
-                torch.reciprocal(bw), nbh._inv_radii, mode.value)
+                torch.reciprocal(bw), nbh._inv_radii, mode.value,
+                symmetric=nbh._equal_samples and nbh.max_neighbors == 0)
             self._pdf = torch.empty(self._neighbors.shape[0], dtype=_F32, device=dev)
             _lib.call("gather_pdf", stream(), i64(self._neighbors.shape[0]), ptr(self._neighbors, _I32),
                 ptr(self._pdf_per_point.detach(), _F32), ptr(self._pdf))

@@ -120,11 +120,12 @@ def _compute_pdf_raw(points, neighbors, ranges, inv_bandwidth, inv_radii, mode):
 
 
 def compute_pdf_pt_grads(points, neighbors, sample_neigh_indices, inv_bandwidth, inv_radii,
-                         pdf_grads, mode):
+                         pdf_grads, mode, symmetric=False):
     """ComputePdfPtGrads (compute_pdf_ops.cpp:58-74): [N, D] gradient of
-    sum(pdf_grads * pdf) with respect to the points."""
+    sum(pdf_grads * pdf) with respect to the points.  `symmetric=True` (the caller
+    vouches that j in N(c) <=> c in N(j)) selects the atomic-free gather."""
     out = torch.empty_like(points)
-    _lib.call("compute_pdf_pt_grads", stream(), i64(points.shape[0]), cint(_dim(points, 1)), ptr(points, _F32),
+    _lib.call("compute_pdf_pt_grads_symmetric" if symmetric else "compute_pdf_pt_grads", stream(), i64(points.shape[0]), cint(_dim(points, 1)), ptr(points, _F32),
         i64(neighbors.shape[0]), cint(neighbors.dim()), cint(_dim(neighbors, 1)),
         ptr(neighbors, _I32), i64(sample_neigh_indices.shape[0]),
         ptr(sample_neigh_indices, _I32), cint(inv_bandwidth.shape[0]),
@@ -135,25 +136,26 @@ def compute_pdf_pt_grads(points, neighbors, sample_neigh_indices, inv_bandwidth,
 
 class _ComputePdf(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, points, neighbors, ranges, inv_bandwidth, inv_radii, mode):
+    def forward(ctx, points, neighbors, ranges, inv_bandwidth, inv_radii, mode, symmetric):
         ctx.save_for_backward(points, neighbors, ranges, inv_bandwidth, inv_radii)
-        ctx.mode = mode
+        ctx.mode, ctx.symmetric = mode, symmetric
         return _compute_pdf_raw(points, neighbors, ranges, inv_bandwidth, inv_radii, mode)
 
     @staticmethod
     def backward(ctx, grad):
         points, neighbors, ranges, inv_bandwidth, inv_radii = ctx.saved_tensors
         g = compute_pdf_pt_grads(points, neighbors, ranges, inv_bandwidth, inv_radii,
-                                 grad.contiguous(), ctx.mode)
-        return g, None, None, None, None, None
+                                 grad.contiguous(), ctx.mode, ctx.symmetric)
+        return g, None, None, None, None, None, None
 
 
 def compute_pdf_with_pt_grads(points, neighbors, sample_neigh_indices, inv_bandwidth,
-                              inv_radii, mode):
+                              inv_radii, mode, symmetric=False):
     """ComputePdfWithPtGrads (compute_pdf_ops.cpp:43-56): Gaussian KDE per point
-    over its neighbour list; differentiable with respect to `points`."""
+    over its neighbour list; differentiable with respect to `points`.
+    `symmetric`: see `compute_pdf_pt_grads`."""
     return _ComputePdf.apply(points, neighbors, sample_neigh_indices, inv_bandwidth,
-                             inv_radii, mode)
+                             inv_radii, mode, symmetric)
 
 
 def _basis_proj_raw(basis, features, neighbors, ranges, centre_order=None):

@@ -198,7 +198,7 @@ def test_deformable_kpconv_and_regularization(oracle, kind):
     normwise(tfeat.grad.cpu().numpy(), tf.grad.numpy(), tol=1e-4)
 
 
-@pytest.mark.parametrize("c", [1, 5, 64, 100])
+@pytest.mark.parametrize("c", [1, 4, 5, 16, 64, 100, 128, 256])
 def test_local_and_global_pooling(oracle, c):
     from tensorflow_graphics_point_clouds_amd import layers, pc
     rng = np.random.default_rng(c)

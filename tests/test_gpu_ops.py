@@ -187,6 +187,10 @@ def test_pdf_and_point_grads(ops, oracle, d, mode):
     gexp = oracle.compute_pdf_pt_grads(g.sorted_points, nbh.neighbors, nbh.ranges, inv_bw,
                                        nbh.inv_radii, up, mode)
     assert_normwise(sp.grad.cpu().numpy(), gexp)
+    # the atomic-free form for symmetric pair tables (a self-neighbourhood is one)
+    sym = ops.compute_pdf_pt_grads(sp.detach(), dev(nbh.neighbors), dev(nbh.ranges), dev(inv_bw),
+                                   dev(nbh.inv_radii), dev(up), mode, symmetric=True)
+    assert_normwise(sym.cpu().numpy(), gexp)
 
 
 # ------------------------------------------------------------- basis_proj ----
