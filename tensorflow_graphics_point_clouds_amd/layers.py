@@ -362,6 +362,73 @@ class MCConv(torch.nn.Module):
         return torch.bmm(p, self.final_weights).permute(1, 0, 2).reshape(n, -1)
 
 
+class PointConv(torch.nn.Module):
+    """PointConv-style Monte-Carlo convolution (pylib/pc/layers/PointConv.py:34-292):
+    one kernel MLP with a single hidden layer on the unscaled point offsets, the
+    densities normalised by their maximum in each neighbourhood and passed
+    through a 1 -> 16 -> 1 MLP before they divide the basis."""
+
+    def __init__(self, num_features_in, num_features_out, num_dims, size_hidden=32,
+                 non_linearity_type="relu", device="cuda", seed=0, weights=None, biases=None,
+                 final_weights=None, pdf_weights=None, pdf_biases=None):
+        super().__init__()
+        if size_hidden not in (8, 16, 32):
+            raise ValueError("size_hidden must be 8, 16 or 32")
+        self._num_features_in, self._num_features_out = num_features_in, num_features_out
+        self._num_dims, self._size_hidden = num_dims, size_hidden
+        self._act = _ACTIVATIONS[non_linearity_type.lower()]
+        gen = torch.Generator().manual_seed(seed)
+
+        def glorot(fan_in, fan_out):          # GlorotNormal, PointConv.py:83-85
+            return (torch.randn((fan_in, fan_out), generator=gen) *
+                    math.sqrt(2.0 / (fan_in + fan_out))).to(device)
+
+        def param(value, default):
+            value = default() if value is None else torch.as_tensor(value).to(device)
+            return torch.nn.Parameter(value.to(_F32).contiguous())
+
+        self.weights = param(weights, lambda: glorot(num_dims, size_hidden))
+        self.biases = param(biases, lambda: torch.zeros((1, size_hidden), device=device))
+        self.final_weights = param(final_weights, lambda: glorot(size_hidden * num_features_in,
+                                                                 num_features_out))
+        pw = pdf_weights or (None, None)
+        pb = pdf_biases or (None, None)
+        self.pdf_weights_1 = param(pw[0], lambda: glorot(1, 16))
+        self.pdf_weights_2 = param(pw[1], lambda: glorot(16, 1))
+        self.pdf_biases_1 = param(pb[0], lambda: torch.zeros((1, 16), device=device))
+        self.pdf_biases_2 = param(pb[1], lambda: torch.zeros((1, 1), device=device))
+        self.last_neighborhood = None
+
+    def forward(self, features, point_cloud_in, point_cloud_out, radius, neighborhood=None,
+                bandwidth=0.2):
+        d, dev = self._num_dims, features.device
+        radii = pc._as_vector(radius, d, dev)
+        if neighborhood is None:
+            grid = pc.Grid(point_cloud_in, radii)
+            neighborhood = pc.Neighborhood(grid, radii, point_cloud_out)
+        self.last_neighborhood = neighborhood
+        pdf = neighborhood.get_pdf(bandwidth=bandwidth, mode=pc.KDEMode.constant)
+        ids, ranges = neighborhood._original_neigh_ids, neighborhood._samples_neigh_ranges
+        m, n_out = ids.shape[0], ranges.shape[0]
+        # hidden layer on the unscaled offsets (PointConv.py:268-272): unit radii, unit pdf
+        ones_d = torch.ones(d, dtype=_F32, device=dev)
+        hidden = _MCBasis.apply(self.weights.reshape(1, d, self._size_hidden),
+                                self.biases.reshape(1, self._size_hidden),
+                                point_cloud_in._points, point_cloud_out._points, ids, ones_d,
+                                torch.ones(m, dtype=_F32, device=dev), self._act)
+        # densities relative to the largest of their neighbourhood, then the pdf MLP
+        # (PointConv.py:166-177)
+        centre = ids[:, 1].long()
+        max_pdf = torch.zeros(n_out, dtype=_F32, device=dev).scatter_reduce(
+            0, centre, pdf, "amax", include_self=False)
+        rel = (pdf / max_pdf[centre]).reshape(-1, 1)
+        cur = torch.relu(rel @ self.pdf_weights_1 + self.pdf_biases_1)
+        cur = cur @ self.pdf_weights_2 + self.pdf_biases_2
+        basis = hidden / cur
+        proj = tfg_custom_ops.basis_proj(basis, features.contiguous(), ids, ranges)
+        return proj.reshape(n_out, -1) @ self.final_weights
+
+
 def _padded_basis_count(num_kernel_points):
     for k in (8, 16, 32, 64):
         if num_kernel_points <= k:

@@ -199,6 +199,7 @@ class Neighborhood:
         self._transposed_table = None
         self._transposed_pdf = None
         self._sorted_view = None
+        self._transposed = None
 
     def transposed_pairs(self):
         """(point_ranges, pair_order): the pairs grouped by neighbour point, used by
@@ -227,6 +228,22 @@ class Neighborhood:
                 self._transposed_pdf = (key, pdf[pair_order.long()].contiguous())
             pdf_t = self._transposed_pdf[1]
         return self._transposed_table, point_ranges, pdf_t
+
+    def get_grid(self):
+        """The grid used for the neighbour search (Neighborhood.py:313-316)."""
+        return self._grid
+
+    def transpose(self):
+        """The neighbourhood with centres and neighbour points switched
+        (Neighborhood.py:318-329): itself for a self-neighbourhood, otherwise a
+        grid over the centres searched from the original points; built once."""
+        if self._transposed is None:
+            if self._equal_samples:
+                self._transposed = self
+            else:
+                grid = Grid(self._point_cloud_sampled, self._radii)
+                self._transposed = Neighborhood(grid, self._radii, self._grid._point_cloud)
+        return self._transposed
 
     def sorted_view(self):
         """The neighbourhood re-expressed in grid order on both sides (built on
@@ -306,3 +323,17 @@ class PointHierarchy:
             self._neighborhoods.append(nbh)
             self._point_clouds.append(cur)
             self._sample_indices.append(idx)
+
+    def get_neighborhood(self, i=None, transposed=False):
+        """Neighbourhood between level i and i+1, or all of them
+        (PointHierarchy.py:159-183); `transposed` gives level i+1 -> i."""
+        if i is None:
+            return [nb.transpose() for nb in self._neighborhoods] if transposed \
+                else self._neighborhoods
+        return self._neighborhoods[i].transpose() if transposed else self._neighborhoods[i]
+
+    def __getitem__(self, index):
+        return self._point_clouds[index]
+
+    def __len__(self):
+        return len(self._point_clouds)
