@@ -504,6 +504,71 @@ class _KPRegularization(torch.autograd.Function):
         return (doff * grad,) + (None,) * 8
 
 
+def _kp_basis_raw(points_in, points_out, neighbors, inv_radii, kernel_points, k, kind, sigma):
+    kp, dims = kernel_points.shape
+    basis = torch.empty((neighbors.shape[0], k), dtype=_F32, device=points_in.device)
+    _lib.call("kp_basis", stream(), i64(neighbors.shape[0]), cint(dims), cint(kp), cint(k),
+              cint(kind), cfloat(sigma), ptr(points_in, _F32), ptr(points_out, _F32),
+              ptr(neighbors, _I32), ptr(inv_radii, _F32), ptr(kernel_points, _F32), ptr(None),
+              ptr(basis), ptr(None))
+    return basis
+
+
+class _KPConvRigidLayer(torch.autograd.Function):
+    """Rigid kernel-point convolution (KPConv.py:165-232) on the neighbourhood's
+    grid-ordered view.  As for the Monte-Carlo convolution, the feature gradient is
+    the same convolution run from the centres back to the points over the
+    transposed pair table, with the kernel-point weights re-evaluated there
+    (offset negated), and the weight gradient is feat^T Q; nothing is scattered and
+    the basis gradient, which a rigid kernel does not need, is never formed."""
+
+    @staticmethod
+    def forward(ctx, dense_weights, features, neighborhood, inv_radii, kernel_points, k, kind,
+                sigma):
+        view = neighborhood.sorted_view()
+        with _lib.region("permute_rows"):
+            feats = features.index_select(0, view.point_order)
+        basis = _kp_basis_raw(view.points_in, view.points_out, view.table, inv_radii,
+                              kernel_points, k, kind, sigma)
+        proj = tfg_custom_ops._basis_proj_raw(basis, feats, view.table, view.ranges)
+        del basis
+        with _lib.region("gemm_out"):
+            out = proj.reshape(proj.shape[0], -1) @ dense_weights
+        if view.centre_order is not None:
+            with _lib.region("permute_rows"):
+                out = torch.empty_like(out).index_copy_(0, view.centre_order, out)
+        ctx.save_for_backward(dense_weights, feats, inv_radii, kernel_points)
+        ctx.neighborhood, ctx.k, ctx.kind, ctx.sigma = neighborhood, k, kind, sigma
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        dense, feats, inv_radii, kernel_points = ctx.saved_tensors
+        view = ctx.neighborhood.sorted_view()
+        k, c, f = ctx.k, feats.shape[1], dense.shape[1]
+        if view.centre_order is not None:
+            with _lib.region("permute_rows"):
+                dout = dout.index_select(0, view.centre_order)
+        else:
+            dout = dout.contiguous()
+        basis_t = _kp_basis_raw(view.points_out, view.points_in, view.table_t, -inv_radii,
+                                kernel_points, k, ctx.kind, ctx.sigma)
+        q = tfg_custom_ops._basis_proj_raw(basis_t, dout, view.table_t, view.ranges_t)
+        del basis_t
+        q = q.reshape(feats.shape[0], f * k)
+        dfeat = ddense = None
+        if ctx.needs_input_grad[1]:
+            w2 = dense.reshape(c, k, f).permute(2, 1, 0).reshape(f * k, c)
+            with _lib.region("gemm_dfeat"):
+                dfeat = q @ w2
+            with _lib.region("permute_rows"):
+                dfeat = torch.empty_like(dfeat).index_copy_(0, view.point_order, dfeat)
+        if ctx.needs_input_grad[0]:
+            ddense = _weight_grad_product(feats, q).reshape(c, f, k).permute(0, 2, 1)
+            ddense = ddense.reshape(c * k, f)
+        return ddense, dfeat, None, None, None, None, None, None
+
+
 class KPConv(torch.nn.Module):
     """Kernel-point convolution, rigid or deformable
     (pylib/pc/layers/KPConv.py:60-429).  The kernel points are scaled by 0.75 as
@@ -514,7 +579,7 @@ class KPConv(torch.nn.Module):
 
     def __init__(self, num_features_in, num_features_out, kernel_points, num_dims=3,
                  kernel_weighting="linear", weights=None, deformable=False,
-                 offset_weights=None, device="cuda", seed=0):
+                 offset_weights=None, device="cuda", seed=0, transposed_grads=True):
         super().__init__()
         kp = torch.as_tensor(kernel_points, dtype=_F32).to(device) * 0.75
         self._kernel_points = kp.contiguous()
@@ -534,6 +599,8 @@ class KPConv(torch.nn.Module):
             weights = glorot(fan_in, num_features_out)
         self.weights = torch.nn.Parameter(weights.to(_F32).contiguous())
         self.deformable = deformable
+        # rigid kernels: feature gradient as a convolution over the transposed pair table
+        self.transposed_grads = transposed_grads
         if deformable:
             if offset_weights is None:
                 offset_weights = glorot(fan_in, self._num_kernel_points * num_dims)
@@ -561,6 +628,10 @@ class KPConv(torch.nn.Module):
         ids, ranges = neighborhood._original_neigh_ids, neighborhood._samples_neigh_ranges
         kp, k, c = self._num_kernel_points, self._num_basis, self._num_features_in
         features = features.contiguous()
+        if not self.deformable and self.transposed_grads:
+            return _KPConvRigidLayer.apply(self._padded(self.weights), features, neighborhood,
+                                           torch.reciprocal(radii), self._kernel_points, k,
+                                           self._kind, sigma)
         transposed = None
         if features.requires_grad and tfg_custom_ops.gathered_grads_supported(c, k):
             transposed = neighborhood.transposed_pairs()

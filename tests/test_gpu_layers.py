@@ -146,8 +146,9 @@ def test_pointconv_forward_backward(oracle, hidden, act):
     normwise(conv.pdf_biases_2.grad.cpu().numpy(), t["pb2"].grad.numpy(), tol=5e-5)
 
 
+@pytest.mark.parametrize("transposed", [True, False])
 @pytest.mark.parametrize("kind,influence", [("linear", None), ("gaussian", 0.3 * 0.15)])
-def test_kpconv_forward_backward(oracle, kind, influence):
+def test_kpconv_forward_backward(oracle, kind, influence, transposed):
     from tensorflow_graphics_point_clouds_amd import layers, pc, synthetic
     rng = np.random.default_rng(5)
     batch, radius, c_in, c_out = 2, 0.15, 16, 24
@@ -165,7 +166,8 @@ def test_kpconv_forward_backward(oracle, kind, influence):
     proj = oracle.basis_proj(padded, feat, ids, nbh.ranges)[:, :, :15]
     expect = proj.reshape(len(ctr), -1) @ wts.astype(np.float64)
 
-    conv = layers.KPConv(c_in, c_out, kp, kernel_weighting=kind, weights=dev(wts))
+    conv = layers.KPConv(c_in, c_out, kp, kernel_weighting=kind, weights=dev(wts),
+                         transposed_grads=transposed)
     tfeat = dev(feat).requires_grad_(True)
     out = conv(tfeat, pc.PointCloud(dev(pts), dev(bids), batch),
                pc.PointCloud(dev(ctr), dev(cb), batch), radius, kernel_influence_dist=influence)
