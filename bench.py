@@ -159,6 +159,42 @@ def cpu_baseline(synthetic, sample_points=60000):
                       "the C/OpenMP oracle with numpy GEMMs" % (n, len(ids), reps)}
 
 
+def kpconv_config5(torch, pc, layers, synthetic, _lib, steps=5):
+    """Rigid kernel-point convolution 128 -> 128, 15 kernel points (padded to 16),
+    linear correlation, fwd+bwd on the scene-scale geometry (configuration 5)."""
+    import numpy as np
+    cfg = synthetic.config5()
+    dev = lambda a: torch.as_tensor(np.ascontiguousarray(a)).cuda()
+    cloud = pc.PointCloud(dev(cfg["points"]), dev(cfg["batch_ids"]), cfg["batch_size"])
+    r = cfg["radius"]
+    nbh = pc.Neighborhood(pc.Grid(cloud, r), r, cloud)
+    N, M, C, CO = cloud._points.shape[0], nbh._neighbors.shape[0], cfg["c_in"], cfg["c_out"]
+    conv = layers.KPConv(C, CO, cfg["kernel_points"] / 0.75, kernel_weighting="linear", seed=5)
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    feats = torch.randn((N, C), device="cuda", generator=gen).requires_grad_(True)
+    up = torch.randn((N, CO), device="cuda", generator=gen)
+
+    def step():
+        conv(feats, cloud, cloud, r, neighborhood=nbh).backward(up)
+        feats.grad = None
+        conv.weights.grad = None
+
+    for _ in range(2):
+        step()
+    torch.cuda.synchronize()
+    _lib.start_timing()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / steps
+    ops = {k.replace("_ordered", ""): round(sum(v) / steps, 3)
+           for k, v in _lib.collect_timing().items()}
+    return {"workload": "config 5: KPConv %d->%d, 15 kernel points, linear, radius %.2f, "
+                        "%d points, %d pairs, fwd+bwd" % (C, CO, r, N, M),
+            "ms_per_step": ms, "points_per_s": N / (ms * 1e-3), "ops_ms": ops}
+
+
 def per_op_times(torch, pc, layers, synthetic, _lib, radius=0.04, reps=5):
     """Every op of the path on the dense case (4 x 200k uniform points, radius
     0.04): average milliseconds from HIP events around each C-ABI call, with
@@ -389,6 +425,8 @@ def main():
                                                             _lib)
         torch.cuda.empty_cache()
         result["per_op_dense_case"] = per_op_times(torch, pc, layers, synthetic, _lib)
+        torch.cuda.empty_cache()
+        result["kpconv_config5"] = kpconv_config5(torch, pc, layers, synthetic, _lib)
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(synthetic)
     else:

@@ -429,6 +429,23 @@ int mccnn_mc_conv_project_grads(
     float *pair_rows_workspace, float *feature_grads_out,
     float *weight_grads_out, float *bias_grads_out);
 
+/* Rigid kernel-point convolution projection (KPConv.py:193-224): kp_basis
+ * followed by basis_proj in one kernel, the correlation weights
+ *   kind 0: max(1 - d/sigma, 0),  kind 1: exp(-(d/(sigma/3))^2),
+ *   d = || delta - kernel_points[k] ||,  delta = (p_in[nbr] - p_out[centre]) * inv_radii
+ * evaluated in registers.  out [N_out, C, 16]; columns >= num_kernel_points are
+ * zero (the padding the reference slices off).  out_rows as for
+ * mccnn_mc_conv_project.  D in {2,3}, C in {16,32,64,128}, 1..16 kernel points.
+ * No counterpart among the reference's ops. */
+int mccnn_kp_conv_project(mccnn_stream_t stream, int num_dims, int64_t num_pts,
+                          const float *points_in, int num_features,
+                          const float *features, int64_t num_samples,
+                          const float *points_out, int64_t num_neighbors,
+                          const int32_t *neighbors, const int32_t *ranges,
+                          const float *inv_radii, int num_kernel_points,
+                          const float *kernel_points, int kind, float sigma,
+                          const int32_t *out_rows, float *out);
+
 /* The whole Monte-Carlo convolution (MCConv.py:137-194) in one kernel:
  *   out[i, f] = sum_{c,k} proj[i, c, k] * final_weights[c*K + k, f]
  * with proj as produced by mccnn_mc_conv_project; the projection is handed from

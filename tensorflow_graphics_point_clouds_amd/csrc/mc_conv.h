@@ -49,17 +49,61 @@ struct PairStage {
     default: { constexpr int ACT = MCCNN_ACT_ELU; __VA_ARGS__; } break;                          \
   }
 
+// Per-lane basis functors: the value of basis column `col` (= lane & 15) for a
+// staged pair g = (delta * inv_radii, weight), weight = 1/pdf or 1 for a live
+// pair and 0 for a padding slot.
+template <int D, int kAct>
+struct MlpBasis {                  // act(delta . W[:, col] + b[col]) / pdf   (MCConv.py:163-171)
+  float w[3], b;
+  __device__ __forceinline__ MlpBasis(const McParams<D> &p) {
+    w[0] = w[1] = w[2] = 0.0f;
+    load_weight_column<D>(p, lane_id() & 15, w, &b);
+  }
+  __device__ __forceinline__ float operator()(const float4 &g) const {
+    const float z = b + g.x * w[0] + g.y * w[1] + g.z * w[2];
+    return act_fwd(kAct, z) * g.w;
+  }
+};
+
+template <int D, int kKind>
+struct KpBasis {                   // kernel-point correlation (KPConv.py:29-57, 193-213)
+  float k[3], sigma;
+  bool live;                       // columns past the last kernel point are zero padding
+  __device__ __forceinline__ KpBasis(const float *__restrict__ kernel_points, int num_kp,
+                                     float sigma_) : sigma(sigma_) {
+    const int col = lane_id() & 15;
+    live = col < num_kp;
+    k[0] = k[1] = k[2] = 0.0f;
+#pragma unroll
+    for (int d = 0; d < D; ++d) k[d] = live ? kernel_points[col * D + d] : 0.0f;
+  }
+  __device__ __forceinline__ float operator()(const float4 &g) const {
+    const float dx = g.x - k[0], dy = g.y - k[1], dz = g.z - k[2];
+    const float dist = sqrtf(dx * dx + dy * dy + dz * dz);
+    float wgt;
+    if (kKind == 0) {
+      const float v = 1.0f - dist / sigma;
+      wgt = v > 0.0f ? v : 0.0f;
+    } else {
+      const float q = dist / (sigma / 3.0f);
+      wgt = expf(-(q * q));
+    }
+    return live ? wgt * g.w : 0.0f;
+  }
+};
+
 // acc[j] += projection of the pairs [a, b) of one centre for the channels
 // col*kCPL + j of the 16*kCPL-channel chunk starting at feat_base.  Rows are
-// row_bytes apart; every byte offset fits 32 bits (checked by the host).
-template <int kCPL, int D, int kAct>
+// row_bytes apart; every byte offset fits 32 bits (checked by the host).  p.pdf
+// may be null (weight 1).
+template <int kCPL, int D, class Basis>
 __device__ __forceinline__ void project_pairs(const char *__restrict__ feat_base,
                                               unsigned row_bytes, const int2 *__restrict__ nbrs,
                                               int a, int b, const McParams<D> &p,
-                                              const float *ctr, PairStage *stage, v4f *acc) {
+                                              const float *ctr, PairStage *stage,
+                                              const Basis &basis, v4f *acc) {
   const int lane = lane_id(), quarter = lane >> 4, col = lane & 15;
-  float wcol[3] = {0.0f, 0.0f, 0.0f}, ir[D], bcol;
-  load_weight_column<D>(p, col, wcol, &bcol);
+  float ir[D];
 #pragma unroll
   for (int d = 0; d < D; ++d) ir[d] = p.inv_radii[d];
   const unsigned lane_off = col * kCPL * 4;
@@ -72,7 +116,7 @@ __device__ __forceinline__ void project_pairs(const char *__restrict__ feat_base
       float dl[3] = {0.0f, 0.0f, 0.0f};
 #pragma unroll
       for (int d = 0; d < D; ++d) dl[d] = (p.pin[(int64_t)idx * D + d] - ctr[d]) * ir[d];
-      g = make_float4(dl[0], dl[1], dl[2], 1.0f / p.pdf[m0 + lane]);
+      g = make_float4(dl[0], dl[1], dl[2], p.pdf ? 1.0f / p.pdf[m0 + lane] : 1.0f);
       row = (unsigned)idx * row_bytes;
     }
     // unused slots of the last step point at the first pair's row with weight 0
@@ -89,8 +133,7 @@ __device__ __forceinline__ void project_pairs(const char *__restrict__ feat_base
         const float4 gn = stage->geo[n];
         const unsigned rn = stage->row[n];
         f[u] = load_vec<kCPL>(reinterpret_cast<const float *>(feat_base + rn + lane_off), true);
-        const float z = bcol + gn.x * wcol[0] + gn.y * wcol[1] + gn.z * wcol[2];
-        w[u] = act_fwd(kAct, z) * gn.w;
+        w[u] = basis(gn);
       }
 #pragma unroll
       for (int u = 0; u < kFusedUnroll; ++u)

@@ -15,11 +15,15 @@
 
 namespace mccnn {
 
-template <int kCPL, int D, int kAct>
-__global__ void __launch_bounds__(256) mc_conv_project16_kernel(
+// One wavefront per (centre, chunk of 16*kCPL channels): projection of the centre's
+// pairs with the basis evaluated in registers, rows written to out_rows[centre]
+// (or centre).
+template <int kCPL, int D, class Basis>
+__device__ __forceinline__ void project_centre_body(
     int64_t n_out, int C, int chunks, const float *__restrict__ feat,
-    const int2 *__restrict__ nbrs, const int *__restrict__ ranges, McParams<D> p,
-    const int *__restrict__ out_rows, float *__restrict__ out) {
+    const int2 *__restrict__ nbrs, const int *__restrict__ ranges, const McParams<D> &p,
+    const Basis &basis, const int *__restrict__ out_rows, float *__restrict__ out,
+    PairStage *stage) {
   constexpr int K = kFusedK;
   constexpr int kCW = 16 * kCPL;
   const int lane = lane_id();
@@ -29,7 +33,6 @@ __global__ void __launch_bounds__(256) mc_conv_project16_kernel(
   const int chunk = (int)(wid - centre * chunks);
   const int quarter = lane >> 4, col = lane & 15;
   const int a = centre > 0 ? ranges[centre - 1] : 0, b = ranges[centre];
-  __shared__ PairStage stages[kWavesPerBlock];
   float ctr[D];
 #pragma unroll
   for (int d = 0; d < D; ++d) ctr[d] = p.pout[centre * D + d];
@@ -38,8 +41,8 @@ __global__ void __launch_bounds__(256) mc_conv_project16_kernel(
   for (int j = 0; j < kCPL; ++j)
 #pragma unroll
     for (int r = 0; r < 4; ++r) acc[j][r] = 0.0f;
-  project_pairs<kCPL, D, kAct>(reinterpret_cast<const char *>(feat + chunk * kCW), (unsigned)C * 4, nbrs,
-                         a, b, p, ctr, &stages[threadIdx.x / kWave], acc);
+  project_pairs<kCPL, D>(reinterpret_cast<const char *>(feat + chunk * kCW), (unsigned)C * 4, nbrs,
+                         a, b, p, ctr, stage, basis, acc);
   const int64_t row = out_rows ? (int64_t)__builtin_amdgcn_readfirstlane(out_rows[centre]) : centre;
   float *o = out + row * (int64_t)C * K + (int64_t)chunk * kCW * K + 4 * quarter;
 #pragma unroll
@@ -47,6 +50,30 @@ __global__ void __launch_bounds__(256) mc_conv_project16_kernel(
     *reinterpret_cast<v4f *>(o + (col * kCPL + j) * K) = acc[j];
 }
 
+template <int kCPL, int D, int kAct>
+__global__ void __launch_bounds__(256) mc_conv_project16_kernel(
+    int64_t n_out, int C, int chunks, const float *__restrict__ feat,
+    const int2 *__restrict__ nbrs, const int *__restrict__ ranges, McParams<D> p,
+    const int *__restrict__ out_rows, float *__restrict__ out) {
+  __shared__ PairStage stages[kWavesPerBlock];
+  const MlpBasis<D, kAct> basis(p);
+  project_centre_body<kCPL, D>(n_out, C, chunks, feat, nbrs, ranges, p, basis, out_rows, out,
+                               &stages[threadIdx.x / kWave]);
+}
+
+// The same projection with the kernel-point correlation of KPConv as basis
+// (KPConv.py:193-224: weights of up to 16 kernel points, zero padding beyond).
+template <int kCPL, int D, int kKind>
+__global__ void __launch_bounds__(256) kp_conv_project16_kernel(
+    int64_t n_out, int C, int chunks, const float *__restrict__ feat,
+    const int2 *__restrict__ nbrs, const int *__restrict__ ranges, McParams<D> p,
+    const float *__restrict__ kernel_points, int num_kp, float sigma,
+    const int *__restrict__ out_rows, float *__restrict__ out) {
+  __shared__ PairStage stages[kWavesPerBlock];
+  const KpBasis<D, kKind> basis(kernel_points, num_kp, sigma);
+  project_centre_body<kCPL, D>(n_out, C, chunks, feat, nbrs, ranges, p, basis, out_rows, out,
+                               &stages[threadIdx.x / kWave]);
+}
 
 // Persistent wavefronts stride over the centres.  Per tile of 16 pairs:
 //   dbasis^T [k x pair] by MFMA (reduction over channels), turned in registers
@@ -521,5 +548,61 @@ extern "C" int mccnn_mc_conv_project_grads(
   if (gathered && num_samples > 0 && num_neighbors > 0)
     return launch_dfeat_gather(s, num_pts, num_features, point_ranges, pair_order, pair_rows,
                                feature_grads_out);
+  return MCCNN_OK;
+}
+
+extern "C" int mccnn_kp_conv_project(mccnn_stream_t stream, int num_dims, int64_t num_pts,
+                                     const float *points_in, int num_features,
+                                     const float *features, int64_t num_samples,
+                                     const float *points_out, int64_t num_neighbors,
+                                     const int32_t *neighbors, const int32_t *ranges,
+                                     const float *inv_radii, int num_kernel_points,
+                                     const float *kernel_points, int kind, float sigma,
+                                     const int32_t *out_rows, float *out) {
+  MCCNN_REQUIRE(fused_supported(num_dims, num_features, kFusedK),
+                "kp_conv_project supports D in {2,3} and C in {16,32,64,128} (got D=%d, C=%d); "
+                "use kp_basis + basis_proj for other shapes", num_dims, num_features);
+  MCCNN_REQUIRE(num_kernel_points > 0 && num_kernel_points <= kFusedK,
+                "kp_conv_project supports 1 to 16 kernel points (got %d)", num_kernel_points);
+  MCCNN_REQUIRE(kind == 0 || kind == 1, "kp_conv_project expects kind 0 (linear) or 1 (gaussian)");
+  MCCNN_REQUIRE(sigma > 0.0f, "kp_conv_project expects a positive sigma");
+  MCCNN_REQUIRE(num_neighbors >= 0 && num_neighbors < ((int64_t)1 << 31) && num_samples >= 0 &&
+                    num_samples < ((int64_t)1 << 31),
+                "kp_conv_project expects sizes in [0, 2^31)");
+  MCCNN_REQUIRE(num_pts >= 0 && num_pts * num_features < ((int64_t)1 << 30),
+                "kp_conv_project expects a feature table of fewer than 2^30 elements");
+  if (num_samples == 0) return MCCNN_OK;
+  MCCNN_REQUIRE(ranges && out && points_out && inv_radii && kernel_points &&
+                    (num_neighbors == 0 || (points_in && features && neighbors)),
+                "kp_conv_project received a null tensor");
+  hipStream_t s = as_stream(stream);
+  int cpl = 1;
+  for (int c = 8; c >= 1; c >>= 1)
+    if (num_features % (16 * c) == 0) { cpl = c; break; }
+  const int chunks = num_features / (16 * cpl);
+  const dim3 grid(wave_grid(num_samples * chunks)), block(256);
+  const int2 *nb = (const int2 *)neighbors;
+#define MCCNN_KP_FWD(CPL_, D_, KIND_)                                                          \
+  {                                                                                            \
+    McParams<D_> prm{points_in, points_out, inv_radii, nullptr, nullptr, nullptr, 1, 0};       \
+    hipLaunchKernelGGL((kp_conv_project16_kernel<CPL_, D_, KIND_>), grid, block, 0, s,         \
+                       num_samples, num_features, chunks, features, nb, ranges, prm,           \
+                       kernel_points, num_kernel_points, sigma, out_rows, out);                \
+  }
+#define MCCNN_KP_FWD_D(CPL_)                                             \
+  if (num_dims == 3) {                                                   \
+    if (kind == 0) MCCNN_KP_FWD(CPL_, 3, 0) else MCCNN_KP_FWD(CPL_, 3, 1) \
+  } else {                                                               \
+    if (kind == 0) MCCNN_KP_FWD(CPL_, 2, 0) else MCCNN_KP_FWD(CPL_, 2, 1) \
+  }
+  switch (cpl) {
+    case 8: MCCNN_KP_FWD_D(8); break;
+    case 4: MCCNN_KP_FWD_D(4); break;
+    case 2: MCCNN_KP_FWD_D(2); break;
+    default: MCCNN_KP_FWD_D(1); break;
+  }
+#undef MCCNN_KP_FWD_D
+#undef MCCNN_KP_FWD
+  MCCNN_LAUNCH_CHECK();
   return MCCNN_OK;
 }

@@ -80,8 +80,9 @@ __global__ void __launch_bounds__(1024) mc_conv_layer16_kernel(
     float ctr[D];
 #pragma unroll
     for (int d = 0; d < D; ++d) ctr[d] = p.pout[centre * D + d];
-    project_pairs<kCPL, D, kAct>(reinterpret_cast<const char *>(feat), (unsigned)C * 4, nbrs, a, b, p,
-                           ctr, reinterpret_cast<PairStage *>(tile) + wave, acc);
+    const MlpBasis<D, kAct> basis(p);
+    project_pairs<kCPL, D>(reinterpret_cast<const char *>(feat), (unsigned)C * 4, nbrs, a, b, p,
+                           ctr, reinterpret_cast<PairStage *>(tile) + wave, basis, acc);
     if (proj_out) {
       float *o = proj_out + centre * (int64_t)C * K + 4 * quarter;
 #pragma unroll

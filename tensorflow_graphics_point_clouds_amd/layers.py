@@ -514,6 +514,28 @@ def _kp_basis_raw(points_in, points_out, neighbors, inv_radii, kernel_points, k,
     return basis
 
 
+def _kp_project(features, points_in, points_out, neighbors, ranges, inv_radii, kernel_points, k,
+                kind, sigma, out_rows=None):
+    """Kernel-point weights + projection -> [N_out, C, k]: one kernel (weights in
+    registers) when the shape is covered, else kp_basis followed by basis_proj."""
+    kp, dims = kernel_points.shape
+    c = features.shape[1]
+    if k == 16 and _lib.lib().mccnn_mc_conv_supported(cint(dims), cint(c), cint(16)):
+        out = torch.empty((ranges.shape[0], c, k), dtype=_F32, device=features.device)
+        _lib.call("kp_conv_project", stream(), cint(dims), i64(features.shape[0]),
+                  ptr(points_in, _F32), cint(c), ptr(features, _F32), i64(ranges.shape[0]),
+                  ptr(points_out, _F32), i64(neighbors.shape[0]), ptr(neighbors, _I32),
+                  ptr(ranges, _I32), ptr(inv_radii, _F32), cint(kp), ptr(kernel_points, _F32),
+                  cint(kind), cfloat(sigma), ptr(out_rows), ptr(out))
+        return out
+    basis = _kp_basis_raw(points_in, points_out, neighbors, inv_radii, kernel_points, k, kind,
+                          sigma)
+    out = tfg_custom_ops._basis_proj_raw(basis, features, neighbors, ranges)
+    if out_rows is not None:
+        out = torch.empty_like(out).index_copy_(0, out_rows.long(), out)
+    return out
+
+
 class _KPConvRigidLayer(torch.autograd.Function):
     """Rigid kernel-point convolution (KPConv.py:165-232) on the neighbourhood's
     grid-ordered view.  As for the Monte-Carlo convolution, the feature gradient is
@@ -528,22 +550,18 @@ class _KPConvRigidLayer(torch.autograd.Function):
         view = neighborhood.sorted_view()
         with _lib.region("permute_rows"):
             feats = features.index_select(0, view.point_order)
-        basis = _kp_basis_raw(view.points_in, view.points_out, view.table, inv_radii,
-                              kernel_points, k, kind, sigma)
-        proj = tfg_custom_ops._basis_proj_raw(basis, feats, view.table, view.ranges)
-        del basis
+        # rows of the projection go straight to the centres' original positions
+        proj = _kp_project(feats, view.points_in, view.points_out, view.table, view.ranges,
+                           inv_radii, kernel_points, k, kind, sigma, view.centre_rows)
         with _lib.region("gemm_out"):
             out = proj.reshape(proj.shape[0], -1) @ dense_weights
-        if view.centre_order is not None:
-            with _lib.region("permute_rows"):
-                out = torch.empty_like(out).index_copy_(0, view.centre_order, out)
-        ctx.save_for_backward(dense_weights, feats, inv_radii, kernel_points)
+        ctx.save_for_backward(dense_weights, feats, features, inv_radii, kernel_points)
         ctx.neighborhood, ctx.k, ctx.kind, ctx.sigma = neighborhood, k, kind, sigma
         return out
 
     @staticmethod
     def backward(ctx, dout):
-        dense, feats, inv_radii, kernel_points = ctx.saved_tensors
+        dense, feats, features, inv_radii, kernel_points = ctx.saved_tensors
         view = ctx.neighborhood.sorted_view()
         k, c, f = ctx.k, feats.shape[1], dense.shape[1]
         if view.centre_order is not None:
@@ -551,20 +569,17 @@ class _KPConvRigidLayer(torch.autograd.Function):
                 dout = dout.index_select(0, view.centre_order)
         else:
             dout = dout.contiguous()
-        basis_t = _kp_basis_raw(view.points_out, view.points_in, view.table_t, -inv_radii,
-                                kernel_points, k, ctx.kind, ctx.sigma)
-        q = tfg_custom_ops._basis_proj_raw(basis_t, dout, view.table_t, view.ranges_t)
-        del basis_t
+        # rows of Q (and so of dfeat) go straight to the points' original positions
+        q = _kp_project(dout, view.points_out, view.points_in, view.table_t, view.ranges_t,
+                        -inv_radii, kernel_points, k, ctx.kind, ctx.sigma, view.point_rows)
         q = q.reshape(feats.shape[0], f * k)
         dfeat = ddense = None
         if ctx.needs_input_grad[1]:
             w2 = dense.reshape(c, k, f).permute(2, 1, 0).reshape(f * k, c)
             with _lib.region("gemm_dfeat"):
                 dfeat = q @ w2
-            with _lib.region("permute_rows"):
-                dfeat = torch.empty_like(dfeat).index_copy_(0, view.point_order, dfeat)
         if ctx.needs_input_grad[0]:
-            ddense = _weight_grad_product(feats, q).reshape(c, f, k).permute(0, 2, 1)
+            ddense = _weight_grad_product(features, q).reshape(c, f, k).permute(0, 2, 1)
             ddense = ddense.reshape(c * k, f)
         return ddense, dfeat, None, None, None, None, None, None
 

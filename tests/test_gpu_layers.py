@@ -146,12 +146,13 @@ def test_pointconv_forward_backward(oracle, hidden, act):
     normwise(conv.pdf_biases_2.grad.cpu().numpy(), t["pb2"].grad.numpy(), tol=5e-5)
 
 
-@pytest.mark.parametrize("transposed", [True, False])
+@pytest.mark.parametrize("c_in,c_out,transposed", [(16, 24, True), (16, 24, False),
+                                                   (64, 32, True), (8, 16, True)])
 @pytest.mark.parametrize("kind,influence", [("linear", None), ("gaussian", 0.3 * 0.15)])
-def test_kpconv_forward_backward(oracle, kind, influence, transposed):
+def test_kpconv_forward_backward(oracle, kind, influence, c_in, c_out, transposed):
     from tensorflow_graphics_point_clouds_amd import layers, pc, synthetic
     rng = np.random.default_rng(5)
-    batch, radius, c_in, c_out = 2, 0.15, 16, 24
+    batch, radius = 2, 0.15
     pts, bids, ctr, cb, nbh = _setup(oracle, rng, batch=batch, radius=radius)
     feat = rng.standard_normal((len(pts), c_in)).astype(np.float32)
     kp = synthetic.spherical_kernel_points_15() * 0.8      # * 0.75 inside the layer = 0.6
