@@ -319,7 +319,14 @@ class MCConv(torch.nn.Module):
         self.fuse_final = fuse_final
 
     def forward(self, features, point_cloud_in, point_cloud_out, radius, neighborhood=None,
-                bandwidth=0.2):
+                bandwidth=0.2, return_sorted=False, return_padded=False):
+        features = point_cloud_in.flatten_features(features)
+        out = self._convolve(features, point_cloud_in, point_cloud_out, radius, neighborhood,
+                             bandwidth)
+        return point_cloud_out.format_output(out, return_sorted, return_padded)
+
+    def _convolve(self, features, point_cloud_in, point_cloud_out, radius, neighborhood,
+                  bandwidth):
         d = self._num_dims
         dev = features.device
         radii = pc._as_vector(radius, d, dev)
@@ -400,7 +407,14 @@ class PointConv(torch.nn.Module):
         self.last_neighborhood = None
 
     def forward(self, features, point_cloud_in, point_cloud_out, radius, neighborhood=None,
-                bandwidth=0.2):
+                bandwidth=0.2, return_sorted=False, return_padded=False):
+        features = point_cloud_in.flatten_features(features)
+        out = self._convolve(features, point_cloud_in, point_cloud_out, radius, neighborhood,
+                             bandwidth)
+        return point_cloud_out.format_output(out, return_sorted, return_padded)
+
+    def _convolve(self, features, point_cloud_in, point_cloud_out, radius, neighborhood,
+                  bandwidth):
         d, dev = self._num_dims, features.device
         radii = pc._as_vector(radius, d, dev)
         if neighborhood is None:
@@ -631,7 +645,14 @@ class KPConv(torch.nn.Module):
         return torch.nn.functional.pad(w.reshape(c, kp, -1), (0, 0, 0, k - kp)).reshape(c * k, -1)
 
     def forward(self, features, point_cloud_in, point_cloud_out, conv_radius, neighborhood=None,
-                kernel_influence_dist=None):
+                kernel_influence_dist=None, return_sorted=False, return_padded=False):
+        features = point_cloud_in.flatten_features(features)
+        out = self._convolve(features, point_cloud_in, point_cloud_out, conv_radius,
+                             neighborhood, kernel_influence_dist)
+        return point_cloud_out.format_output(out, return_sorted, return_padded)
+
+    def _convolve(self, features, point_cloud_in, point_cloud_out, conv_radius, neighborhood,
+                  kernel_influence_dist):
         d, dev = self._num_dims, features.device
         sigma = 1.0 if kernel_influence_dist is None else float(kernel_influence_dist) / float(
             conv_radius)
@@ -701,13 +722,17 @@ class _LocalPointPooling:
     kind = 0
 
     def __call__(self, features, point_cloud_in, point_cloud_out, pooling_radius,
-                 neighborhood=None):
+                 neighborhood=None, return_sorted=False, return_padded=False):
+        features = point_cloud_in.flatten_features(features)
         if neighborhood is None:
             radii = pc._as_vector(pooling_radius, point_cloud_in._dimension, features.device)
             grid = pc.Grid(point_cloud_in, radii)
             neighborhood = pc.Neighborhood(grid, radii, point_cloud_out)
-        return _LocalPool.apply(features.contiguous(), neighborhood._original_neigh_ids,
-                                neighborhood._samples_neigh_ranges, self.kind)
+        if point_cloud_out is None:          # centres of a self-neighbourhood: the sorted points
+            point_cloud_out = neighborhood._point_cloud_sampled
+        out = _LocalPool.apply(features.contiguous(), neighborhood._original_neigh_ids,
+                               neighborhood._samples_neigh_ranges, self.kind)
+        return point_cloud_out.format_output(out, return_sorted, return_padded)
 
 
 class MaxPooling(_LocalPointPooling):
@@ -745,14 +770,22 @@ class _GlobalPool(torch.autograd.Function):
 class GlobalMaxPooling:
     """pylib/pc/layers/Pooling.py:25-61."""
 
-    def __call__(self, features, point_cloud):
-        return _GlobalPool.apply(features.contiguous(), point_cloud._batch_ids,
-                                 point_cloud._batch_size, 0)
+    def __call__(self, features, point_cloud, return_padded=False):
+        features = point_cloud.flatten_features(features)
+        out = _GlobalPool.apply(features.contiguous(), point_cloud._batch_ids,
+                                point_cloud._batch_size, 0)
+        if return_padded and point_cloud._batch_shape is not None:   # Pooling.py:58-61
+            out = out.reshape(tuple(point_cloud._batch_shape) + (-1,))
+        return out
 
 
 class GlobalAveragePooling:
     """pylib/pc/layers/Pooling.py:64-104."""
 
-    def __call__(self, features, point_cloud):
-        return _GlobalPool.apply(features.contiguous(), point_cloud._batch_ids,
-                                 point_cloud._batch_size, 1)
+    def __call__(self, features, point_cloud, return_padded=False):
+        features = point_cloud.flatten_features(features)
+        out = _GlobalPool.apply(features.contiguous(), point_cloud._batch_ids,
+                                point_cloud._batch_size, 1)
+        if return_padded and point_cloud._batch_shape is not None:   # Pooling.py:101-104
+            out = out.reshape(tuple(point_cloud._batch_shape) + (-1,))
+        return out

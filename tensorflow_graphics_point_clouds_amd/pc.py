@@ -1,11 +1,12 @@
 """Thin counterparts of the reference's callers of the op path, on torch GPU
-tensors: `PointCloud` (segmented form only), `Grid`, `Neighborhood`, `sample`
+tensors: `PointCloud` (segmented and padded forms), `Grid`, `Neighborhood`, `sample`
 and `PointHierarchy` (pylib/pc/PointCloud.py, Grid.py, Neighborhood.py,
 sampling.py, PointHierarchy.py).  They only arrange arguments: bounding boxes,
 grid shape, sort and gathers are kernels of libmccnn_hip.so as well.
 """
 import ctypes
 import enum
+import math
 
 import torch
 
@@ -31,19 +32,139 @@ def _as_vector(value, dims, device):
 
 
 class PointCloud:
-    """Points [N, D] with a batch id per point (pylib/pc/PointCloud.py:68-134,
-    segmented input)."""
+    """Points with a cloud id per point (pylib/pc/PointCloud.py:68-290).
 
-    def __init__(self, points, batch_ids, batch_size=None):
-        self._points = torch.as_tensor(points, dtype=_F32).contiguous()
-        self._batch_ids = torch.as_tensor(batch_ids, dtype=_I32,
-                                          device=self._points.device).contiguous()
-        if self._points.dim() != 2 or self._batch_ids.shape[0] != self._points.shape[0]:
-            raise ValueError("expected points [N, D] and batch_ids [N]")
-        if batch_size is None:
-            batch_size = int(self._batch_ids.max().item()) + 1
+    points     [N, D] with `batch_ids` [N] or `sizes` (sum = N), or padded
+               [A1, ..., An, V, D] with optional `sizes` [A1, ..., An] (the first
+               sizes[a] rows of each cloud are real, the rest padding)
+    batch_size number of clouds (default: from batch_ids / sizes / batch shape)
+
+    Internally always the segmented form `_points` [N, D], `_batch_ids` [N]."""
+
+    def __init__(self, points, batch_ids=None, batch_size=None, sizes=None):
+        points = torch.as_tensor(points, dtype=_F32)
+        dev = points.device
+        self._sizes = None if sizes is None else torch.as_tensor(sizes, dtype=_I32, device=dev)
+        self._batch_shape = None
+        if points.dim() < 2:
+            raise ValueError("expected points [N, D] or [A1, ..., An, V, D]")
+        if points.dim() > 2:                                  # PointCloud.py:122-138
+            self._batch_shape = tuple(points.shape[:-2])
+            clouds, v = int(math.prod(self._batch_shape)), points.shape[-2]
+            if self._sizes is None:
+                self._sizes = torch.full(self._batch_shape, v, dtype=_I32, device=dev)
+            if tuple(self._sizes.shape) != self._batch_shape:
+                raise ValueError("sizes must have the batch shape %s" % (self._batch_shape,))
+            flat_sizes = self._sizes.reshape(-1).long()
+            if bool((flat_sizes > v).any()) or bool((flat_sizes < 0).any()):
+                raise ValueError("sizes must lie in [0, V]")
+            if batch_size is None:
+                batch_size = clouds
+            keep = (torch.arange(v, device=dev)[None, :] < flat_sizes[:, None]).reshape(-1)
+            self._points = points.reshape(clouds * v, -1)[keep].contiguous()
+            self._batch_ids = torch.repeat_interleave(
+                torch.arange(clouds, dtype=_I32, device=dev), flat_sizes)
+        else:                                                 # PointCloud.py:140-149
+            self._points = points.contiguous()
+            if batch_ids is None:
+                if self._sizes is None:
+                    raise ValueError("points [N, D] need batch_ids or sizes")
+                flat_sizes = self._sizes.reshape(-1).long()
+                if batch_size is None:
+                    batch_size = flat_sizes.numel()
+                batch_ids = torch.repeat_interleave(
+                    torch.arange(flat_sizes.numel(), dtype=_I32, device=dev), flat_sizes)
+            self._batch_ids = torch.as_tensor(batch_ids, dtype=_I32, device=dev).contiguous()
+            if self._batch_ids.shape[0] != self._points.shape[0]:
+                raise ValueError("expected one batch id (or sizes summing to one) per point")
+            if batch_size is None:
+                batch_size = int(self._batch_ids.max().item()) + 1 if self._points.shape[0] else 0
         self._batch_size = int(batch_size)
         self._dimension = self._points.shape[1]
+
+    def get_sizes(self):
+        """Points per cloud, in the batch shape if one is set (PointCloud.py:184-204)."""
+        if self._sizes is None:
+            self._sizes = torch.bincount(self._batch_ids.long(),
+                                         minlength=self._batch_size).to(_I32)
+            if self._batch_shape is not None:
+                self._sizes = self._sizes.reshape(self._batch_shape)
+        return self._sizes
+
+    def set_batch_shape(self, batch_shape):
+        """PointCloud.py:262-290."""
+        if batch_shape is None:
+            self._batch_shape = None
+            return
+        batch_shape = tuple(int(b) for b in batch_shape)
+        if int(math.prod(batch_shape)) != self._batch_size:
+            raise ValueError("Incompatible batch size. Must be %d but is %d" %
+                             (self._batch_size, int(math.prod(batch_shape))))
+        self._batch_shape = batch_shape
+        if self._sizes is not None:
+            self._sizes = self._sizes.reshape(batch_shape)
+
+    def get_unflatten(self, max_num_points=None):
+        """data [N, ...] -> zero-padded [A1, ..., An, V, ...] (PointCloud.py:206-235):
+        the rows of each cloud in their stored order."""
+        sizes = self.get_sizes().reshape(-1).long()
+        v = int(sizes.max().item()) if sizes.numel() else 0
+        if max_num_points is not None:
+            if max_num_points < v:
+                raise ValueError("max_num_points must be at least the largest cloud")
+            v = int(max_num_points)
+        order = torch.argsort(self._batch_ids.long(), stable=True)
+        starts = torch.cumsum(sizes, 0) - sizes
+        sorted_ids = self._batch_ids.long()[order]
+        slot = sorted_ids * v + (torch.arange(order.numel(), device=order.device) -
+                                 starts[sorted_ids])
+        shape = self._batch_shape if self._batch_shape is not None else (self._batch_size,)
+
+        def unflatten(data):
+            out = torch.zeros((self._batch_size * v,) + tuple(data.shape[1:]), dtype=data.dtype,
+                              device=data.device)
+            out[slot] = data[order]
+            return out.reshape(tuple(shape) + (v,) + tuple(data.shape[1:]))
+
+        return unflatten
+
+    def flatten_features(self, features):
+        """Features [N, C] (returned unchanged) or padded [A1, ..., An, V, C] ->
+        [N, C] in the order of the stored points (pylib/pc/utils.py:75-94)."""
+        features = torch.as_tensor(features, dtype=_F32, device=self._points.device)
+        if features.dim() == 2:
+            if features.shape[0] != self._points.shape[0]:
+                raise ValueError("expected one feature row per point")
+            return features
+        sizes = self.get_sizes().reshape(-1).long()
+        v, c = features.shape[-2], features.shape[-1]
+        keep = (torch.arange(v, device=features.device)[None, :] < sizes[:, None]).reshape(-1)
+        by_cloud = features.reshape(-1, c)[keep]          # rows grouped by cloud
+        order = torch.argsort(self._batch_ids.long(), stable=True)
+        out = torch.empty_like(by_cloud)
+        out[order] = by_cloud
+        return out
+
+    def format_output(self, features, return_sorted=False, return_padded=False):
+        """Layer output [N, C] as is, sorted by cloud id, or zero-padded to
+        [A1, ..., An, V, C] (pylib/pc/layers/utils.py:22-49)."""
+        if return_padded:
+            return self.get_unflatten()(features)
+        if return_sorted:
+            return features[torch.argsort(self._batch_ids.long(), stable=True)]
+        return features
+
+    def get_points(self, id=None, max_num_points=None):
+        """The points of cloud `id` (an int or an index into the batch shape), or all
+        of them padded to [A1, ..., An, V, D] (PointCloud.py:151-182)."""
+        if id is None:
+            return self.get_unflatten(max_num_points)(self._points)
+        if not isinstance(id, int):
+            shape = self._batch_shape if self._batch_shape is not None else (self._batch_size,)
+            id = int(torch.arange(self._batch_size).reshape(shape)[tuple(id)].item())
+        if id >= self._batch_size or id < -self._batch_size:
+            raise IndexError("batch index out of range")
+        return self._points[self._batch_ids == id % self._batch_size]
 
 
 def _sort_keys(keys, key_bits):

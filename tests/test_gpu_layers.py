@@ -325,3 +325,29 @@ def test_projection_grad_product_matches_float64(n, f, r):
     assert got.shape == (n, r)
     if n:
         assert np.abs(got - expect).max() <= 1e-5 * np.abs(expect).max()
+
+
+def test_layers_accept_padded_input_and_return_padded_output():
+    """Padded point clouds / features ([A, V, D], [A, V, C], sizes) give the same
+    result as the segmented form, re-padded on request (layers/utils.py:22-49,
+    pc/utils.py:75-94)."""
+    from tensorflow_graphics_point_clouds_amd import layers, pc
+    rng = np.random.default_rng(11)
+    sizes, v, c = [700, 400, 900], 900, 16
+    pts = rng.random((3, v, 3)).astype(np.float32)
+    feat = rng.standard_normal((3, v, c)).astype(np.float32)
+    padded = pc.PointCloud(dev(pts), sizes=sizes)
+    flat_pts = np.concatenate([pts[b, :n] for b, n in enumerate(sizes)])
+    flat_feat = np.concatenate([feat[b, :n] for b, n in enumerate(sizes)])
+    bids = np.repeat(np.arange(3), sizes).astype(np.int32)
+    flat = pc.PointCloud(dev(flat_pts), dev(bids), 3)
+    conv = layers.MCConv(c, 16, 3, num_mlps=1, mlp_size=[16], seed=4)
+    a = conv(dev(feat), padded, padded, 0.2, return_padded=True).detach()
+    b = conv(dev(flat_feat), flat, flat, 0.2)
+    assert a.shape == (3, v, 16)
+    for i, n in enumerate(sizes):
+        start = sum(sizes[:i])
+        assert torch.equal(a[i, :n], b[start:start + n])
+        assert float(a[i, n:].abs().sum()) == 0.0
+    pool = layers.MaxPooling()(dev(feat), padded, padded, 0.2, return_sorted=True)
+    assert torch.equal(pool, layers.MaxPooling()(dev(flat_feat), flat, flat, 0.2))
