@@ -212,6 +212,26 @@ class Grid:
         _lib.call("gather_points", stream(), i64(n), cint(d), ptr(pc._points), ptr(pc._batch_ids),
             ptr(self._sorted_indices), ptr(self._sorted_points), ptr(self._sorted_batch_ids))
         self._fast_DS = None
+        self._sorted_positions = None
+        self._self_neighborhoods = {}
+
+    def sorted_positions(self):
+        """Inverse of the sort: position of every original point in the sorted order."""
+        if self._sorted_positions is None:
+            n, dev = self._sorted_indices.shape[0], self._sorted_indices.device
+            inv = torch.empty(n, dtype=_I32, device=dev)
+            inv[self._sorted_indices.long()] = torch.arange(n, dtype=_I32, device=dev)
+            self._sorted_positions = inv
+        return self._sorted_positions
+
+    def self_neighborhood(self, radii, max_neighbors=0):
+        """The neighbourhood of the grid's sorted points among themselves for these
+        radii, built once and shared (densities, grid-ordered view, same-cloud
+        convolutions)."""
+        key = (tuple(float(r) for r in radii.tolist()), int(max_neighbors))
+        if key not in self._self_neighborhoods:
+            self._self_neighborhoods[key] = Neighborhood(self, radii, None, max_neighbors)
+        return self._self_neighborhoods[key]
 
     def get_DS(self):
         if self._fast_DS is None:
@@ -244,13 +264,15 @@ class _SortedView:
             self.centre_order = self.centre_rows = None
             self.points_out = grid._sorted_points
             self.table, self.ranges = nbh._neighbors, nbh._samples_neigh_ranges
+        elif nbh._self_neighborhood is not None:     # same cloud: the shared sorted search
+            own = nbh._self_neighborhood
+            self.centre_rows = grid._sorted_indices
+            self.centre_order = grid._sorted_indices.long()
+            self.points_out = grid._sorted_points
+            self.table, self.ranges = own._neighbors, own._samples_neigh_ranges
         else:
-            if samples is grid._point_cloud:
-                order = grid._sorted_indices
-                self.points_out = grid._sorted_points
-            else:
-                order = nbh.compute_centre_order()
-                self.points_out = samples._points[order.long()].contiguous()
+            order = nbh.compute_centre_order()
+            self.points_out = samples._points[order.long()].contiguous()
             self.centre_rows = order
             self.centre_order = order.long()
             L = _lib.lib()
@@ -263,10 +285,18 @@ class _SortedView:
                       ptr(nbh._samples_neigh_ranges, _I32), i64(nbh._neighbors.shape[0]),
                       ptr(nbh._neighbors, _I32), ptr(order, _I32), ptr(ws),
                       _lib.csize(ws.numel()), ptr(self.ranges), ptr(self.table))
-        self.ranges_t, pair_order = tfg_custom_ops.transpose_neighbors(
-            self.table, self.points_in.shape[0])
-        sel = pair_order.long()
-        self.table_t = torch.stack((self.table[sel, 1], self.table[sel, 0]), dim=1).contiguous()
+        if (nbh._equal_samples or nbh._self_neighborhood is not None) and nbh.max_neighbors == 0:
+            # An untruncated self-neighbourhood is symmetric (the distance test is exact
+            # under negation): the rows (x, p) of segment p are at once "x is a neighbour
+            # of centre p" and "p is a neighbour of centre x", so the table is its own
+            # transpose.
+            self.table_t, self.ranges_t = self.table, self.ranges
+        else:
+            self.ranges_t, pair_order = tfg_custom_ops.transpose_neighbors(
+                self.table, self.points_in.shape[0])
+            sel = pair_order.long()
+            self.table_t = torch.stack((self.table[sel, 1], self.table[sel, 0]),
+                                       dim=1).contiguous()
         self._pdf_key, self.pdf, self.pdf_t = None, None, None
 
     def pair_pdf(self, nbh):
@@ -304,10 +334,29 @@ class Neighborhood:
         self.max_neighbors = max_neighbors
         self._inv_radii = torch.reciprocal(self._radii)
         s = self._point_cloud_sampled
-        self._samples_neigh_ranges, self._neighbors = tfg_custom_ops.find_neighbors(
-            s._points, s._batch_ids, grid._sorted_points, grid._sorted_keys, grid.get_DS(),
-            grid._num_cells, grid._scaled_aabb_min, grid._inv_cell_sizes, self._inv_radii,
-            max_neighbors)
+        self._self_neighborhood = None
+        if point_cloud_sample is grid._point_cloud:
+            # The centres are the grid's own points in the caller's order: search once
+            # from the sorted points (consecutive centres then walk the same cells;
+            # the same search also serves the densities and the grid-ordered view of
+            # the layers) and regroup the segments.  The pairs of a centre depend on
+            # its coordinates only, so the table equals that of a direct search.
+            own = grid.self_neighborhood(self._radii, max_neighbors)
+            self._self_neighborhood = own
+            n = s._points.shape[0]
+            L = _lib.lib()
+            ws = _lib.workspace(L.mccnn_reorder_neighbors_workspace_bytes(i64(n)), dev)
+            self._samples_neigh_ranges = torch.empty_like(own._samples_neigh_ranges)
+            self._neighbors = torch.empty_like(own._neighbors)
+            _lib.call("reorder_neighbors", stream(), i64(n), ptr(own._samples_neigh_ranges, _I32),
+                      i64(own._neighbors.shape[0]), ptr(own._neighbors, _I32),
+                      ptr(grid.sorted_positions(), _I32), ptr(ws), _lib.csize(ws.numel()),
+                      ptr(self._samples_neigh_ranges), ptr(self._neighbors))
+        else:
+            self._samples_neigh_ranges, self._neighbors = tfg_custom_ops.find_neighbors(
+                s._points, s._batch_ids, grid._sorted_points, grid._sorted_keys, grid.get_DS(),
+                grid._num_cells, grid._scaled_aabb_min, grid._inv_cell_sizes, self._inv_radii,
+                max_neighbors)
         # pairs addressed by original point ids (Neighborhood.py:246-250)
         self._original_neigh_ids = torch.empty_like(self._neighbors)
         _lib.call("original_neighbor_ids", stream(), i64(self._neighbors.shape[0]), ptr(self._neighbors, _I32),
@@ -389,7 +438,7 @@ class Neighborhood:
         if mode == KDEMode.no_pdf:
             self._pdf = torch.ones(self._neighbors.shape[0], dtype=_F32, device=dev)
         else:
-            nbh = self if self._equal_samples else Neighborhood(self._grid, self._radii, None)
+            nbh = self if self._equal_samples else self._grid.self_neighborhood(self._radii)
             bw = _as_vector(bandwidth, d, dev)
             self._pdf_per_point = tfg_custom_ops.compute_pdf_with_pt_grads(
                 self._grid._sorted_points, nbh._neighbors, nbh._samples_neigh_ranges,
