@@ -65,6 +65,35 @@ def test_invalid_arguments_return_status_not_abort(lib):
     assert rc == 1 and b"batch size" in lib.mccnn_last_error()
 
 
+def test_layer_entry_points_reject_uncovered_shapes(lib):
+    i64, sz = ctypes.c_int64, ctypes.c_size_t
+    assert lib.mccnn_mc_conv_supported(3, 64, 16) == 1 and lib.mccnn_mc_conv_supported(3, 24, 16) == 0
+    assert lib.mccnn_mc_conv_layer_supported(3, 64, 16, 64) == 1
+    assert lib.mccnn_mc_conv_layer_supported(4, 64, 16, 64) == 0
+    assert lib.mccnn_weight_grad_product_supported(64, 1024) == 1
+    assert lib.mccnn_weight_grad_product_supported(48, 1024) == 0
+    assert lib.mccnn_projection_grad_product_supported(64, 1024) == 1
+    assert lib.mccnn_projection_grad_product_supported(128, 1024) == 0
+    # K = 8 is not covered by the fused projection
+    rc = lib.mccnn_mc_conv_project(None, 3, i64(10), None, 64, None, i64(10), None, i64(20), None,
+                                   None, None, 8, 1, 0, None, None, None, None, None)
+    assert rc == 1 and b"K = 16" in lib.mccnn_last_error()
+    rc = lib.mccnn_kp_conv_project(None, 3, i64(10), None, 64, None, i64(10), None, i64(20), None,
+                                   None, None, 17, None, 0, ctypes.c_float(1.0), None, None)
+    assert rc == 1 and b"kernel points" in lib.mccnn_last_error()
+    rc = lib.mccnn_weight_grad_product(None, i64(10), 48, None, 1024, None, None, sz(0), None)
+    assert rc == 1 and b"output rows" in lib.mccnn_last_error()
+    rc = lib.mccnn_projection_grad_product(None, i64(10), 128, None, 1024, None, None)
+    assert rc == 1 and b"input columns" in lib.mccnn_last_error()
+    # a feature table too large for 32-bit byte offsets is refused, not truncated
+    rc = lib.mccnn_mc_conv_project(None, 3, i64(1 << 25), None, 64, None, i64(10), None, i64(20),
+                                   None, None, None, 16, 1, 0, None, None, None, None, None)
+    assert rc == 1 and b"2^30" in lib.mccnn_last_error()
+    fn = lib.mccnn_mc_conv_project_grads_workspace_bytes
+    fn.restype = sz
+    assert fn(3, 16, i64(1000)) >= 32 * 64 * 4
+
+
 def test_workspace_queries(lib):
     for name in ("mccnn_sort_keys_workspace_bytes", "mccnn_sampling_workspace_bytes"):
         fn = getattr(lib, name)
