@@ -407,6 +407,9 @@ int mccnn_mc_basis_grads(mccnn_stream_t stream, int64_t num_neighbors,
  * counterpart among the reference's ops, which materialise the basis in
  * TensorFlow. */
 int mccnn_mc_conv_supported(int num_dims, int num_features, int num_basis);
+/* ... and for the forward alone (also mccnn_kp_conv_project): any multiple of 16
+ * channels up to 512. */
+int mccnn_mc_conv_project_supported(int num_dims, int num_features, int num_basis);
 int mccnn_mc_conv_project(mccnn_stream_t stream, int num_dims, int64_t num_pts,
                           const float *points_in, int num_features,
                           const float *features, int64_t num_samples,

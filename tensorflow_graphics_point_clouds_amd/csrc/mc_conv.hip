@@ -398,16 +398,25 @@ static int launch_fused_backward(hipStream_t s, int64_t num_samples, const float
   return MCCNN_OK;
 }
 
+// Shapes of the weight-gradient / feature-gradient kernels (C is a template parameter).
 static bool fused_supported(int D, int C, int K) {
   return (D == 2 || D == 3) && K == kFusedK && (C == 16 || C == 32 || C == 64 || C == 128);
 }
 
-static int check_fused_args(const char *op, int num_dims, int num_features, int num_basis,
-                            int num_mlps, int activation, int64_t num_neighbors,
+// Shapes of the projection kernels: any multiple of 16 channels, in chunks of up
+// to 128 channels per wavefront.
+static bool project_supported(int D, int C, int K) {
+  return (D == 2 || D == 3) && K == kFusedK && C >= 16 && C <= 512 && C % 16 == 0;
+}
+
+static int check_fused_args(const char *op, bool project_only, int num_dims, int num_features,
+                            int num_basis, int num_mlps, int activation, int64_t num_neighbors,
                             int64_t num_samples) {
-  MCCNN_REQUIRE(fused_supported(num_dims, num_features, num_basis),
-                "%s supports D in {2,3}, K = 16 and C in {16,32,64,128} (got D=%d, K=%d, C=%d); "
-                "use mc_basis + basis_proj for other shapes", op, num_dims, num_basis,
+  MCCNN_REQUIRE(project_only ? project_supported(num_dims, num_features, num_basis)
+                             : fused_supported(num_dims, num_features, num_basis),
+                "%s supports D in {2,3}, K = 16 and C in %s (got D=%d, K=%d, C=%d); "
+                "use mc_basis + basis_proj for other shapes", op,
+                project_only ? "{16, 32, ..., 512}" : "{16,32,64,128}", num_dims, num_basis,
                 num_features);
   MCCNN_REQUIRE(num_mlps > 0 && num_basis % num_mlps == 0,
                 "%s expects the number of basis functions to be divisible by the number of "
@@ -427,6 +436,10 @@ extern "C" int mccnn_mc_conv_supported(int num_dims, int num_features, int num_b
   return fused_supported(num_dims, num_features, num_basis) ? 1 : 0;
 }
 
+extern "C" int mccnn_mc_conv_project_supported(int num_dims, int num_features, int num_basis) {
+  return project_supported(num_dims, num_features, num_basis) ? 1 : 0;
+}
+
 extern "C" int mccnn_mc_conv_project(mccnn_stream_t stream, int num_dims, int64_t num_pts,
                                      const float *points_in, int num_features,
                                      const float *features, int64_t num_samples,
@@ -435,7 +448,7 @@ extern "C" int mccnn_mc_conv_project(mccnn_stream_t stream, int num_dims, int64_
                                      const float *inv_radii, int num_basis, int num_mlps,
                                      int activation, const float *weights, const float *biases,
                                      const float *pdf, const int32_t *out_rows, float *out) {
-  int rc = check_fused_args("mc_conv_project", num_dims, num_features, num_basis, num_mlps,
+  int rc = check_fused_args("mc_conv_project", true, num_dims, num_features, num_basis, num_mlps,
                             activation, num_neighbors, num_samples);
   if (rc != MCCNN_OK) return rc;
   MCCNN_REQUIRE(num_pts >= 0 && num_pts * num_features < ((int64_t)1 << 30),
@@ -494,7 +507,7 @@ extern "C" int mccnn_mc_conv_project_grads(
   MCCNN_REQUIRE(!gathered || (point_ranges && pair_order),
                 "mc_conv_project_grads needs the transposed pair lists with a pair-row "
                 "workspace");
-  int rc = check_fused_args("mc_conv_project_grads", num_dims, num_features, num_basis, num_mlps,
+  int rc = check_fused_args("mc_conv_project_grads", false, num_dims, num_features, num_basis, num_mlps,
                             activation, num_neighbors, num_samples);
   if (rc != MCCNN_OK) return rc;
   MCCNN_REQUIRE(num_pts >= 0 && num_pts * num_features < ((int64_t)1 << 30),
@@ -559,8 +572,8 @@ extern "C" int mccnn_kp_conv_project(mccnn_stream_t stream, int num_dims, int64_
                                      const float *inv_radii, int num_kernel_points,
                                      const float *kernel_points, int kind, float sigma,
                                      const int32_t *out_rows, float *out) {
-  MCCNN_REQUIRE(fused_supported(num_dims, num_features, kFusedK),
-                "kp_conv_project supports D in {2,3} and C in {16,32,64,128} (got D=%d, C=%d); "
+  MCCNN_REQUIRE(project_supported(num_dims, num_features, kFusedK),
+                "kp_conv_project supports D in {2,3} and C in {16, 32, ..., 512} (got D=%d, C=%d); "
                 "use kp_basis + basis_proj for other shapes", num_dims, num_features);
   MCCNN_REQUIRE(num_kernel_points > 0 && num_kernel_points <= kFusedK,
                 "kp_conv_project supports 1 to 16 kernel points (got %d)", num_kernel_points);

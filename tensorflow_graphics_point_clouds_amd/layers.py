@@ -325,6 +325,33 @@ class MCConv(torch.nn.Module):
                              bandwidth)
         return point_cloud_out.format_output(out, return_sorted, return_padded)
 
+    def _convolve_on_view(self, features, neighborhood, radii, biases, k):
+        """The fused path on the grid-ordered view; channel counts it does not cover
+        are zero-padded (features, rows / columns of the final weights) and the
+        result is cut back.  None if the shape is out of reach."""
+        d, c, f, l, h = (self._num_dims, self._num_features_in, self._num_features_out,
+                         self._num_mlps, self._hidden)
+        if k != 16 or d not in (2, 3):
+            return None
+        pad = _layer_padding(c, f, l)
+        if pad is None:
+            return None
+        c_pad, g_pad = pad
+        g = f // l
+        fuse_final = self.fuse_final and bool(_lib.lib().mccnn_mc_conv_layer_supported(
+            cint(d), cint(c_pad), cint(k), cint(g_pad * l)))
+        final = self.final_weights
+        if c_pad != c or g_pad != g:
+            final = torch.nn.functional.pad(final.reshape(l, c, h, g),
+                                            (0, g_pad - g, 0, 0, 0, c_pad - c))
+            final = final.reshape(l, c_pad * h, g_pad)
+            features = torch.nn.functional.pad(features, (0, c_pad - c))
+        out = _MCConvLayer.apply(self.weights, biases, final, features, neighborhood,
+                                 torch.reciprocal(radii), self._act, fuse_final)
+        if g_pad != g:
+            out = out.reshape(-1, l, g_pad)[:, :, :g].reshape(-1, f)
+        return out
+
     def _convolve(self, features, point_cloud_in, point_cloud_out, radius, neighborhood,
                   bandwidth):
         d = self._num_dims
@@ -339,11 +366,10 @@ class MCConv(torch.nn.Module):
         k = self._num_mlps * self._hidden
         fused = self.fused and _lib.lib().mccnn_mc_conv_supported(
             cint(d), cint(self._num_features_in), cint(k))
-        if fused and self.transposed_grads and _lib.lib().mccnn_mc_conv_layer_supported(
-                cint(d), cint(self._num_features_in), cint(k), cint(self._num_features_out)):
-            return _MCConvLayer.apply(self.weights, biases, self.final_weights, features,
-                                      neighborhood, torch.reciprocal(radii), self._act,
-                                      self.fuse_final)
+        if self.fused and self.transposed_grads:
+            out = self._convolve_on_view(features, neighborhood, radii, biases, k)
+            if out is not None:
+                return out
         transposed = None
         if self.gathered_grads and features.requires_grad and \
                 tfg_custom_ops.gathered_grads_supported(self._num_features_in, k):
@@ -367,6 +393,19 @@ class MCConv(torch.nn.Module):
             return proj.reshape(n, c * h) @ self.final_weights[0]
         p = proj.reshape(n, c, l, h).permute(2, 0, 1, 3).reshape(l, n, c * h)
         return torch.bmm(p, self.final_weights).permute(1, 0, 2).reshape(n, -1)
+
+
+def _layer_padding(c, f, num_mlps):
+    """Channel counts the grid-ordered layer path runs on, or None: C rounded up to
+    16/32/64/128, and per kernel MLP as many output columns G' >= G as make the
+    total a multiple of 16 (at most 512)."""
+    c_pad = next((v for v in (16, 32, 64, 128) if v >= c), None)
+    step = 16 // math.gcd(16, num_mlps)
+    g = f // num_mlps
+    g_pad = -(-g // step) * step
+    if c_pad is None or g_pad * num_mlps > 512:
+        return None
+    return c_pad, g_pad
 
 
 class PointConv(torch.nn.Module):
@@ -534,7 +573,7 @@ def _kp_project(features, points_in, points_out, neighbors, ranges, inv_radii, k
     registers) when the shape is covered, else kp_basis followed by basis_proj."""
     kp, dims = kernel_points.shape
     c = features.shape[1]
-    if k == 16 and _lib.lib().mccnn_mc_conv_supported(cint(dims), cint(c), cint(16)):
+    if k == 16 and _lib.lib().mccnn_mc_conv_project_supported(cint(dims), cint(c), cint(16)):
         out = torch.empty((ranges.shape[0], c, k), dtype=_F32, device=features.device)
         _lib.call("kp_conv_project", stream(), cint(dims), i64(features.shape[0]),
                   ptr(points_in, _F32), cint(c), ptr(features, _F32), i64(ranges.shape[0]),
