@@ -94,16 +94,18 @@ __global__ void __launch_bounds__(256) mc_basis_grads_kernel(
   }
 }
 
-// weight_grads [L, D, H], bias_grads [L, H] from partials [blocks][(D+1)][K].
-__global__ void mc_basis_grads_reduce_kernel(int blocks, int D, int K, int H,
-                                             const float *__restrict__ partials,
-                                             float *__restrict__ dweights,
-                                             float *__restrict__ dbiases) {
-  const int t = blockIdx.x * blockDim.x + threadIdx.x;
-  if (t >= (D + 1) * K) return;
+// weight_grads [L, D, H], bias_grads [L, H] from partials [blocks][(D+1)][K]: one
+// wavefront per output, lanes stride over the blocks, fixed summation order.
+__global__ void __launch_bounds__(64) mc_basis_grads_reduce_kernel(
+    int blocks, int D, int K, int H, const float *__restrict__ partials,
+    float *__restrict__ dweights, float *__restrict__ dbiases) {
+  const int t = blockIdx.x;
   const int q = t / K, j = t - q * K;
   float s = 0.0f;
-  for (int b = 0; b < blocks; ++b) s += partials[((int64_t)b * (D + 1) + q) * K + j];
+  for (int b = threadIdx.x; b < blocks; b += kWave)
+    s += partials[((int64_t)b * (D + 1) + q) * K + j];
+  s = wave_sum(s);
+  if (threadIdx.x != 0) return;
   const int l = j / H, h = j - l * H;
   if (q < D) dweights[(l * D + q) * H + h] = s;
   else dbiases[j] = s;
@@ -387,7 +389,7 @@ extern "C" int mccnn_mc_basis_grads(mccnn_stream_t stream, int64_t num_neighbors
                                                 (float *)workspace));
   MCCNN_LAUNCH_CHECK();
   const int outs = (num_dims + 1) * num_basis;
-  hipLaunchKernelGGL(mc_basis_grads_reduce_kernel, dim3(blocks_for(outs, 64)), dim3(64), 0, s,
+  hipLaunchKernelGGL(mc_basis_grads_reduce_kernel, dim3(outs), dim3(kWave), 0, s,
                      blocks, num_dims, num_basis, num_basis / num_mlps,
                      (const float *)workspace, weight_grads_out, bias_grads_out);
   MCCNN_LAUNCH_CHECK();

@@ -366,8 +366,6 @@ class Neighborhood:
         # optional visiting order of the centres for the projection kernels
         self._centre_order = None
         self._transposed_pairs = None
-        self._transposed_table = None
-        self._transposed_pdf = None
         self._sorted_view = None
         self._transposed = None
 
@@ -378,26 +376,6 @@ class Neighborhood:
             self._transposed_pairs = tfg_custom_ops.transpose_neighbors(
                 self._original_neigh_ids, self._grid._point_cloud._points.shape[0])
         return self._transposed_pairs
-
-    def transposed_table(self, pdf=None):
-        """The pair table seen from the neighbour points: rows (centre, point) sorted
-        by point with inclusive end offsets per point, and `pdf` (per pair) in the same
-        order.  A convolution over this table carries values from the centres back
-        to the points (Neighborhood.py:313-329 builds the same view); the layers use
-        it for their feature gradients.  Built on first use and kept."""
-        point_ranges, pair_order = self.transposed_pairs()
-        if self._transposed_table is None:
-            order = pair_order.long()
-            ids = self._original_neigh_ids
-            self._transposed_table = torch.stack((ids[order, 1], ids[order, 0]),
-                                                 dim=1).contiguous()
-        pdf_t = None
-        if pdf is not None:
-            key = (pdf.data_ptr(), pdf._version)
-            if self._transposed_pdf is None or self._transposed_pdf[0] != key:
-                self._transposed_pdf = (key, pdf[pair_order.long()].contiguous())
-            pdf_t = self._transposed_pdf[1]
-        return self._transposed_table, point_ranges, pdf_t
 
     def get_grid(self):
         """The grid used for the neighbour search (Neighborhood.py:313-316)."""
