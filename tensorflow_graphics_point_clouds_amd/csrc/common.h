@@ -111,6 +111,17 @@ __device__ __forceinline__ void cell_of_point(const float *p, const float *smin,
 
 __device__ __forceinline__ int lane_id() { return threadIdx.x & (kWave - 1); }
 
+// Orders the LDS traffic of one wavefront: what any lane wrote before the call
+// is what every lane reads after it.  The hardware already serves the LDS
+// accesses of a wavefront in program order; the call keeps the compiler from
+// moving (or duplicating into divergent branches) loads and stores across it.
+// Every lane of the wavefront must reach it.
+__device__ __forceinline__ void wave_lds_sync() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
 // Inclusive prefix sum across the 64 lanes of a wave.
 __device__ __forceinline__ int wave_inclusive_scan(int v) {
   const int lane = lane_id();

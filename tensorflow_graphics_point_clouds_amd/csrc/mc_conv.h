@@ -123,6 +123,7 @@ __device__ __forceinline__ void project_pairs(const char *__restrict__ feat_base
     const unsigned row0 = __builtin_amdgcn_readfirstlane(row);
     stage->geo[lane] = g;
     stage->row[lane] = lane < cnt ? row : row0;
+    wave_lds_sync();
     const int steps = (cnt + 3) >> 2;
     for (int t = 0; t < steps; t += kFusedUnroll) {
       FVec<kCPL> f[kFusedUnroll];
@@ -143,6 +144,7 @@ __device__ __forceinline__ void project_pairs(const char *__restrict__ feat_base
             acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(w[u], f[u].v[j], acc[j], 0, 0, 0);
         }
     }
+    wave_lds_sync();                        // the stage is free for the next chunk
   }
 }
 

@@ -302,6 +302,7 @@ __global__ void __launch_bounds__(256) mc_conv_weight_grads16_kernel(
       const unsigned row0 = __builtin_amdgcn_readfirstlane(row);
       stage->geo[lane] = g;
       stage->row[lane] = lane < cnt ? row : row0;
+      wave_lds_sync();
       const int tiles = (cnt + 15) >> 4;
       FVec<kQuarterC> f = load_vec<kQuarterC>(
           reinterpret_cast<const float *>(feat_lane + stage->row[col]), true);
@@ -328,6 +329,7 @@ __global__ void __launch_bounds__(256) mc_conv_weight_grads16_kernel(
         }
         f = fn;
       }
+      wave_lds_sync();                      // the stage is free for the next chunk
     }
   }
   // reduce over the 16 pair-lanes of each quarter
