@@ -169,7 +169,8 @@ def kpconv_config5(torch, pc, layers, synthetic, _lib, steps=5):
     r = cfg["radius"]
     nbh = pc.Neighborhood(pc.Grid(cloud, r), r, cloud)
     N, M, C, CO = cloud._points.shape[0], nbh._neighbors.shape[0], cfg["c_in"], cfg["c_out"]
-    conv = layers.KPConv(C, CO, cfg["kernel_points"] / 0.75, kernel_weighting="linear", seed=5)
+    conv = layers.KPConv(C, CO, custom_kernel_points=cfg["kernel_points"] / 0.75,
+                         kp_interpolation="linear", seed=5)
     gen = torch.Generator(device="cuda").manual_seed(5)
     feats = torch.randn((N, C), device="cuda", generator=gen).requires_grad_(True)
     up = torch.randn((N, CO), device="cuda", generator=gen)

@@ -5,9 +5,11 @@ their gradients are kernels of libmccnn_hip.so; the dense
 [N, C*K] x [C*K, C_out] product is a plain library GEMM (torch.matmul)."""
 import math
 
+import numpy as np
 import torch
 
 from . import _lib, pc, tfg_custom_ops
+from .kernel_points import cube_kernel_points, spherical_kernel_points
 from ._lib import cfloat, cint, i64, ptr, stream
 
 _F32, _I32 = torch.float32, torch.int32
@@ -639,21 +641,29 @@ class _KPConvRigidLayer(torch.autograd.Function):
 
 class KPConv(torch.nn.Module):
     """Kernel-point convolution, rigid or deformable
-    (pylib/pc/layers/KPConv.py:60-429).  The kernel points are scaled by 0.75 as
-    in the reference (:131); `kernel_points` is [K, D] in units of the convolution
-    radius.  With `deformable=True` a rigid kernel-point convolution predicts a
-    per-centre offset for every kernel point (:317-392) and
-    `regularization_loss()` returns the fitting + repulsive loss (:394-429)."""
+    (pylib/pc/layers/KPConv.py:60-429).  The kernel points are one of the
+    spherical layouts, randomly rotated (seeded), or `custom_kernel_points`
+    [K, D] in units of the convolution radius (required when num_dims != 3,
+    :117-128); either is scaled by 0.75 as in the reference (:131).  With
+    `deformable=True` a rigid kernel-point convolution predicts a per-centre
+    offset for every kernel point (:317-392) and `regularization_loss()` returns
+    the fitting + repulsive loss (:394-429)."""
 
-    def __init__(self, num_features_in, num_features_out, kernel_points, num_dims=3,
-                 kernel_weighting="linear", weights=None, deformable=False,
-                 offset_weights=None, device="cuda", seed=0, transposed_grads=True):
+    def __init__(self, num_features_in, num_features_out, num_kernel_points=15, num_dims=3,
+                 deformable=False, kp_interpolation="linear", custom_kernel_points=None,
+                 weights=None, offset_weights=None, device="cuda", seed=0,
+                 transposed_grads=True):
         super().__init__()
-        kp = torch.as_tensor(kernel_points, dtype=_F32).to(device) * 0.75
+        if custom_kernel_points is None:
+            if num_dims != 3:
+                raise ValueError("For dimension not 3 custom kernel points must be provided!")
+            custom_kernel_points = spherical_kernel_points(
+                num_kernel_points, rotate=True, rng=np.random.default_rng(seed))
+        kp = torch.as_tensor(np.asarray(custom_kernel_points, dtype=np.float32)).to(device) * 0.75
         self._kernel_points = kp.contiguous()
         self._num_kernel_points = kp.shape[0]
         self._num_basis = _padded_basis_count(kp.shape[0])
-        self._kind = {"linear": 0, "gaussian": 1}[kernel_weighting]
+        self._kind = {"linear": 0, "gaussian": 1}[kp_interpolation]
         self._num_features_in, self._num_features_out = num_features_in, num_features_out
         self._num_dims = num_dims
         gen = torch.Generator().manual_seed(seed)

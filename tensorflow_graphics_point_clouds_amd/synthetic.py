@@ -6,6 +6,8 @@ shrinks the point counts so the same shapes can be used in CPU-sized tests.
 """
 import numpy as np
 
+from .kernel_points import spherical_kernel_points
+
 
 def _batch_ids(sizes):
     return np.repeat(np.arange(len(sizes), dtype=np.int32), sizes)
@@ -56,8 +58,9 @@ def _random_rotation(rng):
     return q
 
 
-def _primitive(rng, n):
-    kind = rng.integers(0, 4)
+def _primitive(rng, n, kind=None):
+    if kind is None:
+        kind = rng.integers(0, 4)
     if kind == 0:      # sphere
         v = rng.standard_normal((n, 3))
         p = v / np.linalg.norm(v, axis=1, keepdims=True)
@@ -105,6 +108,16 @@ def config2(seed=1002, batch=16, points_per_cloud=1024):
                 radii=(0.1, 0.2, 0.4), channels=(3, 64, 128, 256))
 
 
+def labelled_primitives(count, points_per_cloud=1024, seed=0):
+    """A four-class stand-in for a shape-classification set: `count` clouds of
+    points on spheres, boxes, tori and cylinders (class 0..3) of random size and
+    orientation inside the unit sphere -> (points [count, P, 3], labels [count])."""
+    rng = np.random.default_rng(seed)
+    labels = rng.integers(0, 4, count)
+    pts = np.stack([_primitive(rng, points_per_cloud, int(k)) for k in labels])
+    return pts.astype(np.float32), labels.astype(np.int64)
+
+
 def config3(seed=1003, scale=1.0, batch=8):
     """Scene-scale clustered clouds of uneven size; radius 0.15.
 
@@ -139,28 +152,8 @@ def config4(seed=1004, scale=1.0, batch=4):
                 c_in=128, basis=32)
 
 
-def spherical_kernel_points_15():
-    """The 15-point kernel layout of the reference, unrotated: centre, two poles
-    and two six-point rings at height sqrt(3)/2, the second ring mirrored and
-    with x and y exchanged (pylib/pc/layers/utils.py:79-100, 204-209; the ring
-    lists one of its points twice, which is kept because it is the data the
-    reference convolves with)."""
-    phi = np.sqrt(3.0) / 2.0
-    ring = np.array([[0, 1, 0], [0, -1, 0], [0.5, phi, 0], [0.5, -phi, 0],
-                     [-0.5, phi, 0], [0.5, -phi, 0]], dtype=np.float64)
-
-    def hexagon(scale, z_shift):
-        pts = ring * scale
-        pts[:, 2] += z_shift
-        return pts
-
-    pts = np.concatenate([[[0, 0, 0], [0, 0, 1], [0, 0, -1]], hexagon(0.5, phi),
-                          hexagon(-0.5, phi)[:, [1, 0, 2]]], axis=0)
-    return pts.astype(np.float32)
-
-
 def config5(seed=1005, scale=1.0, batch=8):
     """KPConv on the scene-scale geometry: 15 kernel points at 0.6 r, 128 -> 128."""
     cfg = config3(seed=seed, scale=scale, batch=batch)
-    cfg.update(c_in=128, c_out=128, kernel_points=spherical_kernel_points_15() * 0.6)
+    cfg.update(c_in=128, c_out=128, kernel_points=spherical_kernel_points(15, rotate=False) * 0.6)
     return cfg

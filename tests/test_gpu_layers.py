@@ -156,7 +156,7 @@ def test_kpconv_forward_backward(oracle, kind, influence, c_in, c_out, transpose
     batch, radius = 2, 0.15
     pts, bids, ctr, cb, nbh = _setup(oracle, rng, batch=batch, radius=radius)
     feat = rng.standard_normal((len(pts), c_in)).astype(np.float32)
-    kp = synthetic.spherical_kernel_points_15() * 0.8      # * 0.75 inside the layer = 0.6
+    kp = synthetic.spherical_kernel_points(15, rotate=False) * 0.8      # * 0.75 inside the layer = 0.6
     wts = (rng.standard_normal((15 * c_in, c_out)) * 0.1).astype(np.float32)
     sigma = 1.0 if influence is None else influence / radius
     ids = nbh.original_neigh_ids
@@ -168,7 +168,8 @@ def test_kpconv_forward_backward(oracle, kind, influence, c_in, c_out, transpose
     proj = oracle.basis_proj(padded, feat, ids, nbh.ranges)[:, :, :15]
     expect = proj.reshape(len(ctr), -1) @ wts.astype(np.float64)
 
-    conv = layers.KPConv(c_in, c_out, kp, kernel_weighting=kind, weights=dev(wts),
+    conv = layers.KPConv(c_in, c_out, custom_kernel_points=kp, kp_interpolation=kind,
+                         weights=dev(wts),
                          transposed_grads=transposed)
     tfeat = dev(feat).requires_grad_(True)
     out = conv(tfeat, pc.PointCloud(dev(pts), dev(bids), batch),
@@ -195,7 +196,7 @@ def test_deformable_kpconv_and_regularization(oracle, kind):
     batch, radius, c_in, c_out, kpn = 2, 0.2, 16, 8, 15
     pts, bids, ctr, cb, nbh = _setup(oracle, rng, n=1500, n_out=400, batch=batch, radius=radius)
     feat = rng.standard_normal((len(pts), c_in)).astype(np.float32)
-    kp = synthetic.spherical_kernel_points_15() * 0.8
+    kp = synthetic.spherical_kernel_points(15, rotate=False) * 0.8
     wts = (rng.standard_normal((kpn * c_in, c_out)) * 0.1).astype(np.float32)
     woff = (rng.standard_normal((kpn * c_in, kpn * 3)) * 0.002).astype(np.float32)
     influence = 0.5 * radius
@@ -230,7 +231,8 @@ def test_deformable_kpconv_and_regularization(oracle, kind):
     rep = weight(kd) * (1 - torch.eye(kpn, dtype=torch.float64))[None]
     ref_loss = fit.sum() + rep.sum()
 
-    conv = layers.KPConv(c_in, c_out, kp, kernel_weighting=kind, weights=dev(wts),
+    conv = layers.KPConv(c_in, c_out, custom_kernel_points=kp, kp_interpolation=kind,
+                         weights=dev(wts),
                          deformable=True, offset_weights=dev(woff))
     tfeat = dev(feat).requires_grad_(True)
     out = conv(tfeat, pc.PointCloud(dev(pts), dev(bids), batch),
