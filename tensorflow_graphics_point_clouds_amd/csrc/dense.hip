@@ -140,7 +140,8 @@ __global__ void __launch_bounds__(256) nt_product_kernel(int64_t n, int R,
       const int64_t pt = 16 * t + 4 * kk + r;
       if (pt < n) {
         const v4f v = {acc[0][r], acc[1][r], acc[2][r], acc[3][r]};
-        *reinterpret_cast<v4f *>(out + pt * R + col0 + 4 * c16) = v;
+        // streamed: the product is read once, by a later kernel
+        __builtin_nontemporal_store(v, reinterpret_cast<v4f *>(out + pt * R + col0 + 4 * c16));
       }
     }
     a = an;

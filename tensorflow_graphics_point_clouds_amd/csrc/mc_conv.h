@@ -124,13 +124,16 @@ __device__ __forceinline__ void project_pairs(const char *__restrict__ feat_base
     stage->geo[lane] = g;
     stage->row[lane] = lane < cnt ? row : row0;
     wave_lds_sync();
+    // Steps of 4 pairs, taken kFusedUnroll at a time without a branch: the slots
+    // past the last pair hold weight 0 and a valid row, so the steps that round the
+    // count up add exact zeros.
     const int steps = (cnt + 3) >> 2;
     for (int t = 0; t < steps; t += kFusedUnroll) {
       FVec<kCPL> f[kFusedUnroll];
       float w[kFusedUnroll];
 #pragma unroll
       for (int u = 0; u < kFusedUnroll; ++u) {
-        const int n = (4 * (t + u) + quarter) & (kWave - 1);
+        const int n = 4 * (t + u) + quarter;
         const float4 gn = stage->geo[n];
         const unsigned rn = stage->row[n];
         f[u] = load_vec<kCPL>(reinterpret_cast<const float *>(feat_base + rn + lane_off), true);
@@ -138,11 +141,9 @@ __device__ __forceinline__ void project_pairs(const char *__restrict__ feat_base
       }
 #pragma unroll
       for (int u = 0; u < kFusedUnroll; ++u)
-        if (t + u < steps) {
 #pragma unroll
-          for (int j = 0; j < kCPL; ++j)
-            acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(w[u], f[u].v[j], acc[j], 0, 0, 0);
-        }
+        for (int j = 0; j < kCPL; ++j)
+          acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(w[u], f[u].v[j], acc[j], 0, 0, 0);
     }
     wave_lds_sync();                        // the stage is free for the next chunk
   }

@@ -393,3 +393,47 @@ def test_three_level_mcconv_network_matches_oracle(oracle):
         feat_ref = np.maximum(expect, 0.0)
         feat = dev(feat_ref.astype(np.float32))
         cur_pts, cur_bids = nxt_pts, nxt_bids
+
+
+@pytest.mark.parametrize("d,c,n_out,radius", [(3, 64, 803, 0.3), (2, 32, 517, 0.12), (3, 128, 99, 0.35),
+                                              (3, 16, 5, 0.3)])
+def test_projection_runs_with_empty_and_crowded_centres(oracle, d, c, n_out, radius):
+    """The projection kernel walks runs of 8 consecutive centres in chunks of 64
+    pairs: centre counts that are no multiple of 8, neighbourhoods of several
+    chunks, empty centres (a whole empty run first, single ones in between, the
+    last centres), two channel chunks (C = 128) and D = 2, with and without row
+    indirection, against the oracle's basis and projection."""
+    from tensorflow_graphics_point_clouds_amd import layers
+    rng = np.random.default_rng(d * 100 + c)
+    n, batch = 3000, 2
+    pts = rng.random((n, d)).astype(np.float32)
+    bids = np.sort(rng.integers(0, batch, n)).astype(np.int32)
+    ctr = rng.random((n_out, d)).astype(np.float32)
+    cb = np.sort(rng.integers(0, batch, n_out)).astype(np.int32)
+    far = np.zeros(n_out, bool)
+    far[:min(9, n_out - 2)] = True
+    far[-2:] = True
+    far[rng.random(n_out) < 0.2] = True
+    far[n_out // 2] = False
+    ctr[far] += 5.0                                        # no neighbours out there
+    g = oracle.Grid(pts, bids, batch, np.float32(radius))
+    nbh = oracle.Neighborhood(g, np.float32(radius), ctr, cb)
+    counts = np.diff(np.concatenate([[0], nbh.ranges]))
+    assert counts[far].max() == 0 and (counts.max() > 64 or d == 2)
+    pdf = (0.5 + rng.random(len(nbh.neighbors))).astype(np.float32)
+    w = (rng.standard_normal((1, d, 16)) * 0.7).astype(np.float32)
+    b = (rng.standard_normal((1, 1, 16)) * 0.1).astype(np.float32)
+    feat = rng.standard_normal((n, c)).astype(np.float32)
+    ids = nbh.original_neigh_ids
+    diff = (pts[ids[:, 0]] - ctr[ids[:, 1]]) / np.float32(radius)
+    basis = oracle.mc_basis(diff, pdf, w, b, "leaky_relu")
+    expect = oracle.basis_proj(basis.astype(np.float32), feat, ids, nbh.ranges)
+    inv = dev(np.full(d, 1.0 / np.float32(radius), np.float32))
+    args = (dev(w), dev(b.reshape(-1)), dev(feat), dev(pts), dev(ctr), dev(ids), dev(nbh.ranges), inv,
+            dev(pdf), 1)
+    out = layers._mc_project(*args)
+    normwise(out.cpu().numpy(), expect)
+    assert float(out[dev(far)].abs().max()) == 0.0
+    rows = rng.permutation(n_out).astype(np.int32)
+    moved = layers._mc_project(*args, out_rows=dev(rows))
+    assert torch.equal(moved[dev(rows).long()], out)
