@@ -391,7 +391,7 @@ def main():
                              algorithmic_bytes=pby, GBps_dense=round(pby * calls / ms / 1e6, 1),
                              library="hipBLASLt via torch.matmul" if name.startswith("gemm_")
                              else "hand-written")
-        if name == "permute_rows":
+        if name in ("permute_rows", "gather_rows"):
             ops[name].update(GBps_copy=round(8 * N * C * calls / ms / 1e6, 1))
     kernel_ms = sum(v["ms"] for v in ops.values())
     ops["host_gaps_and_small_kernels"] = {"ms": round(ms_per_step - kernel_ms, 4)}
@@ -405,7 +405,11 @@ def main():
             "algorithmic_bytes": ops[dominant]["algorithmic_bytes"],
             "note": "algorithmic bytes count every per-pair feature row read (4*C per pair); "
                     "on the grid-ordered view most of those reads are served by L2, so "
-                    "`traffic` (HBM bytes measured by counters) is below them"}
+                    "`traffic` (HBM bytes measured by counters) is below them and `frac` can "
+                    "exceed 1; `traffic_frac` is the measured traffic over launch time and peak"}
+    if roof["traffic"]:
+        roof["traffic_frac"] = round(roof["traffic"] / (roof["launch_ms"] * 1e-3) / 1e9 /
+                                     HBM_PEAK_GBS, 4)
 
     result = {
         "metric": "MCConv layer fwd+bwd points/sec", "value": N / (ms_per_step * 1e-3),

@@ -99,7 +99,9 @@ int mccnn_grid_setup(mccnn_stream_t stream, int64_t num_pts, int num_dims,
  *   original ids  out[m] = (sorted_indices[neighbors[m,0]], neighbors[m,1])
  *                 pylib/pc/Neighborhood.py:246-250
  *   pdf per pair  out[m] = pdf[neighbors[m,0]]   pylib/pc/Neighborhood.py:287
- *   int32 gather  out[i] = src[indices[i]]       pylib/pc/sampling.py:142-146 */
+ *   int32 gather  out[i] = src[indices[i]]       pylib/pc/sampling.py:142-146
+ *   row gather    out[i,:] = src[indices[i],:]   (tf.gather of feature rows, e.g.
+ *                 pylib/pc/layers/utils.py:47; num_cols a multiple of 4, rows 16-byte aligned) */
 int mccnn_original_neighbor_ids(mccnn_stream_t stream, int64_t num_neighbors,
                                 const int32_t *neighbors,
                                 const int32_t *sorted_indices,
@@ -109,6 +111,8 @@ int mccnn_gather_pdf(mccnn_stream_t stream, int64_t num_neighbors,
                      float *pdf_per_pair_out);
 int mccnn_gather_i32(mccnn_stream_t stream, int64_t count, const int32_t *src,
                      const int32_t *indices, int32_t *out);
+int mccnn_gather_rows(mccnn_stream_t stream, int64_t num_rows, int num_cols, const float *src,
+                      const int32_t *indices, float *out);
 
 /* BuildGridDs: build_grid_ds/cc/ops/build_grid_ds_ops.cpp:27-115.
  * ds_out is int32 [batch_size, num_cells[0], num_cells[1], 2]: (first, last+1)

@@ -78,6 +78,19 @@ __global__ void __launch_bounds__(256) gather_i32_kernel(int64_t n, const int *_
     out[i] = src[idx[i]];
 }
 
+// out[i, :] = src[idx[i], :] for rows of 4 * row_vecs floats, 16 bytes per lane.
+__global__ void __launch_bounds__(256) gather_rows_kernel(int64_t total, int row_vecs,
+                                                          const float4 *__restrict__ src,
+                                                          const int *__restrict__ idx,
+                                                          float4 *__restrict__ out) {
+  for (int64_t t = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; t < total;
+       t += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t row = t / row_vecs;
+    const int v = (int)(t - row * row_vecs);
+    out[t] = src[(int64_t)idx[row] * row_vecs + v];
+  }
+}
+
 // ------------------------------------------------------------ grid table ----
 
 // Column of a key in the [B, n0, n1] table: key / prod(n[2:]).
@@ -358,6 +371,21 @@ extern "C" int mccnn_gather_pdf(mccnn_stream_t stream, int64_t num_neighbors,
   hipLaunchKernelGGL(gather_pdf_kernel, dim3(capped_grid(num_neighbors)), dim3(256), 0,
                      as_stream(stream), num_neighbors, (const int2 *)neighbors, pdf,
                      pdf_per_pair_out);
+  MCCNN_LAUNCH_CHECK();
+  return MCCNN_OK;
+}
+
+extern "C" int mccnn_gather_rows(mccnn_stream_t stream, int64_t num_rows, int num_cols,
+                                 const float *src, const int32_t *indices, float *out) {
+  MCCNN_REQUIRE(num_rows >= 0, "gather_rows expects a non-negative size");
+  MCCNN_REQUIRE(num_cols > 0 && num_cols % 4 == 0,
+                "gather_rows expects a row length that is a multiple of 4 (got %d)", num_cols);
+  if (num_rows == 0) return MCCNN_OK;
+  MCCNN_REQUIRE(src && indices && out, "gather_rows received a null tensor");
+  const int64_t total = num_rows * (num_cols / 4);
+  hipLaunchKernelGGL(gather_rows_kernel, dim3(capped_grid(total)), dim3(256), 0,
+                     as_stream(stream), total, num_cols / 4, (const float4 *)src, indices,
+                     (float4 *)out);
   MCCNN_LAUNCH_CHECK();
   return MCCNN_OK;
 }

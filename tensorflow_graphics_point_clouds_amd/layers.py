@@ -137,6 +137,17 @@ def _mc_layer(weights, biases, features, points_in, points_out, neighbors, range
     return out, proj
 
 
+def _gather_rows(x, rows):
+    """x[rows] for x [N, C] and int32 row indices."""
+    x = x.contiguous()
+    if x.shape[1] % 4 != 0:
+        return x.index_select(0, rows.long())
+    out = torch.empty((rows.shape[0], x.shape[1]), dtype=_F32, device=x.device)
+    _lib.call("gather_rows", stream(), i64(rows.shape[0]), cint(x.shape[1]), ptr(x, _F32),
+              ptr(rows, _I32), ptr(out))
+    return out
+
+
 def _weight_grad_product(x, y):
     """x^T y for [N, C] and [N, R] operands with the long reduction over N."""
     c, r = x.shape[1], y.shape[1]
@@ -196,8 +207,7 @@ class _MCConvLayer(torch.autograd.Function):
                 fuse_final):
         view = neighborhood.sorted_view()
         pdf, _ = view.pair_pdf(neighborhood)
-        with _lib.region("permute_rows"):
-            feats = features.index_select(0, view.point_order)
+        feats = _gather_rows(features, view.point_rows)
         dense = _dense_final_weights(final_weights, features.shape[1])
         if fuse_final:
             out, _ = _mc_layer(weights, biases, feats, view.points_in, view.points_out,
@@ -227,8 +237,7 @@ class _MCConvLayer(torch.autograd.Function):
         g = final_weights.shape[2]
         f = g * l
         if view.centre_order is not None:
-            with _lib.region("permute_rows"):
-                dout = dout.index_select(0, view.centre_order)
+            dout = _gather_rows(dout, view.centre_rows)
         else:
             dout = dout.contiguous()
         dense = _dense_final_weights(final_weights, c)               # [C*K, F]
@@ -603,8 +612,7 @@ class _KPConvRigidLayer(torch.autograd.Function):
     def forward(ctx, dense_weights, features, neighborhood, inv_radii, kernel_points, k, kind,
                 sigma):
         view = neighborhood.sorted_view()
-        with _lib.region("permute_rows"):
-            feats = features.index_select(0, view.point_order)
+        feats = _gather_rows(features, view.point_rows)
         # rows of the projection go straight to the centres' original positions
         proj = _kp_project(feats, view.points_in, view.points_out, view.table, view.ranges,
                            inv_radii, kernel_points, k, kind, sigma, view.centre_rows)
@@ -620,8 +628,7 @@ class _KPConvRigidLayer(torch.autograd.Function):
         view = ctx.neighborhood.sorted_view()
         k, c, f = ctx.k, feats.shape[1], dense.shape[1]
         if view.centre_order is not None:
-            with _lib.region("permute_rows"):
-                dout = dout.index_select(0, view.centre_order)
+            dout = _gather_rows(dout, view.centre_rows)
         else:
             dout = dout.contiguous()
         # rows of Q (and so of dfeat) go straight to the points' original positions
