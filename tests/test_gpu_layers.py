@@ -437,3 +437,70 @@ def test_projection_runs_with_empty_and_crowded_centres(oracle, d, c, n_out, rad
     rows = rng.permutation(n_out).astype(np.int32)
     moved = layers._mc_project(*args, out_rows=dev(rows))
     assert torch.equal(moved[dev(rows).long()], out)
+
+
+def test_mcconv_layer_at_full_scene_size():
+    """The benchmark configuration at its real size (8 clouds, 763 k points, 28 M
+    pairs, 64 -> 64 channels): rows of the output and of the feature gradient at
+    sampled points against float64 numpy on the layer's own pair table and
+    densities (whose integer parity is pinned elsewhere), and two properties over
+    the whole tensors: linearity in the features and <up, conv(x)> == <dfeat, x>."""
+    from tensorflow_graphics_point_clouds_amd import layers, pc, synthetic
+    cfg = synthetic.config3()
+    cloud = pc.PointCloud(dev(cfg["points"]), dev(cfg["batch_ids"]), cfg["batch_size"])
+    radius, c = cfg["radius"], 64
+    n = cloud._points.shape[0]
+    conv = layers.MCConv(c, c, 3, num_mlps=1, mlp_size=[16], non_linearity_type="leaky_relu", seed=3)
+    gen = torch.Generator(device="cuda").manual_seed(1)
+    x = torch.randn((n, c), device="cuda", generator=gen).requires_grad_(True)
+    y = torch.randn((n, c), device="cuda", generator=gen)
+    up = torch.randn((n, c), device="cuda", generator=gen)
+    out = conv(x, cloud, cloud, radius, bandwidth=0.2)
+    nbh = conv.last_neighborhood
+    out.backward(up)
+    dfeat = x.grad
+
+    with torch.no_grad():
+        out_y = conv(y, cloud, cloud, radius, neighborhood=nbh)
+        out_xy = conv(x.detach() + 2 * y, cloud, cloud, radius, neighborhood=nbh)
+        assert float((out_xy - (out + 2 * out_y)).abs().max()) <= 2e-5 * float(out_xy.abs().max())
+    lhs = float((up.double() * out.detach().double()).sum())
+    rhs = float((dfeat.double() * x.detach().double()).sum())
+    assert abs(lhs - rhs) <= 1e-5 * (float((up.double() * out.detach().double()).abs().sum()))
+
+    # sampled rows in float64
+    ids = nbh._original_neigh_ids.long()
+    ranges = nbh._samples_neigh_ranges.long()
+    pdf = nbh.get_pdf().double()
+    w = conv.weights.detach().double()[0]                # [3, 16]
+    b = conv.biases.detach().double().reshape(1, 16)
+    final = conv.final_weights.detach().double()[0]      # [C*16, C]
+    pts = cloud._points.double()
+    rng = np.random.default_rng(0)
+    picks = torch.as_tensor(rng.choice(n, 200, replace=False), device="cuda")
+    starts = torch.where(picks > 0, ranges[(picks - 1).clamp(min=0)], torch.zeros_like(picks))
+
+    def basis_of(seg):                                   # pairs seg -> [len, 16]
+        diff = (pts[ids[seg, 0]] - pts[ids[seg, 1]]) / radius
+        return torch.nn.functional.leaky_relu(diff @ w + b, 0.2) / pdf[seg].reshape(-1, 1)
+
+    xs, ups = x.detach().double(), up.double()
+    for centre, a, e in zip(picks.tolist(), starts.tolist(), ranges[picks].tolist()):
+        seg = torch.arange(a, e, device="cuda")
+        assert bool((ids[seg, 1] == centre).all())
+        proj = torch.einsum("mc,mk->ck", xs[ids[seg, 0]], basis_of(seg)).reshape(1, -1)
+        normwise(out[centre].detach().cpu().numpy(), (proj @ final).cpu().numpy()[0], tol=2e-5)
+    # the feature gradient of point j collects the pairs (j, i); the pairs of the
+    # self-neighbourhood are symmetric, so they are found through j's own segment
+    pair_key = ids[:, 0] * n + ids[:, 1]
+    order = torch.argsort(pair_key)
+    sorted_key = pair_key[order]
+    w3 = final.reshape(c, 16, c)
+    for j, a, e in list(zip(picks.tolist(), starts.tolist(), ranges[picks].tolist()))[:60]:
+        centres = ids[torch.arange(a, e, device="cuda"), 0]          # by symmetry: the i with j in N(i)
+        pos = torch.searchsorted(sorted_key, j * n + centres)
+        seg = order[pos]
+        assert bool((ids[seg, 0] == j).all()) and bool((ids[seg, 1] == centres).all())
+        dproj = torch.einsum("mf,ckf->mck", ups[centres], w3)         # [len, C, 16]
+        expect = torch.einsum("mck,mk->c", dproj, basis_of(seg))
+        normwise(dfeat[j].cpu().numpy(), expect.cpu().numpy(), tol=2e-5)
