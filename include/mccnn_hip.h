@@ -99,6 +99,7 @@ int mccnn_grid_setup(mccnn_stream_t stream, int64_t num_pts, int num_dims,
  *   original ids  out[m] = (sorted_indices[neighbors[m,0]], neighbors[m,1])
  *                 pylib/pc/Neighborhood.py:246-250
  *   pdf per pair  out[m] = pdf[neighbors[m,0]]   pylib/pc/Neighborhood.py:287
+ *                 (_column: of either column, for the transposed pair table)
  *   int32 gather  out[i] = src[indices[i]]       pylib/pc/sampling.py:142-146
  *   row gather    out[i,:] = src[indices[i],:]   (tf.gather of feature rows, e.g.
  *                 pylib/pc/layers/utils.py:47; num_cols a multiple of 4, rows 16-byte aligned) */
@@ -109,6 +110,9 @@ int mccnn_original_neighbor_ids(mccnn_stream_t stream, int64_t num_neighbors,
 int mccnn_gather_pdf(mccnn_stream_t stream, int64_t num_neighbors,
                      const int32_t *neighbors, const float *pdf,
                      float *pdf_per_pair_out);
+int mccnn_gather_pdf_column(mccnn_stream_t stream, int64_t num_neighbors,
+                            const int32_t *neighbors, int column, const float *pdf,
+                            float *pdf_per_pair_out);
 int mccnn_gather_i32(mccnn_stream_t stream, int64_t count, const int32_t *src,
                      const int32_t *indices, int32_t *out);
 int mccnn_gather_rows(mccnn_stream_t stream, int64_t num_rows, int num_cols, const float *src,

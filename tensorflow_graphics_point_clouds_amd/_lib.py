@@ -4,6 +4,7 @@ built, or a tensor is not a contiguous GPU tensor of the right dtype, the call
 raises."""
 import ctypes
 import os
+import threading
 import subprocess
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
@@ -81,6 +82,22 @@ def ptr(t, dtype=None):
     if not t.is_contiguous():
         raise TypeError("expected a contiguous tensor")
     return vptr(t.data_ptr())
+
+
+_host_counts = threading.local()
+
+
+def host_count():
+    """One int64 in pinned host memory per thread: the `_count` halves of the
+    dynamic-size ops copy their total there, and a device-to-host copy into pinned
+    memory completes without the staging a pageable destination needs.
+    -> (tensor [1], pointer)."""
+    import torch
+    t = getattr(_host_counts, "tensor", None)
+    if t is None:
+        t = torch.zeros(1, dtype=torch.int64, pin_memory=True)
+        _host_counts.tensor = t
+    return t, vptr(t.data_ptr())
 
 
 def workspace(nbytes, device):

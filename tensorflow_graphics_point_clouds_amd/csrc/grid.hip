@@ -63,11 +63,13 @@ __global__ void __launch_bounds__(256) original_ids_kernel(int64_t m,
 }
 
 __global__ void __launch_bounds__(256) gather_pdf_kernel(int64_t m, const int2 *__restrict__ nbrs,
-                                                         const float *__restrict__ pdf,
+                                                         int column, const float *__restrict__ pdf,
                                                          float *__restrict__ out) {
   for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < m;
-       i += (int64_t)gridDim.x * blockDim.x)
-    out[i] = pdf[nbrs[i].x];
+       i += (int64_t)gridDim.x * blockDim.x) {
+    const int2 p = nbrs[i];
+    out[i] = pdf[column == 0 ? p.x : p.y];
+  }
 }
 
 __global__ void __launch_bounds__(256) gather_i32_kernel(int64_t n, const int *__restrict__ src,
@@ -362,17 +364,24 @@ extern "C" int mccnn_original_neighbor_ids(mccnn_stream_t stream, int64_t num_ne
   return MCCNN_OK;
 }
 
-extern "C" int mccnn_gather_pdf(mccnn_stream_t stream, int64_t num_neighbors,
-                                const int32_t *neighbors, const float *pdf,
-                                float *pdf_per_pair_out) {
+extern "C" int mccnn_gather_pdf_column(mccnn_stream_t stream, int64_t num_neighbors,
+                                       const int32_t *neighbors, int column, const float *pdf,
+                                       float *pdf_per_pair_out) {
   MCCNN_REQUIRE(num_neighbors >= 0, "gather_pdf expects a non-negative size");
+  MCCNN_REQUIRE(column == 0 || column == 1, "gather_pdf expects column 0 or 1 (got %d)", column);
   if (num_neighbors == 0) return MCCNN_OK;
   MCCNN_REQUIRE(neighbors && pdf && pdf_per_pair_out, "gather_pdf received a null tensor");
   hipLaunchKernelGGL(gather_pdf_kernel, dim3(capped_grid(num_neighbors)), dim3(256), 0,
-                     as_stream(stream), num_neighbors, (const int2 *)neighbors, pdf,
+                     as_stream(stream), num_neighbors, (const int2 *)neighbors, column, pdf,
                      pdf_per_pair_out);
   MCCNN_LAUNCH_CHECK();
   return MCCNN_OK;
+}
+
+extern "C" int mccnn_gather_pdf(mccnn_stream_t stream, int64_t num_neighbors,
+                                const int32_t *neighbors, const float *pdf,
+                                float *pdf_per_pair_out) {
+  return mccnn_gather_pdf_column(stream, num_neighbors, neighbors, 0, pdf, pdf_per_pair_out);
 }
 
 extern "C" int mccnn_gather_rows(mccnn_stream_t stream, int64_t num_rows, int num_cols,

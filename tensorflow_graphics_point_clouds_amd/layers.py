@@ -372,7 +372,7 @@ class MCConv(torch.nn.Module):
             grid = pc.Grid(point_cloud_in, radii)
             neighborhood = pc.Neighborhood(grid, radii, point_cloud_out)
         self.last_neighborhood = neighborhood
-        pdf = neighborhood.get_pdf(bandwidth=bandwidth, mode=pc.KDEMode.constant)
+        neighborhood.point_pdf(bandwidth=bandwidth, mode=pc.KDEMode.constant)
         biases = self.biases.reshape(self._num_mlps, self._hidden)
         k = self._num_mlps * self._hidden
         fused = self.fused and _lib.lib().mccnn_mc_conv_supported(
@@ -381,6 +381,7 @@ class MCConv(torch.nn.Module):
             out = self._convolve_on_view(features, neighborhood, radii, biases, k)
             if out is not None:
                 return out
+        pdf = neighborhood.get_pdf()
         transposed = None
         if self.gathered_grads and features.requires_grad and \
                 tfg_custom_ops.gathered_grads_supported(self._num_features_in, k):
@@ -717,13 +718,13 @@ class KPConv(torch.nn.Module):
             grid = pc.Grid(point_cloud_in, radii)
             neighborhood = pc.Neighborhood(grid, radii, point_cloud_out)
         self.last_neighborhood = neighborhood
-        ids, ranges = neighborhood._original_neigh_ids, neighborhood._samples_neigh_ranges
         kp, k, c = self._num_kernel_points, self._num_basis, self._num_features_in
         features = features.contiguous()
         if not self.deformable and self.transposed_grads:
             return _KPConvRigidLayer.apply(self._padded(self.weights), features, neighborhood,
                                            torch.reciprocal(radii), self._kernel_points, k,
                                            self._kind, sigma)
+        ids, ranges = neighborhood._original_neigh_ids, neighborhood._samples_neigh_ranges
         transposed = None
         if features.requires_grad and tfg_custom_ops.gathered_grads_supported(c, k):
             transposed = neighborhood.transposed_pairs()

@@ -309,8 +309,11 @@ class _SortedView:
                 self.pdf = self.pdf_t = torch.ones(m, dtype=_F32, device=dev)
             else:
                 per_point = per_point.detach()
-                self.pdf = per_point[self.table[:, 0].long()].contiguous()
-                self.pdf_t = per_point[self.table_t[:, 1].long()].contiguous()
+                self.pdf = torch.empty(m, dtype=_F32, device=dev)
+                self.pdf_t = torch.empty(m, dtype=_F32, device=dev)
+                for out, table, column in ((self.pdf, self.table, 0), (self.pdf_t, self.table_t, 1)):
+                    _lib.call("gather_pdf_column", stream(), i64(m), ptr(table, _I32), cint(column),
+                              ptr(per_point, _F32), ptr(out))
             self._pdf_key = key
         return self.pdf, self.pdf_t
 
@@ -335,39 +338,67 @@ class Neighborhood:
         self._inv_radii = torch.reciprocal(self._radii)
         s = self._point_cloud_sampled
         self._self_neighborhood = None
+        self._table = self._ranges = self._original = None
         if point_cloud_sample is grid._point_cloud:
             # The centres are the grid's own points in the caller's order: search once
             # from the sorted points (consecutive centres then walk the same cells;
             # the same search also serves the densities and the grid-ordered view of
-            # the layers) and regroup the segments.  The pairs of a centre depend on
-            # its coordinates only, so the table equals that of a direct search.
-            own = grid.self_neighborhood(self._radii, max_neighbors)
-            self._self_neighborhood = own
-            n = s._points.shape[0]
-            L = _lib.lib()
-            ws = _lib.workspace(L.mccnn_reorder_neighbors_workspace_bytes(i64(n)), dev)
-            self._samples_neigh_ranges = torch.empty_like(own._samples_neigh_ranges)
-            self._neighbors = torch.empty_like(own._neighbors)
-            _lib.call("reorder_neighbors", stream(), i64(n), ptr(own._samples_neigh_ranges, _I32),
-                      i64(own._neighbors.shape[0]), ptr(own._neighbors, _I32),
-                      ptr(grid.sorted_positions(), _I32), ptr(ws), _lib.csize(ws.numel()),
-                      ptr(self._samples_neigh_ranges), ptr(self._neighbors))
+            # the layers).  The table in the caller's centre order is the same
+            # segments regrouped (the pairs of a centre depend on its coordinates
+            # only); it is built when somebody asks for it, which the layers on the
+            # grid-ordered view never do.
+            self._self_neighborhood = grid.self_neighborhood(self._radii, max_neighbors)
         else:
-            self._samples_neigh_ranges, self._neighbors = tfg_custom_ops.find_neighbors(
+            self._ranges, self._table = tfg_custom_ops.find_neighbors(
                 s._points, s._batch_ids, grid._sorted_points, grid._sorted_keys, grid.get_DS(),
                 grid._num_cells, grid._scaled_aabb_min, grid._inv_cell_sizes, self._inv_radii,
                 max_neighbors)
-        # pairs addressed by original point ids (Neighborhood.py:246-250)
-        self._original_neigh_ids = torch.empty_like(self._neighbors)
-        _lib.call("original_neighbor_ids", stream(), i64(self._neighbors.shape[0]), ptr(self._neighbors, _I32),
-            ptr(grid._sorted_indices, _I32), ptr(self._original_neigh_ids))
         self._pdf = None
         self._pdf_per_point = None
+        self._pdf_args = None
         # optional visiting order of the centres for the projection kernels
         self._centre_order = None
         self._transposed_pairs = None
         self._sorted_view = None
         self._transposed = None
+
+    def _regroup(self):
+        own, grid = self._self_neighborhood, self._grid
+        n = self._point_cloud_sampled._points.shape[0]
+        dev = own._neighbors.device
+        L = _lib.lib()
+        ws = _lib.workspace(L.mccnn_reorder_neighbors_workspace_bytes(i64(n)), dev)
+        self._ranges = torch.empty_like(own._samples_neigh_ranges)
+        self._table = torch.empty_like(own._neighbors)
+        _lib.call("reorder_neighbors", stream(), i64(n), ptr(own._samples_neigh_ranges, _I32),
+                  i64(own._neighbors.shape[0]), ptr(own._neighbors, _I32),
+                  ptr(grid.sorted_positions(), _I32), ptr(ws), _lib.csize(ws.numel()),
+                  ptr(self._ranges), ptr(self._table))
+
+    @property
+    def _neighbors(self):
+        """[M, 2] pairs (sorted point index, centre index), grouped by centre."""
+        if self._table is None:
+            self._regroup()
+        return self._table
+
+    @property
+    def _samples_neigh_ranges(self):
+        """[N_out] inclusive end offset of every centre's pairs."""
+        if self._ranges is None:
+            self._regroup()
+        return self._ranges
+
+    @property
+    def _original_neigh_ids(self):
+        """The pairs addressed by original point ids (Neighborhood.py:246-250);
+        built on first use."""
+        if self._original is None:
+            nb = self._neighbors
+            self._original = torch.empty_like(nb)
+            _lib.call("original_neighbor_ids", stream(), i64(nb.shape[0]), ptr(nb, _I32),
+                      ptr(self._grid._sorted_indices, _I32), ptr(self._original))
+        return self._original
 
     def transposed_pairs(self):
         """(point_ranges, pair_order): the pairs grouped by neighbour point, used by
@@ -411,26 +442,43 @@ class Neighborhood:
         return self._centre_order
 
     def compute_pdf(self, bandwidth=0.2, mode=KDEMode.constant, normalize=False):
-        d = self._grid._point_cloud._dimension
-        dev = self._neighbors.device
-        if mode == KDEMode.no_pdf:
-            self._pdf = torch.ones(self._neighbors.shape[0], dtype=_F32, device=dev)
-        else:
-            nbh = self if self._equal_samples else self._grid.self_neighborhood(self._radii)
-            bw = _as_vector(bandwidth, d, dev)
-            self._pdf_per_point = tfg_custom_ops.compute_pdf_with_pt_grads(
-                self._grid._sorted_points, nbh._neighbors, nbh._samples_neigh_ranges,
-                torch.reciprocal(bw), nbh._inv_radii, mode.value,
-                symmetric=nbh._equal_samples and nbh.max_neighbors == 0)
-            self._pdf = torch.empty(self._neighbors.shape[0], dtype=_F32, device=dev)
-            _lib.call("gather_pdf", stream(), i64(self._neighbors.shape[0]), ptr(self._neighbors, _I32),
-                ptr(self._pdf_per_point.detach(), _F32), ptr(self._pdf))
+        """Densities of the grid's points from their self-neighbourhood
+        (Neighborhood.py:257-293); the per-pair values follow on `get_pdf()`."""
         if normalize:
             raise NotImplementedError("normalised densities are not part of the op path")
+        d = self._grid._point_cloud._dimension
+        dev = self._grid._sorted_points.device
+        self._pdf = None
+        self._pdf_args = (bandwidth, mode)
+        if mode == KDEMode.no_pdf:
+            self._pdf_per_point = None
+            return
+        nbh = self if self._equal_samples else self._grid.self_neighborhood(self._radii)
+        bw = _as_vector(bandwidth, d, dev)
+        self._pdf_per_point = tfg_custom_ops.compute_pdf_with_pt_grads(
+            self._grid._sorted_points, nbh._neighbors, nbh._samples_neigh_ranges,
+            torch.reciprocal(bw), nbh._inv_radii, mode.value,
+            symmetric=nbh._equal_samples and nbh.max_neighbors == 0)
+
+    def point_pdf(self, **kwargs):
+        """Density per sorted point (None with KDEMode.no_pdf), computed on first use
+        with `kwargs` as for `compute_pdf`."""
+        if self._pdf_args is None:
+            self.compute_pdf(**kwargs)
+        return self._pdf_per_point
 
     def get_pdf(self, **kwargs):
+        """Density of the neighbour point of every pair of `_neighbors`
+        (Neighborhood.py:287)."""
+        per_point = self.point_pdf(**kwargs)
         if self._pdf is None:
-            self.compute_pdf(**kwargs)
+            nb = self._neighbors
+            if per_point is None:
+                self._pdf = torch.ones(nb.shape[0], dtype=_F32, device=nb.device)
+            else:
+                self._pdf = torch.empty(nb.shape[0], dtype=_F32, device=nb.device)
+                _lib.call("gather_pdf", stream(), i64(nb.shape[0]), ptr(nb, _I32),
+                          ptr(per_point.detach(), _F32), ptr(self._pdf))
         return self._pdf
 
 

@@ -63,7 +63,7 @@ def find_neighbors(samples, samples_batch_ids, points, point_keys, grid_acc_ds, 
     ws_bytes = L.mccnn_find_neighbors_workspace_bytes(cint(nd), i64(ns))
     ws = _lib.workspace(ws_bytes, dev)
     ranges = torch.empty(ns, dtype=_I32, device=dev)
-    total = ctypes.c_int64(0)
+    total, total_ptr = _lib.host_count()
     dsr = grid_acc_ds.dim()
     _lib.call("find_neighbors_count", stream(), i64(ns), cint(nd), ptr(samples, _F32), i64(samples_batch_ids.shape[0]),
         ptr(samples_batch_ids, _I32), i64(points.shape[0]), cint(_dim(points, 1)),
@@ -73,8 +73,8 @@ def find_neighbors(samples, samples_batch_ids, points, point_keys, grid_acc_ds, 
         ptr(num_cells, _I32), cint(_dim(scaled_aabb_min, 1)), ptr(scaled_aabb_min, _F32),
         cint(inv_cell_sizes.shape[0]), ptr(inv_cell_sizes, _F32), cint(inv_radii.shape[0]),
         ptr(inv_radii, _F32), cint(max_neighs), ptr(ws), _lib.csize(ws.numel()), ptr(ranges),
-        ctypes.byref(total))
-    m = int(total.value)
+        total_ptr)
+    m = int(total[0])
     neighbors = torch.empty((m, 2), dtype=_I32, device=dev)
     _lib.call("find_neighbors_fill", stream(), i64(ns), cint(nd), ptr(samples, _F32), ptr(samples_batch_ids, _I32),
         i64(points.shape[0]), ptr(points, _F32), ptr(point_keys, _I64), ptr(grid_acc_ds, _I32),
@@ -92,14 +92,14 @@ def sampling(points, batch_ids, point_keys, num_cells, neighbors, sample_neigh_i
     n, nd = points.shape[0], _dim(points, 1)
     dev = points.device
     ws = _lib.workspace(L.mccnn_sampling_workspace_bytes(i64(n)), dev)
-    total = ctypes.c_int64(0)
+    total, total_ptr = _lib.host_count()
     _lib.call("sampling_count", stream(), cint(mode), i64(n), cint(nd), ptr(points, _F32), i64(batch_ids.shape[0]),
         ptr(batch_ids, _I32), i64(point_keys.shape[0]), ptr(point_keys, _I64),
         cint(num_cells.shape[0]), ptr(num_cells, _I32), i64(neighbors.shape[0]),
         cint(neighbors.dim()), cint(_dim(neighbors, 1)), ptr(neighbors, _I32),
         i64(sample_neigh_indices.shape[0]), ptr(sample_neigh_indices, _I32), ptr(ws),
-        _lib.csize(ws.numel()), ctypes.byref(total))
-    s = int(total.value)
+        _lib.csize(ws.numel()), total_ptr)
+    s = int(total[0])
     out_pts = torch.empty((s, nd), dtype=_F32, device=dev)
     out_bids = torch.empty(s, dtype=_I32, device=dev)
     out_idx = torch.empty(s, dtype=_I32, device=dev)
