@@ -300,18 +300,28 @@ class MCConv(torch.nn.Module):
         if num_features_out % num_mlps != 0:
             raise ValueError("The number of output features must be divisible by the number"
                              " of kernel MLPs")
-        if len(mlp_size) != 1:
-            raise NotImplementedError("only one hidden layer is evaluated by the HIP kernel")
-        hidden = int(mlp_size[0])
+        if len(mlp_size) < 1:
+            raise ValueError("mlp_size needs at least one layer")
+        first, hidden = int(mlp_size[0]), int(mlp_size[-1])
         self._num_features_in, self._num_features_out = num_features_in, num_features_out
         self._num_dims, self._num_mlps, self._hidden = num_dims, num_mlps, hidden
         self._act = _ACTIVATIONS[non_linearity_type.lower()]
         gen = torch.Generator().manual_seed(seed)
         if weights is None:      # MCConv.py:100-135: truncated normal, He scale
-            weights = _truncated_normal((num_mlps, num_dims, hidden),
+            weights = _truncated_normal((num_mlps, num_dims, first),
                                         math.sqrt(2.0 / num_dims), gen, device)
         if biases is None:
-            biases = torch.zeros((num_mlps, 1, hidden), dtype=_F32, device=device)
+            biases = torch.zeros((num_mlps, 1, first), dtype=_F32, device=device)
+        # Kernel MLPs with further layers (MCConv.py:100-120: scale sqrt(1 / fan-in)):
+        # the HIP kernels evaluate one-layer kernels in registers; deeper ones are
+        # evaluated per pair with dense products and handed to basis_proj.
+        self.deep_weights = torch.nn.ParameterList()
+        self.deep_biases = torch.nn.ParameterList()
+        for prev, cur in zip(mlp_size[:-1], mlp_size[1:]):
+            self.deep_weights.append(torch.nn.Parameter(_truncated_normal(
+                (num_mlps, int(prev), int(cur)), math.sqrt(1.0 / int(prev)), gen, device)))
+            self.deep_biases.append(torch.nn.Parameter(
+                torch.zeros((num_mlps, 1, int(cur)), dtype=_F32, device=device)))
         if final_weights is None:
             final_weights = _truncated_normal(
                 (num_mlps, hidden * num_features_in, num_features_out // num_mlps),
@@ -335,6 +345,28 @@ class MCConv(torch.nn.Module):
         out = self._convolve(features, point_cloud_in, point_cloud_out, radius, neighborhood,
                              bandwidth)
         return point_cloud_out.format_output(out, return_sorted, return_padded)
+
+    def _convolve_deep(self, features, point_cloud_in, point_cloud_out, radii, neighborhood):
+        """Kernel MLPs of several layers (MCConv.py:163-194): per-pair offsets through
+        the layers as batched dense products, divided by the densities, then
+        basis_proj and the final product.  The [M, K] basis is materialised, as in
+        the reference."""
+        ids = neighborhood._original_neigh_ids.long()
+        l, c, h = self._num_mlps, self._num_features_in, self._hidden
+        diff = (point_cloud_in._points[ids[:, 0]] - point_cloud_out._points[ids[:, 1]]) / radii
+        cur = diff.unsqueeze(0).expand(l, -1, -1)
+        layers_w = [self.weights] + list(self.deep_weights)
+        layers_b = [self.biases] + list(self.deep_biases)
+        for w, b in zip(layers_w, layers_b):
+            cur = _activate(torch.bmm(cur, w) + b, self._act)
+        basis = cur.permute(1, 0, 2).reshape(ids.shape[0], l * h) / \
+            neighborhood.get_pdf().reshape(-1, 1)
+        proj = tfg_custom_ops.basis_proj(basis.contiguous(), features.contiguous(),
+                                         neighborhood._original_neigh_ids,
+                                         neighborhood._samples_neigh_ranges)
+        n = proj.shape[0]
+        p = proj.reshape(n, c, l, h).permute(2, 0, 1, 3).reshape(l, n, c * h)
+        return torch.bmm(p, self.final_weights).permute(1, 0, 2).reshape(n, -1)
 
     def _convolve_on_view(self, features, neighborhood, radii, biases, k):
         """The fused path on the grid-ordered view; channel counts it does not cover
@@ -373,6 +405,9 @@ class MCConv(torch.nn.Module):
             neighborhood = pc.Neighborhood(grid, radii, point_cloud_out)
         self.last_neighborhood = neighborhood
         neighborhood.point_pdf(bandwidth=bandwidth, mode=pc.KDEMode.constant)
+        if len(self.deep_weights) > 0:
+            return self._convolve_deep(features, point_cloud_in, point_cloud_out, radii,
+                                       neighborhood)
         biases = self.biases.reshape(self._num_mlps, self._hidden)
         k = self._num_mlps * self._hidden
         fused = self.fused and _lib.lib().mccnn_mc_conv_supported(
@@ -405,6 +440,14 @@ class MCConv(torch.nn.Module):
             return proj.reshape(n, c * h) @ self.final_weights[0]
         p = proj.reshape(n, c, l, h).permute(2, 0, 1, 3).reshape(l, n, c * h)
         return torch.bmm(p, self.final_weights).permute(1, 0, 2).reshape(n, -1)
+
+
+def _activate(x, act):
+    if act == 0:
+        return torch.relu(x)
+    if act == 1:
+        return torch.nn.functional.leaky_relu(x, 0.2)
+    return torch.nn.functional.elu(x)
 
 
 def _layer_padding(c, f, num_mlps):
