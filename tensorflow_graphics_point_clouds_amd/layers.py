@@ -346,11 +346,14 @@ class MCConv(torch.nn.Module):
                              bandwidth)
         return point_cloud_out.format_output(out, return_sorted, return_padded)
 
-    def _convolve_deep(self, features, point_cloud_in, point_cloud_out, radii, neighborhood):
-        """Kernel MLPs of several layers (MCConv.py:163-194): per-pair offsets through
-        the layers as batched dense products, divided by the densities, then
-        basis_proj and the final product.  The [M, K] basis is materialised, as in
-        the reference."""
+    def _convolve_deep(self, features, point_cloud_in, point_cloud_out, radii, neighborhood,
+                       pdf=None):
+        """The layer as the reference composes it (MCConv.py:163-194), differentiable
+        in everything: per-pair offsets through the layers of the kernel MLPs as
+        batched dense products, divided by the densities, then basis_proj and the
+        final product.  Used for kernel MLPs of several layers and for point
+        clouds whose coordinates require a gradient; the [M, K] basis is
+        materialised, as in the reference."""
         ids = neighborhood._original_neigh_ids.long()
         l, c, h = self._num_mlps, self._num_features_in, self._hidden
         diff = (point_cloud_in._points[ids[:, 0]] - point_cloud_out._points[ids[:, 1]]) / radii
@@ -359,8 +362,8 @@ class MCConv(torch.nn.Module):
         layers_b = [self.biases] + list(self.deep_biases)
         for w, b in zip(layers_w, layers_b):
             cur = _activate(torch.bmm(cur, w) + b, self._act)
-        basis = cur.permute(1, 0, 2).reshape(ids.shape[0], l * h) / \
-            neighborhood.get_pdf().reshape(-1, 1)
+        pdf = neighborhood.get_pdf() if pdf is None else pdf
+        basis = cur.permute(1, 0, 2).reshape(ids.shape[0], l * h) / pdf.reshape(-1, 1)
         proj = tfg_custom_ops.basis_proj(basis.contiguous(), features.contiguous(),
                                          neighborhood._original_neigh_ids,
                                          neighborhood._samples_neigh_ranges)
@@ -405,9 +408,11 @@ class MCConv(torch.nn.Module):
             neighborhood = pc.Neighborhood(grid, radii, point_cloud_out)
         self.last_neighborhood = neighborhood
         neighborhood.point_pdf(bandwidth=bandwidth, mode=pc.KDEMode.constant)
-        if len(self.deep_weights) > 0:
+        moving = _moving(point_cloud_in, point_cloud_out)
+        if len(self.deep_weights) > 0 or moving:
+            pdf = _differentiable_pdf(neighborhood, bandwidth) if moving else None
             return self._convolve_deep(features, point_cloud_in, point_cloud_out, radii,
-                                       neighborhood)
+                                       neighborhood, pdf)
         biases = self.biases.reshape(self._num_mlps, self._hidden)
         k = self._num_mlps * self._hidden
         fused = self.fused and _lib.lib().mccnn_mc_conv_supported(
@@ -440,6 +445,27 @@ class MCConv(torch.nn.Module):
             return proj.reshape(n, c * h) @ self.final_weights[0]
         p = proj.reshape(n, c, l, h).permute(2, 0, 1, 3).reshape(l, n, c * h)
         return torch.bmm(p, self.final_weights).permute(1, 0, 2).reshape(n, -1)
+
+
+def _differentiable_pdf(neighborhood, bandwidth):
+    """Per-pair densities as a function of the grid cloud's point coordinates
+    (the gradient registered for ComputePdfWithPtGrads,
+    custom_ops_wrapper.py:159-169), for point clouds whose coordinates require a
+    gradient."""
+    grid = neighborhood._grid
+    points = grid._point_cloud._points
+    d, dev = points.shape[1], points.device
+    own = neighborhood if neighborhood._equal_samples else \
+        grid.self_neighborhood(neighborhood._radii)
+    per_point = tfg_custom_ops.compute_pdf_with_pt_grads(
+        points[grid._sorted_indices.long()], own._neighbors, own._samples_neigh_ranges,
+        torch.reciprocal(pc._as_vector(bandwidth, d, dev)), own._inv_radii,
+        pc.KDEMode.constant.value, symmetric=own._equal_samples and own.max_neighbors == 0)
+    return per_point[neighborhood._neighbors[:, 0].long()]
+
+
+def _moving(*clouds):
+    return any(c._points.requires_grad for c in clouds)
 
 
 def _activate(x, act):
@@ -515,15 +541,22 @@ class PointConv(torch.nn.Module):
             grid = pc.Grid(point_cloud_in, radii)
             neighborhood = pc.Neighborhood(grid, radii, point_cloud_out)
         self.last_neighborhood = neighborhood
-        pdf = neighborhood.get_pdf(bandwidth=bandwidth, mode=pc.KDEMode.constant)
         ids, ranges = neighborhood._original_neigh_ids, neighborhood._samples_neigh_ranges
         m, n_out = ids.shape[0], ranges.shape[0]
-        # hidden layer on the unscaled offsets (PointConv.py:268-272): unit radii, unit pdf
-        ones_d = torch.ones(d, dtype=_F32, device=dev)
-        hidden = _MCBasis.apply(self.weights.reshape(1, d, self._size_hidden),
-                                self.biases.reshape(1, self._size_hidden),
-                                point_cloud_in._points, point_cloud_out._points, ids, ones_d,
-                                torch.ones(m, dtype=_F32, device=dev), self._act)
+        if _moving(point_cloud_in, point_cloud_out):
+            # coordinates that require a gradient: the same expressions in torch
+            pdf = _differentiable_pdf(neighborhood, bandwidth)
+            diff = point_cloud_in._points[ids[:, 0].long()] - \
+                point_cloud_out._points[ids[:, 1].long()]
+            hidden = _activate(diff @ self.weights + self.biases, self._act)
+        else:
+            pdf = neighborhood.get_pdf(bandwidth=bandwidth, mode=pc.KDEMode.constant)
+            # hidden layer on the unscaled offsets (PointConv.py:268-272): unit radii, unit pdf
+            ones_d = torch.ones(d, dtype=_F32, device=dev)
+            hidden = _MCBasis.apply(self.weights.reshape(1, d, self._size_hidden),
+                                    self.biases.reshape(1, self._size_hidden),
+                                    point_cloud_in._points, point_cloud_out._points, ids, ones_d,
+                                    torch.ones(m, dtype=_F32, device=dev), self._act)
         # densities relative to the largest of their neighbourhood, then the pdf MLP
         # (PointConv.py:166-177)
         centre = ids[:, 1].long()
@@ -763,6 +796,9 @@ class KPConv(torch.nn.Module):
         self.last_neighborhood = neighborhood
         kp, k, c = self._num_kernel_points, self._num_basis, self._num_features_in
         features = features.contiguous()
+        if _moving(point_cloud_in, point_cloud_out):
+            return self._convolve_moving(features, point_cloud_in, point_cloud_out, radii,
+                                         neighborhood, sigma)
         if not self.deformable and self.transposed_grads:
             return _KPConvRigidLayer.apply(self._padded(self.weights), features, neighborhood,
                                            torch.reciprocal(radii), self._kernel_points, k,
@@ -786,6 +822,43 @@ class KPConv(torch.nn.Module):
         self._last = (offsets, geometry, sigma)
         basis = _KPBasis.apply(offsets, *geometry, k, self._kind, sigma)
         return project(basis).reshape(-1, c * k) @ self._padded(self.weights)
+
+    def _convolve_moving(self, features, point_cloud_in, point_cloud_out, radii, neighborhood,
+                         sigma):
+        """KPConv.py:165-232, 317-392 with the kernel-point correlation written in
+        torch, for point clouds whose coordinates require a gradient (the norm is
+        taken with a floor of 1e-10 so that a point sitting on a kernel point has
+        a finite gradient)."""
+        kp, k, c, d = self._num_kernel_points, self._num_basis, self._num_features_in, \
+            self._num_dims
+        ids, ranges = neighborhood._original_neigh_ids, neighborhood._samples_neigh_ranges
+        centre = ids[:, 1].long()
+        diff = (point_cloud_in._points[ids[:, 0].long()] - point_cloud_out._points[centre]) / radii
+
+        def correlation(offsets):
+            delta = diff[:, None, :] - self._kernel_points[None]
+            if offsets is not None:
+                delta = delta - offsets[centre]
+            dist = torch.sqrt((delta * delta).sum(dim=2) + 1e-20)
+            if self._kind == 0:
+                wgt = torch.relu(1.0 - dist / sigma)
+            else:
+                wgt = torch.exp(-(dist / (sigma / 3.0)) ** 2)
+            return torch.nn.functional.pad(wgt, (0, k - kp)).contiguous()
+
+        def project(basis):
+            return tfg_custom_ops.basis_proj(basis, features, ids, ranges).reshape(-1, c * k)
+
+        offsets = None
+        if self.deformable:
+            offsets = (project(correlation(None)) @ self._padded(self.offset_weights))
+            offsets = offsets.reshape(-1, kp, d)
+        self._last = None
+        if self.deformable:
+            geometry = (point_cloud_in._points.detach(), point_cloud_out._points.detach(), ids,
+                        ranges, torch.reciprocal(radii), self._kernel_points)
+            self._last = (offsets, geometry, sigma)
+        return project(correlation(offsets)) @ self._padded(self.weights)
 
     def regularization_loss(self):
         """Fitting + repulsive loss of the last deformable call (KPConv.py:394-429)."""

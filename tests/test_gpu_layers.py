@@ -549,3 +549,127 @@ def test_mcconv_with_deeper_kernel_mlp(oracle, mlp_size, num_mlps, act):
     normwise(tfeat.grad.cpu().numpy(), tf.grad.numpy(), tol=2e-5)
     for p, r in zip(params, ref):
         normwise(p.grad.cpu().numpy(), r.grad.numpy(), tol=5e-5)
+
+
+def test_mcconv_gradient_with_respect_to_points(oracle):
+    """Point coordinates that require a gradient (monte_carlo_conv_test.py:196-230
+    checks this Jacobian): the layer output depends on them through the kernel
+    inputs and through the densities.  Against float64 autograd of the whole
+    expression, Gaussian KDE included, on the oracle's pair tables."""
+    from tensorflow_graphics_point_clouds_amd import layers, pc
+    rng = np.random.default_rng(5)
+    n, batch, radius, bw, c_in, c_out, hidden = 600, 2, 0.25, 0.2, 4, 6, 8
+    pts = rng.random((n, 3)).astype(np.float32)
+    bids = np.sort(rng.integers(0, batch, n)).astype(np.int32)
+    feat = rng.standard_normal((n, c_in)).astype(np.float32)
+    g = oracle.Grid(pts, bids, batch, np.float32(radius))
+    own = oracle.Neighborhood(g, np.float32(radius))                 # sorted self-neighbourhood
+    nbh = oracle.Neighborhood(g, np.float32(radius), pts, bids)     # centres in the caller's order
+    conv = layers.MCConv(c_in, c_out, 3, num_mlps=1, mlp_size=[hidden], non_linearity_type="elu",
+                         seed=2)
+    tpts = dev(pts).requires_grad_(True)
+    cloud = pc.PointCloud(tpts, dev(bids), batch)
+    out = conv(dev(feat), cloud, cloud, radius, bandwidth=bw)
+    up = rng.standard_normal(tuple(out.shape)).astype(np.float32)
+    out.backward(dev(up))
+
+    p = torch.tensor(pts.astype(np.float64), requires_grad=True)
+    order = torch.tensor(g.sorted_indices).long()
+    sp = p[order]
+    on = torch.tensor(own.neighbors).long()
+    u = (sp[on[:, 0]] - sp[on[:, 1]]) / (bw * radius)
+    kde = torch.prod(torch.exp(-0.5 * u * u) * (0.3989422804014327 / bw), dim=1)
+    per_point = torch.zeros(n, dtype=torch.float64).index_add(0, on[:, 1], kde)
+    ids = torch.tensor(nbh.original_neigh_ids).long()
+    pdf = per_point[torch.tensor(nbh.neighbors[:, 0]).long()]
+    w, b = conv.weights.detach().cpu().double()[0], conv.biases.detach().cpu().double()[0]
+    basis = torch.nn.functional.elu(((p[ids[:, 0]] - p[ids[:, 1]]) / radius) @ w + b) / pdf[:, None]
+    per_pair = torch.tensor(feat.astype(np.float64))[ids[:, 0]][:, :, None] * basis[:, None, :]
+    proj = torch.zeros(n, c_in, hidden, dtype=torch.float64).index_add(0, ids[:, 1], per_pair)
+    ref = proj.reshape(n, -1) @ conv.final_weights.detach().cpu().double()[0]
+    normwise(out.detach().cpu().numpy(), ref.detach().numpy(), tol=2e-5)
+    (ref * torch.tensor(up.astype(np.float64))).sum().backward()
+    normwise(tpts.grad.cpu().numpy(), p.grad.numpy(), tol=1e-4)
+
+
+def _kde_per_point(p, g, own, bw, radius):
+    """float64 Gaussian KDE over the sorted self-neighbourhood, per original point."""
+    order = torch.tensor(g.sorted_indices).long()
+    sp = p[order]
+    on = torch.tensor(own.neighbors).long()
+    u = (sp[on[:, 0]] - sp[on[:, 1]]) / (bw * radius)
+    kde = torch.prod(torch.exp(-0.5 * u * u) * (0.3989422804014327 / bw), dim=1)
+    return torch.zeros(len(p), dtype=torch.float64).index_add(0, on[:, 1], kde)   # by sorted index
+
+
+@pytest.mark.parametrize("layer", ["kp_linear", "kp_gaussian_deformable", "pointconv"])
+def test_kpconv_and_pointconv_gradient_with_respect_to_points(oracle, layer):
+    """kernel_point_conv_test.py:218-260 and point_conv_test.py:218-260 check the
+    Jacobian with respect to the point coordinates; here both clouds require a
+    gradient and the result is compared with float64 autograd of the same
+    expressions (kernel-point correlation, offsets of the deformable kernel,
+    relative densities and their MLP)."""
+    from tensorflow_graphics_point_clouds_amd import layers, pc, synthetic
+    rng = np.random.default_rng(11)
+    batch, radius, c_in, c_out, bw = 2, 0.25, 4, 6, 0.2
+    pts, bids, ctr, cb, nbh = _setup(oracle, rng, n=700, n_out=150, batch=batch, radius=radius)
+    feat = rng.standard_normal((len(pts), c_in)).astype(np.float32)
+    ids = torch.tensor(nbh.original_neigh_ids).long()
+    tpts, tctr = dev(pts).requires_grad_(True), dev(ctr).requires_grad_(True)
+    cin, cout = pc.PointCloud(tpts, dev(bids), batch), pc.PointCloud(tctr, dev(cb), batch)
+    p = torch.tensor(pts.astype(np.float64), requires_grad=True)
+    q = torch.tensor(ctr.astype(np.float64), requires_grad=True)
+    f64 = lambda t: t.detach().cpu().double()
+    tf = torch.tensor(feat.astype(np.float64))
+
+    def project(basis):
+        per_pair = tf[ids[:, 0]][:, :, None] * basis[:, None, :]
+        return torch.zeros(len(ctr), c_in, basis.shape[1], dtype=torch.float64).index_add(
+            0, ids[:, 1], per_pair).reshape(len(ctr), -1)
+
+    if layer == "pointconv":
+        conv = layers.PointConv(c_in, c_out, 3, size_hidden=8, non_linearity_type="elu", seed=3)
+        with torch.no_grad():
+            conv.pdf_biases_2.fill_(0.7)
+        out = conv(dev(feat), cin, cout, radius, bandwidth=bw)
+        g = oracle.Grid(pts, bids, batch, np.float32(radius))
+        per_sorted = _kde_per_point(p, g, oracle.Neighborhood(g, np.float32(radius)), bw, radius)
+        pdf = per_sorted[torch.tensor(nbh.neighbors[:, 0]).long()]
+        mx = torch.zeros(len(ctr), dtype=torch.float64).scatter_reduce(0, ids[:, 1], pdf, "amax",
+                                                                       include_self=False)
+        rel = (pdf / mx[ids[:, 1]]).reshape(-1, 1)
+        cur = torch.relu(rel @ f64(conv.pdf_weights_1) + f64(conv.pdf_biases_1))
+        cur = cur @ f64(conv.pdf_weights_2) + f64(conv.pdf_biases_2)
+        hid = torch.nn.functional.elu((p[ids[:, 0]] - q[ids[:, 1]]) @ f64(conv.weights) +
+                                      f64(conv.biases))
+        ref = project(hid / cur) @ f64(conv.final_weights)
+    else:
+        deform = layer.endswith("deformable")
+        kp = synthetic.spherical_kernel_points(15, rotate=False) * 0.8
+        conv = layers.KPConv(c_in, c_out, custom_kernel_points=kp, deformable=deform,
+                             kp_interpolation="gaussian" if deform else "linear", seed=3)
+        if deform:
+            with torch.no_grad():
+                conv.offset_weights.mul_(0.05)
+        sigma = 0.6
+        out = conv(dev(feat), cin, cout, radius, kernel_influence_dist=sigma * radius)
+        tkp = torch.tensor(kp.astype(np.float64) * 0.75)
+        diff = (p[ids[:, 0]] - q[ids[:, 1]]) / radius
+
+        def correlation(offsets):
+            delta = diff[:, None, :] - tkp[None] - (0 if offsets is None else offsets[ids[:, 1]])
+            dist = torch.sqrt((delta * delta).sum(2) + 1e-20)
+            if deform:
+                return torch.exp(-(dist / (sigma / 3)) ** 2)
+            return torch.relu(1 - dist / sigma)
+
+        offsets = None
+        if deform:
+            offsets = (project(correlation(None)) @ f64(conv.offset_weights)).reshape(-1, 15, 3)
+        ref = project(correlation(offsets)) @ f64(conv.weights)
+    normwise(out.detach().cpu().numpy(), ref.detach().numpy(), tol=2e-5)
+    up = rng.standard_normal(tuple(out.shape)).astype(np.float32)
+    out.backward(dev(up))
+    (ref * torch.tensor(up.astype(np.float64))).sum().backward()
+    normwise(tpts.grad.cpu().numpy(), p.grad.numpy(), tol=1e-4)
+    normwise(tctr.grad.cpu().numpy(), q.grad.numpy(), tol=1e-4)
