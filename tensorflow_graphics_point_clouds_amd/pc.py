@@ -31,6 +31,26 @@ def _as_vector(value, dims, device):
     return t.to(device).contiguous()
 
 
+class AABB:
+    """Axis-aligned bounding box per cloud (pylib/pc/PointCloud.py:23-66)."""
+
+    def __init__(self, point_cloud):
+        pts, ids = point_cloud._points.detach(), point_cloud._batch_ids.long()
+        b, d = point_cloud._batch_size, pts.shape[1]
+        index = ids[:, None].expand(-1, d)
+        self._batch_shape = point_cloud._batch_shape
+        self._aabb_min = torch.zeros((b, d), dtype=_F32, device=pts.device).scatter_reduce(
+            0, index, pts, "amin", include_self=False) - 1e-9
+        self._aabb_max = torch.zeros((b, d), dtype=_F32, device=pts.device).scatter_reduce(
+            0, index, pts, "amax", include_self=False) + 1e-9
+
+    def get_diameter(self, ord="euclidean"):
+        """Norm of the box extent per cloud, [A1, ..., An] (or [B])."""
+        extent = self._aabb_max - self._aabb_min
+        diam = torch.linalg.vector_norm(extent, ord=2 if ord == "euclidean" else ord, dim=-1)
+        return diam if self._batch_shape is None else diam.reshape(self._batch_shape)
+
+
 class PointCloud:
     """Points with a cloud id per point (pylib/pc/PointCloud.py:68-290).
 
@@ -81,6 +101,12 @@ class PointCloud:
                 batch_size = int(self._batch_ids.max().item()) + 1 if self._points.shape[0] else 0
         self._batch_size = int(batch_size)
         self._dimension = self._points.shape[1]
+
+    def get_AABB(self):
+        """The bounding boxes, computed on the first call (PointCloud.py:235-247)."""
+        if getattr(self, "_aabb", None) is None:
+            self._aabb = AABB(self)
+        return self._aabb
 
     def get_sizes(self):
         """Points per cloud, in the batch shape if one is set (PointCloud.py:184-204)."""
@@ -356,6 +382,7 @@ class Neighborhood:
         self._pdf = None
         self._pdf_per_point = None
         self._pdf_args = None
+        self._pdf_normalize = False
         # optional visiting order of the centres for the projection kernels
         self._centre_order = None
         self._transposed_pairs = None
@@ -444,12 +471,11 @@ class Neighborhood:
     def compute_pdf(self, bandwidth=0.2, mode=KDEMode.constant, normalize=False):
         """Densities of the grid's points from their self-neighbourhood
         (Neighborhood.py:257-293); the per-pair values follow on `get_pdf()`."""
-        if normalize:
-            raise NotImplementedError("normalised densities are not part of the op path")
         d = self._grid._point_cloud._dimension
         dev = self._grid._sorted_points.device
         self._pdf = None
         self._pdf_args = (bandwidth, mode)
+        self._pdf_normalize = bool(normalize)
         if mode == KDEMode.no_pdf:
             self._pdf_per_point = None
             return
@@ -479,6 +505,10 @@ class Neighborhood:
                 self._pdf = torch.empty(nb.shape[0], dtype=_F32, device=nb.device)
                 _lib.call("gather_pdf", stream(), i64(nb.shape[0]), ptr(nb, _I32),
                           ptr(per_point.detach(), _F32), ptr(self._pdf))
+            if self._pdf_normalize:       # divided by the size of the pair's neighbourhood
+                ends = self._samples_neigh_ranges.long()
+                counts = (ends - torch.cat([ends.new_zeros(1), ends[:-1]])).to(_F32)
+                self._pdf = self._pdf / counts[nb[:, 1].long()]
         return self._pdf
 
 
@@ -499,6 +529,30 @@ def sample(neighborhood, sample_mode="poisson"):
         _lib.call("gather_i32", stream(), i64(idx.shape[0]), ptr(g._sorted_indices, _I32), ptr(idx, _I32),
             ptr(original))
     return PointCloud(pts, bids, g._batch_size), original
+
+
+def poisson_disk_sampling(point_cloud, radius=None, neighborhood=None, return_ids=False):
+    """Poisson-disk sample of a point cloud (pylib/pc/sampling.py:31-78) -> PointCloud
+    (and the original indices of the kept points).  The reference passes the mode
+    of the other sampler here (:67, and :114 below); this follows the names."""
+    if radius is None and neighborhood is None:
+        raise ValueError("Missing Argument! Either radius or neighborhood must be given!")
+    if neighborhood is None:
+        radii = _as_vector(radius, point_cloud._dimension, point_cloud._points.device)
+        neighborhood = Neighborhood(Grid(point_cloud, radii), radii)
+    cloud, ids = sample(neighborhood, "poisson")
+    return (cloud, ids) if return_ids else cloud
+
+
+def cell_average_sampling(point_cloud, cell_sizes=None, grid=None):
+    """One point per occupied cell, the mean of the cell's points
+    (pylib/pc/sampling.py:81-120) -> PointCloud."""
+    if cell_sizes is None and grid is None:
+        raise ValueError("Missing Argument! Either cell_sizes or grid must be given!")
+    if grid is None:
+        grid = Grid(point_cloud, _as_vector(cell_sizes, point_cloud._dimension,
+                                            point_cloud._points.device))
+    return sample(Neighborhood(grid, grid._cell_sizes), "average")[0]
 
 
 class PointHierarchy:
@@ -527,6 +581,20 @@ class PointHierarchy:
             return [nb.transpose() for nb in self._neighborhoods] if transposed \
                 else self._neighborhoods
         return self._neighborhoods[i].transpose() if transposed else self._neighborhoods[i]
+
+    def get_points(self, batch_id=None, max_num_points=None):
+        """Per level: the points of cloud `batch_id`, or all of them padded
+        (PointHierarchy.py:100-122)."""
+        return [c.get_points(batch_id, max_num_points) for c in self._point_clouds]
+
+    def get_sizes(self):
+        """Per level: points per cloud (PointHierarchy.py:124-138)."""
+        return [c.get_sizes() for c in self._point_clouds]
+
+    def set_batch_shape(self, batch_shape):
+        """PointHierarchy.py:140-157."""
+        for c in self._point_clouds:
+            c.set_batch_shape(batch_shape)
 
     def __getitem__(self, index):
         return self._point_clouds[index]

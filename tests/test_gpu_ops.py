@@ -481,3 +481,49 @@ def test_gathered_feature_gradient(ops, oracle, c, k):
     # points that are nobody's neighbour get an exact zero row
     unused = np.setdiff1d(np.arange(n), ids[:, 0])
     assert len(unused) > 0 and float(df1[dev(unused).long()].abs().sum()) == 0.0
+
+
+def test_sampling_wrappers_hierarchy_accessors_and_normalised_pdf(ops, oracle):
+    """poisson_disk_sampling / cell_average_sampling (sampling.py:31-120) against the
+    oracle's sampler, the per-level accessors of the hierarchy, and densities
+    divided by the size of their neighbourhood (Neighborhood.py:288-293)."""
+    from tensorflow_graphics_point_clouds_amd import pc
+    rng = np.random.default_rng(8)
+    pts, bids = _cloud(rng, 3, 4000, 3)
+    cloud = pc.PointCloud(dev(pts), dev(bids), 3)
+    r = np.float32(0.07)
+    g = oracle.Grid(pts, bids, 3, r)
+    nbh = oracle.Neighborhood(g, r)
+    for mode, fn in ((0, lambda: pc.poisson_disk_sampling(cloud, float(r), return_ids=True)),
+                     (1, lambda: (pc.cell_average_sampling(cloud, float(r)), None))):
+        spts, sbids, sidx = oracle.sampling(g.sorted_points, g.sorted_batch_ids, g.sorted_keys,
+                                            g.num_cells, nbh.neighbors, nbh.ranges, mode)
+        got, ids = fn()
+        assert np.array_equal(got._points.cpu().numpy(), spts)
+        assert np.array_equal(got._batch_ids.cpu().numpy(), sbids)
+        if mode == 0:
+            assert np.array_equal(ids.cpu().numpy(), g.sorted_indices[sidx])
+            assert np.array_equal(pts[ids.cpu().numpy()], spts)
+    with pytest.raises(ValueError):
+        pc.poisson_disk_sampling(cloud)
+    with pytest.raises(ValueError):
+        pc.cell_average_sampling(cloud)
+
+    hier = pc.PointHierarchy(cloud, [0.1, 0.2], "cell average")
+    sizes = hier.get_sizes()
+    assert [int(s.sum()) for s in sizes] == [c._points.shape[0] for c in hier._point_clouds]
+    padded = hier.get_points()
+    assert [tuple(p.shape[:1]) for p in padded] == [(3,)] * 3
+    assert [p.shape[1] for p in padded] == [int(s.max()) for s in sizes]
+    assert hier.get_points(1)[2].shape[0] == int(sizes[2][1])
+    hier.set_batch_shape([3, 1])
+    assert all(tuple(s.shape) == (3, 1) for s in hier.get_sizes())
+
+    ctr, cb = _cloud(rng, 3, 500, 3)
+    gn = pc.Neighborhood(pc.Grid(cloud, float(r) * 2), float(r) * 2, pc.PointCloud(dev(ctr), dev(cb), 3))
+    plain = gn.get_pdf(bandwidth=0.2).clone()
+    gn.compute_pdf(bandwidth=0.2, normalize=True)
+    ends = gn._samples_neigh_ranges.long()
+    counts = ends - torch.cat([ends.new_zeros(1), ends[:-1]])
+    expect = plain / counts[gn._neighbors[:, 1].long()].float()
+    assert torch.allclose(gn.get_pdf(), expect, rtol=1e-6)

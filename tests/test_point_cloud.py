@@ -84,3 +84,24 @@ def test_flatten_features_and_format_output_round_trip():
     assert cloud.flatten_features(feats) is feats
     with pytest.raises(ValueError):
         cloud.flatten_features(feats[:4])
+
+
+def test_bounding_boxes_and_diameter():
+    """aabb_test.py:30-78: per-cloud minima / maxima and the norms of the extent."""
+    rng = np.random.default_rng(3)
+    pts = rng.random((500, 3)).astype(np.float32) * np.array([2.0, 1.0, 0.5], np.float32)
+    bids = rng.integers(0, 4, 500).astype(np.int32)
+    bids[:4] = np.arange(4)
+    cloud = pc.PointCloud(torch.as_tensor(pts), torch.as_tensor(bids), 4)
+    box = cloud.get_AABB()
+    assert cloud.get_AABB() is box
+    for b in range(4):
+        sel = pts[bids == b]
+        assert np.allclose(box._aabb_min[b].numpy(), sel.min(0) - 1e-9)
+        assert np.allclose(box._aabb_max[b].numpy(), sel.max(0) + 1e-9)
+    extent = np.stack([pts[bids == b].max(0) - pts[bids == b].min(0) for b in range(4)])
+    assert np.allclose(box.get_diameter().numpy(), np.linalg.norm(extent, axis=1), rtol=1e-6)
+    assert np.allclose(box.get_diameter(ord=1).numpy(), extent.sum(1), rtol=1e-6)
+    assert np.allclose(box.get_diameter(ord=np.inf).numpy(), extent.max(1), rtol=1e-6)
+    cloud.set_batch_shape([2, 2])
+    assert pc.AABB(cloud).get_diameter().shape == (2, 2)
