@@ -527,3 +527,33 @@ def test_sampling_wrappers_hierarchy_accessors_and_normalised_pdf(ops, oracle):
     counts = ends - torch.cat([ends.new_zeros(1), ends[:-1]])
     expect = plain / counts[gn._neighbors[:, 1].long()].float()
     assert torch.allclose(gn.get_pdf(), expect, rtol=1e-6)
+
+
+def test_object_level_adapters_match_the_callers(ops):
+    """custom_ops (the wrapper layer of custom_ops_wrapper.py:20-198) gives what the
+    Grid / Neighborhood callers compute through the positional ops."""
+    from tensorflow_graphics_point_clouds_amd import custom_ops, pc
+    rng = np.random.default_rng(12)
+    pts, bids = _cloud(rng, 3, 5000, 3)
+    ctr, cb = _cloud(rng, 3, 700, 3)
+    cloud, centres = pc.PointCloud(dev(pts), dev(bids), 3), pc.PointCloud(dev(ctr), dev(cb), 3)
+    radii = dev(np.full(3, 0.08, np.float32))
+    grid = pc.Grid(cloud, radii)
+    assert torch.equal(custom_ops.compute_keys(cloud, grid._num_cells, grid._cell_sizes),
+                       grid._cur_keys)
+    assert torch.equal(custom_ops.build_grid_ds(grid._sorted_keys, grid._num_cells, 3),
+                       grid.get_DS())
+    nbh = pc.Neighborhood(grid, radii, centres)
+    ranges, nbrs = custom_ops.find_neighbors(grid, centres, radii)
+    assert torch.equal(ranges, nbh._samples_neigh_ranges) and torch.equal(nbrs, nbh._neighbors)
+    own = pc.Neighborhood(grid, radii)
+    for mode, name in ((0, "poisson"), (1, "average")):
+        spts, sbids, _ = custom_ops.sampling(own, mode)
+        expect = pc.sample(own, name)[0]
+        assert torch.equal(spts, expect._points) and torch.equal(sbids, expect._batch_ids)
+    bw = dev(np.full(3, 0.2, np.float32))
+    assert torch.equal(custom_ops.compute_pdf(own, bw, 0), own.point_pdf(bandwidth=0.2))
+    basis = torch.rand((nbrs.shape[0], 8), device="cuda")
+    feat = torch.randn((5000, 8), device="cuda")
+    assert torch.equal(custom_ops.basis_proj(basis, feat, nbh),
+                       ops.basis_proj(basis, feat, nbh._original_neigh_ids, ranges))
