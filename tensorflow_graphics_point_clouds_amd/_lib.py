@@ -67,8 +67,12 @@ def check(rc):
 
 
 def stream():
+    """torch's current stream on the current device as a raw hipStream_t."""
     import torch
-    return vptr(torch.cuda.current_stream().cuda_stream)
+    try:        # the raw accessors skip the Stream object and its device bookkeeping
+        return vptr(torch._C._cuda_getCurrentRawStream(torch._C._cuda_getDevice()))
+    except AttributeError:
+        return vptr(torch.cuda.current_stream().cuda_stream)
 
 
 def ptr(t, dtype=None):
