@@ -7,7 +7,8 @@
 //           of sorted points that lies in the offset cell row
 //           (find_ranges_grid_ds_kernels.cu.cc:48-235);
 //   count   16 lanes per centre stride over the slices and test
-//           |(s - p) * inv_radii| < 1 (count_neighbors_kernels.cu.cc:83-86);
+//           |(s - p) * inv_radii| < 1 (count_neighbors_kernels.cu.cc:83-86; as the
+//           squared length against 1, which decides identically);
 //   fill    same traversal; the slot of a hit is the centre's start offset plus
 //           a ballot prefix inside the 16-lane group, so the pairs of a centre
 //           come out in ascending sorted-point index without atomics or a sort.
@@ -109,7 +110,12 @@ __device__ __forceinline__ bool within_radius(const float *s, const float *__res
     const float sq = sc * sc;
     acc = acc + sq;
   }
-  return sqrtf(acc) < 1.0f;
+  // The reference tests sqrtf(acc) < 1 (count_neighbors_kernels.cu.cc:83-86).  The
+  // correctly rounded root is monotonic, sqrtf(1) = 1 and the root of the largest
+  // float below 1 is again that float, so acc < 1 decides the same for every
+  // float, infinities and NaN included, without the twenty instructions of an
+  // IEEE square root per candidate.
+  return acc < 1.0f;
 }
 
 // kFill == false: counts[c] = number of hits (clamped to max_neighs when > 0).
@@ -136,18 +142,24 @@ __global__ void __launch_bounds__(kNbrThreads) nbr_visit_kernel(
   int found = 0;                                   // kFill: slots used so far
   int64_t start = 0;
   if (kFill) start = c > 0 ? ends[c - 1] : 0;
-  for (int r = 0; r < R; ++r) {
-    const int2 span = ranges[c * R + r];
-    for (int j0 = span.x; j0 < span.y; j0 += kGroup) {
-      const int j = j0 + sub;
-      const bool hit = j < span.y && within_radius<D>(s, pts, j, ir);
-      if (kFill) {
-        const uint64_t hits = __ballot(hit) & group_mask;
-        const int slot = found + __popcll(hits & below_mask);
-        if (hit && slot < limit) nbrs[start + slot] = make_int2(j, (int)c);
-        found += __popcll(hits);
-      } else {
-        found += hit ? 1 : 0;
+  // the slices of the centre, 16 at a time: lane `sub` fetches one, the group then
+  // takes them in turn (one round trip to memory instead of one per slice)
+  for (int r0 = 0; r0 < R; r0 += kGroup) {
+    const int2 mine = r0 + sub < R ? ranges[c * R + r0 + sub] : make_int2(0, 0);
+    const int lim = R - r0 < kGroup ? R - r0 : kGroup;
+    for (int r = 0; r < lim; ++r) {
+      const int2 span = make_int2(__shfl(mine.x, r, kGroup), __shfl(mine.y, r, kGroup));
+      for (int j0 = span.x; j0 < span.y; j0 += kGroup) {
+        const int j = j0 + sub;
+        const bool hit = j < span.y && within_radius<D>(s, pts, j, ir);
+        if (kFill) {
+          const uint64_t hits = __ballot(hit) & group_mask;
+          const int slot = found + __popcll(hits & below_mask);
+          if (hit && slot < limit) nbrs[start + slot] = make_int2(j, (int)c);
+          found += __popcll(hits);
+        } else {
+          found += hit ? 1 : 0;
+        }
       }
     }
   }
