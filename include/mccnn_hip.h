@@ -401,7 +401,9 @@ int mccnn_mc_basis_grads(mccnn_stream_t stream, int64_t num_neighbors,
  * and biases from the upstream [N_out, C, K] gradient).  Same results as the
  * separate entry points up to fp32 summation order; the [M, K] basis and its
  * gradient are never written.  mccnn_mc_conv_supported() tells whether a shape
- * is covered (D in {2,3}, K = 16, C in {16,32,64,128}); other shapes return
+ * is covered (D in {2,3}, K = 16, C in {16,32,64,128}; see the two queries below
+ * for the wider shapes of the forward and of the weights-only backward); other
+ * shapes return
  * MCCNN_INVALID_ARGUMENT and must use the separate entry points.  out_rows
  * (optional permutation of 0..N_out-1) makes the forward write the projection of
  * centre i to row out_rows[i] of out, so that a caller working on re-ordered
@@ -415,8 +417,11 @@ int mccnn_mc_basis_grads(mccnn_stream_t stream, int64_t num_neighbors,
  * counterpart among the reference's ops, which materialise the basis in
  * TensorFlow. */
 int mccnn_mc_conv_supported(int num_dims, int num_features, int num_basis);
-/* ... and for the forward alone (also mccnn_kp_conv_project): any multiple of 16
- * channels up to 512. */
+/* ... for the backward without the feature gradient (feature_grads_out NULL):
+ * also K = 32 and K = 64 ... */
+int mccnn_mc_conv_weight_grads_supported(int num_dims, int num_features, int num_basis);
+/* ... and for the forward alone (also mccnn_kp_conv_project, K = 16 there): any
+ * multiple of 16 channels up to 512, K in {16, 32, 64}. */
 int mccnn_mc_conv_project_supported(int num_dims, int num_features, int num_basis);
 int mccnn_mc_conv_project(mccnn_stream_t stream, int num_dims, int64_t num_pts,
                           const float *points_in, int num_features,

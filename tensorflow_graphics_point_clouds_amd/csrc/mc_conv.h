@@ -49,18 +49,21 @@ struct PairStage {
     default: { constexpr int ACT = MCCNN_ACT_ELU; __VA_ARGS__; } break;                          \
   }
 
-// Per-lane basis functors: the value of basis column `col` (= lane & 15) for a
-// staged pair g = (delta * inv_radii, weight), weight = 1/pdf or 1 for a live
-// pair and 0 for a padding slot.
-template <int D, int kAct>
+// Per-lane basis functors: the value of basis column `col + 16 kt` (col = lane & 15)
+// for a staged pair g = (delta * inv_radii, weight), weight = 1/pdf or 1 for a
+// live pair and 0 for a padding slot.
+template <int D, int kAct, int KT = 1>
 struct MlpBasis {                  // act(delta . W[:, col] + b[col]) / pdf   (MCConv.py:163-171)
-  float w[3], b;
+  float w[KT][3], b[KT];           // columns col, col + 16, ... of the flattened kernel matrix
   __device__ __forceinline__ MlpBasis(const McParams<D> &p) {
-    w[0] = w[1] = w[2] = 0.0f;
-    load_weight_column<D>(p, lane_id() & 15, w, &b);
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt) {
+      w[kt][0] = w[kt][1] = w[kt][2] = 0.0f;
+      load_weight_column<D>(p, 16 * kt + (lane_id() & 15), w[kt], &b[kt]);
+    }
   }
-  __device__ __forceinline__ float operator()(const float4 &g) const {
-    const float z = b + g.x * w[0] + g.y * w[1] + g.z * w[2];
+  __device__ __forceinline__ float operator()(const float4 &g, int kt = 0) const {
+    const float z = b[kt] + g.x * w[kt][0] + g.y * w[kt][1] + g.z * w[kt][2];
     return act_fwd(kAct, z) * g.w;
   }
 };
@@ -77,7 +80,7 @@ struct KpBasis {                   // kernel-point correlation (KPConv.py:29-57,
 #pragma unroll
     for (int d = 0; d < D; ++d) k[d] = live ? kernel_points[col * D + d] : 0.0f;
   }
-  __device__ __forceinline__ float operator()(const float4 &g) const {
+  __device__ __forceinline__ float operator()(const float4 &g, int = 0) const {
     const float dx = g.x - k[0], dy = g.y - k[1], dz = g.z - k[2];
     const float dist = sqrtf(dx * dx + dy * dy + dz * dz);
     float wgt;

@@ -6,8 +6,9 @@
 // [M, K] basis tensor and its gradient never reach HBM.  Forward produces the
 // same [N_out, C, K] projection as mc_basis + basis_proj; backward produces the
 // feature gradient and the kernel-MLP weight / bias gradients from the upstream
-// [N_out, C, K] gradient.  K = 16 (v_mfma_f32_16x16x4f32), D = 2 or 3,
-// C in {16, 32, 64, 128}; other shapes use the separate kernels.
+// [N_out, C, K] gradient.  K in {16, 32, 64} (tiles of v_mfma_f32_16x16x4f32),
+// D = 2 or 3, C a multiple of 16 (forward) or in {16, 32, 64, 128} (kernel-MLP
+// gradients); other shapes use the separate kernels.
 #include "common.h"
 #include "fill.h"
 #include "mfma.h"
@@ -34,13 +35,13 @@ constexpr int kProjRun = 8;        // consecutive centres per wavefront
 // other centres' pairs weighted 0, the finished accumulators are stored and
 // cleared, and the walk goes on.  Centres without pairs get their zeros the
 // same way.
-template <int kCPL, int D, class Basis>
+template <int kCPL, int D, int KT, class Basis>
 __device__ __forceinline__ void project_run_body(
     int64_t n_out, int C, int chunks, const float *__restrict__ feat,
     const int2 *__restrict__ nbrs, const int *__restrict__ ranges, const McParams<D> &p,
     const Basis &basis, const int *__restrict__ out_rows, float *__restrict__ out,
     PairStage *stage) {
-  constexpr int K = kFusedK;
+  constexpr int K = kFusedK * KT;          // basis columns, KT tiles of 16
   constexpr int kCW = 16 * kCPL;
   const int lane = lane_id();
   const int64_t wid = wave_slot();
@@ -96,18 +97,23 @@ __device__ __forceinline__ void project_run_body(
     return q;
   };
 
-  v4f acc[kCPL];
+  v4f acc[kCPL][KT];
 #pragma unroll
-  for (int j = 0; j < kCPL; ++j) acc[j] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+  for (int j = 0; j < kCPL; ++j)
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt) acc[j][kt] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
   int cur = 0, cur_start = begin, cur_end = ends[0];
   auto finish_centre = [&]() {          // store and clear the accumulators, move to the next centre
     const int64_t row = __builtin_amdgcn_readlane(my_row, cur);
     float *o = out_base + row * (int64_t)C * K;
 #pragma unroll
-    for (int j = 0; j < kCPL; ++j) {
-      __builtin_nontemporal_store(acc[j], reinterpret_cast<v4f *>(o + (j * 16 + col) * K));
-      acc[j] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
-    }
+    for (int j = 0; j < kCPL; ++j)
+#pragma unroll
+      for (int kt = 0; kt < KT; ++kt) {
+        __builtin_nontemporal_store(acc[j][kt],
+                                    reinterpret_cast<v4f *>(o + (j * 16 + col) * K + 16 * kt));
+        acc[j][kt] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+      }
     ++cur;
     cur_start = cur_end;
     cur_end = __builtin_amdgcn_readlane(my_end, cur < nc ? cur : nc - 1);
@@ -134,7 +140,7 @@ __device__ __forceinline__ void project_run_body(
     const int steps = (cnt + 3) >> 2;
     for (int t = 0; t < steps; t += kFusedUnroll) {
       FVec<kCPL> f[kFusedUnroll];
-      float w[kFusedUnroll];
+      float w[kFusedUnroll][KT];
 #pragma unroll
       for (int u = 0; u < kFusedUnroll; ++u) {
         const int n = 4 * (t + u) + quarter;
@@ -143,7 +149,8 @@ __device__ __forceinline__ void project_run_body(
 #pragma unroll
         for (int j = 0; j < kCPL; ++j)
           f[u].v[j] = *reinterpret_cast<const float *>(feat_base + rn + lane_off + j * 64);
-        w[u] = basis(gn);
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt) w[u][kt] = basis(gn, kt);
       }
 #pragma unroll
       for (int u = 0; u < kFusedUnroll; ++u) {
@@ -151,18 +158,26 @@ __device__ __forceinline__ void project_run_body(
         const int mine = first + quarter;
         while (cur < nc && cur_end <= first + 4) {    // a centre ends inside this step
           if (cur_end > first && cur_end > cur_start) {
-            const float wm = (mine >= cur_start && mine < cur_end) ? w[u] : 0.0f;
+            const bool in = mine >= cur_start && mine < cur_end;
 #pragma unroll
-            for (int j = 0; j < kCPL; ++j)
-              acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(wm, f[u].v[j], acc[j], 0, 0, 0);
+            for (int kt = 0; kt < KT; ++kt) {
+              const float wm = in ? w[u][kt] : 0.0f;
+#pragma unroll
+              for (int j = 0; j < kCPL; ++j)
+                acc[j][kt] = __builtin_amdgcn_mfma_f32_16x16x4f32(wm, f[u].v[j], acc[j][kt], 0, 0, 0);
+            }
           }
           finish_centre();
         }
         if (cur < nc && cur_start < first + 4) {      // the rest of the step belongs to a centre that goes on
-          const float wm = mine >= cur_start ? w[u] : 0.0f;
+          const bool in = mine >= cur_start;
 #pragma unroll
-          for (int j = 0; j < kCPL; ++j)
-            acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(wm, f[u].v[j], acc[j], 0, 0, 0);
+          for (int kt = 0; kt < KT; ++kt) {
+            const float wm = in ? w[u][kt] : 0.0f;
+#pragma unroll
+            for (int j = 0; j < kCPL; ++j)
+              acc[j][kt] = __builtin_amdgcn_mfma_f32_16x16x4f32(wm, f[u].v[j], acc[j][kt], 0, 0, 0);
+          }
         }
       }
     }
@@ -170,15 +185,15 @@ __device__ __forceinline__ void project_run_body(
   while (cur < nc) finish_centre();     // a run without pairs, or trailing empty centres
 }
 
-template <int kCPL, int D, int kAct>
+template <int kCPL, int D, int kAct, int KT>
 __global__ void __launch_bounds__(256) mc_conv_project16_kernel(
     int64_t n_out, int C, int chunks, const float *__restrict__ feat,
     const int2 *__restrict__ nbrs, const int *__restrict__ ranges, McParams<D> p,
     const int *__restrict__ out_rows, float *__restrict__ out) {
   __shared__ PairStage stages[kWavesPerBlock];
-  const MlpBasis<D, kAct> basis(p);
-  project_run_body<kCPL, D>(n_out, C, chunks, feat, nbrs, ranges, p, basis, out_rows, out,
-                            &stages[threadIdx.x / kWave]);
+  const MlpBasis<D, kAct, KT> basis(p);
+  project_run_body<kCPL, D, KT>(n_out, C, chunks, feat, nbrs, ranges, p, basis, out_rows, out,
+                                &stages[threadIdx.x / kWave]);
 }
 
 // The same projection with the kernel-point correlation of KPConv as basis
@@ -191,8 +206,8 @@ __global__ void __launch_bounds__(256) kp_conv_project16_kernel(
     const int *__restrict__ out_rows, float *__restrict__ out) {
   __shared__ PairStage stages[kWavesPerBlock];
   const KpBasis<D, kKind> basis(kernel_points, num_kp, sigma);
-  project_run_body<kCPL, D>(n_out, C, chunks, feat, nbrs, ranges, p, basis, out_rows, out,
-                            &stages[threadIdx.x / kWave]);
+  project_run_body<kCPL, D, 1>(n_out, C, chunks, feat, nbrs, ranges, p, basis, out_rows, out,
+                               &stages[threadIdx.x / kWave]);
 }
 
 // Persistent wavefronts stride over the centres.  Per tile of 16 pairs:
@@ -361,21 +376,23 @@ static int64_t grad_blocks(int64_t num_samples) {
   return b < 1 ? 1 : b;
 }
 
-template <int C, int D, int kAct>
+template <int C, int D, int kAct, int KT>
 __global__ void __launch_bounds__(256) mc_conv_weight_grads16_kernel(
     int64_t n_out, const float *__restrict__ feat, const int2 *__restrict__ nbrs,
     const int *__restrict__ ranges, McParams<D> p, const float *__restrict__ in_grad,
     float *__restrict__ partials) {
-  constexpr int K = kFusedK;
+  constexpr int K = kFusedK;               // a block works on basis columns k0 .. k0 + 15
+  constexpr int num_basis = kFusedK * KT;  // of the KT * 16 the layer has
   constexpr int kQuarterC = C / 4;
   __shared__ float red[kWavesPerBlock][(D + 1) * K];
   __shared__ float4 wlds[K];               // column j: weights (z = 0 for D = 2), bias in w
   __shared__ PairStage stages[kWavesPerBlock];
   const int lane = lane_id(), wave = threadIdx.x / kWave;
   const int quarter = lane >> 4, col = lane & 15;
+  const int k0 = blockIdx.y * K;
   if (threadIdx.x < K) {
     float w[3] = {0.0f, 0.0f, 0.0f}, bias;
-    load_weight_column<D>(p, threadIdx.x, w, &bias);
+    load_weight_column<D>(p, k0 + threadIdx.x, w, &bias);
     wlds[threadIdx.x] = make_float4(w[0], w[1], w[2], bias);
   }
   __syncthreads();
@@ -399,10 +416,10 @@ __global__ void __launch_bounds__(256) mc_conv_weight_grads16_kernel(
   for (int64_t centre = first; centre < last; ++centre) {
     const int a = centre > 0 ? ranges[centre - 1] : 0, b = ranges[centre];
     if (b <= a) continue;
-    const float *gi = in_grad + centre * (int64_t)C * K;
+    const float *gi = in_grad + centre * (int64_t)C * num_basis + k0;
     float gk[kQuarterC];
 #pragma unroll
-    for (int s = 0; s < kQuarterC; ++s) gk[s] = gi[(quarter * kQuarterC + s) * K + col];
+    for (int s = 0; s < kQuarterC; ++s) gk[s] = gi[(quarter * kQuarterC + s) * num_basis + col];
     float ctr[D];
 #pragma unroll
     for (int d = 0; d < D; ++d) ctr[d] = p.pout[centre * D + d];
@@ -476,7 +493,8 @@ __global__ void __launch_bounds__(256) mc_conv_weight_grads16_kernel(
     float s = 0.0f;
 #pragma unroll
     for (int w = 0; w < kWavesPerBlock; ++w) s += red[w][threadIdx.x];
-    partials[(int64_t)blockIdx.x * (D + 1) * K + threadIdx.x] = s;
+    const int q = threadIdx.x / K, j = threadIdx.x - q * K;
+    partials[(int64_t)blockIdx.x * (D + 1) * num_basis + q * num_basis + k0 + j] = s;
   }
 }
 
@@ -508,11 +526,23 @@ __global__ void __launch_bounds__(256) mc_conv_reduce_kernel(int64_t blocks, int
 template <int C, int D, int ACT>
 static int launch_fused_backward(hipStream_t s, int64_t num_samples, const float *features,
                                  const int2 *nb, const int *ranges, const McParams<D> &prm,
-                                 const float *in_grads, float *feature_grads_out,
+                                 int num_basis, const float *in_grads, float *feature_grads_out,
                                  float *pair_rows, float *workspace, bool want_dfeat) {
-  hipLaunchKernelGGL((mc_conv_weight_grads16_kernel<C, D, ACT>),
-                     dim3((unsigned)grad_blocks(num_samples)), dim3(256), 0, s, num_samples,
-                     features, nb, ranges, prm, in_grads, workspace);
+  const dim3 grid((unsigned)grad_blocks(num_samples), (unsigned)(num_basis / kFusedK));
+  switch (num_basis / kFusedK) {
+    case 1:
+      hipLaunchKernelGGL((mc_conv_weight_grads16_kernel<C, D, ACT, 1>), grid, dim3(256), 0, s,
+                         num_samples, features, nb, ranges, prm, in_grads, workspace);
+      break;
+    case 2:
+      hipLaunchKernelGGL((mc_conv_weight_grads16_kernel<C, D, ACT, 2>), grid, dim3(256), 0, s,
+                         num_samples, features, nb, ranges, prm, in_grads, workspace);
+      break;
+    default:
+      hipLaunchKernelGGL((mc_conv_weight_grads16_kernel<C, D, ACT, 4>), grid, dim3(256), 0, s,
+                         num_samples, features, nb, ranges, prm, in_grads, workspace);
+      break;
+  }
   if (want_dfeat)        // the feature half keeps no running sums: one wavefront per centre
     hipLaunchKernelGGL((mc_conv_project_grads16_kernel<C, D, ACT, false, true>),
                        dim3(wave_grid(num_samples)), dim3(256), 0, s, num_samples, features, nb,
@@ -520,24 +550,29 @@ static int launch_fused_backward(hipStream_t s, int64_t num_samples, const float
   return MCCNN_OK;
 }
 
-// Shapes of the weight-gradient / feature-gradient kernels (C is a template parameter).
-static bool fused_supported(int D, int C, int K) {
-  return (D == 2 || D == 3) && K == kFusedK && (C == 16 || C == 32 || C == 64 || C == 128);
+static bool fused_basis_count(int K) { return K == 16 || K == 32 || K == 64; }
+
+// Shapes of the weight-gradient kernel (C is a template parameter); the
+// feature-gradient half that goes with it exists for 16 basis columns only.
+static bool fused_supported(int D, int C, int K, bool weights_only) {
+  return (D == 2 || D == 3) && (weights_only ? fused_basis_count(K) : K == kFusedK) &&
+         (C == 16 || C == 32 || C == 64 || C == 128);
 }
 
 // Shapes of the projection kernels: any multiple of 16 channels, in chunks of up
-// to 128 channels per wavefront.
+// to 128 channels per wavefront, 16 / 32 / 64 basis columns.
 static bool project_supported(int D, int C, int K) {
-  return (D == 2 || D == 3) && K == kFusedK && C >= 16 && C <= 512 && C % 16 == 0;
+  return (D == 2 || D == 3) && fused_basis_count(K) && C >= 16 && C <= 512 && C % 16 == 0;
 }
 
-static int check_fused_args(const char *op, bool project_only, int num_dims, int num_features,
-                            int num_basis, int num_mlps, int activation, int64_t num_neighbors,
-                            int64_t num_samples) {
+static int check_fused_args(const char *op, bool project_only, bool weights_only, int num_dims,
+                            int num_features, int num_basis, int num_mlps, int activation,
+                            int64_t num_neighbors, int64_t num_samples) {
   MCCNN_REQUIRE(project_only ? project_supported(num_dims, num_features, num_basis)
-                             : fused_supported(num_dims, num_features, num_basis),
-                "%s supports D in {2,3}, K = 16 and C in %s (got D=%d, K=%d, C=%d); "
+                             : fused_supported(num_dims, num_features, num_basis, weights_only),
+                "%s supports D in {2,3}, K in %s and C in %s (got D=%d, K=%d, C=%d); "
                 "use mc_basis + basis_proj for other shapes", op,
+                project_only || weights_only ? "{16,32,64}" : "{16}",
                 project_only ? "{16, 32, ..., 512}" : "{16,32,64,128}", num_dims, num_basis,
                 num_features);
   MCCNN_REQUIRE(num_mlps > 0 && num_basis % num_mlps == 0,
@@ -555,7 +590,12 @@ static int check_fused_args(const char *op, bool project_only, int num_dims, int
 using namespace mccnn;
 
 extern "C" int mccnn_mc_conv_supported(int num_dims, int num_features, int num_basis) {
-  return fused_supported(num_dims, num_features, num_basis) ? 1 : 0;
+  return fused_supported(num_dims, num_features, num_basis, false) ? 1 : 0;
+}
+
+extern "C" int mccnn_mc_conv_weight_grads_supported(int num_dims, int num_features,
+                                                    int num_basis) {
+  return fused_supported(num_dims, num_features, num_basis, true) ? 1 : 0;
 }
 
 extern "C" int mccnn_mc_conv_project_supported(int num_dims, int num_features, int num_basis) {
@@ -570,8 +610,8 @@ extern "C" int mccnn_mc_conv_project(mccnn_stream_t stream, int num_dims, int64_
                                      const float *inv_radii, int num_basis, int num_mlps,
                                      int activation, const float *weights, const float *biases,
                                      const float *pdf, const int32_t *out_rows, float *out) {
-  int rc = check_fused_args("mc_conv_project", true, num_dims, num_features, num_basis, num_mlps,
-                            activation, num_neighbors, num_samples);
+  int rc = check_fused_args("mc_conv_project", true, false, num_dims, num_features, num_basis,
+                            num_mlps, activation, num_neighbors, num_samples);
   if (rc != MCCNN_OK) return rc;
   MCCNN_REQUIRE(num_pts >= 0 && num_pts * num_features < ((int64_t)1 << 30),
                 "mc_conv_project expects a feature table of fewer than 2^30 elements");
@@ -580,28 +620,35 @@ extern "C" int mccnn_mc_conv_project(mccnn_stream_t stream, int num_dims, int64_
                     (num_neighbors == 0 || (points_in && features && neighbors && pdf)),
                 "mc_conv_project received a null tensor");
   hipStream_t s = as_stream(stream);
+  // channels per lane and pass: at most 8 accumulator tiles of 16 x 16 per wavefront
+  const int kt = num_basis / kFusedK;
   int cpl = 1;
-  for (int c = 8; c >= 1; c >>= 1)
+  for (int c = 8 / kt; c >= 1; c >>= 1)
     if (num_features % (16 * c) == 0) { cpl = c; break; }
   const int chunks = num_features / (16 * cpl);
   const dim3 grid(wave_grid((num_samples + kProjRun - 1) / kProjRun * chunks)), block(256);
   const int2 *nb = (const int2 *)neighbors;
-#define MCCNN_FUSED_FWD(CPL_, D_)                                                              \
+#define MCCNN_FUSED_FWD(CPL_, D_, KT_)                                                         \
   {                                                                                            \
     McParams<D_> prm{points_in, points_out, inv_radii, weights, biases, pdf,                   \
                      num_basis / num_mlps, activation};                                        \
     MCCNN_ACT_SWITCH(activation,                                                               \
-                     hipLaunchKernelGGL((mc_conv_project16_kernel<CPL_, D_, ACT>), grid, block, \
-                                        0, s, num_samples, num_features, chunks, features, nb, \
-                                        ranges, prm, out_rows, out));                          \
+                     hipLaunchKernelGGL((mc_conv_project16_kernel<CPL_, D_, ACT, KT_>), grid,  \
+                                        block, 0, s, num_samples, num_features, chunks,        \
+                                        features, nb, ranges, prm, out_rows, out));            \
   }
-#define MCCNN_FUSED_FWD_D(CPL_) \
-  if (num_dims == 3) MCCNN_FUSED_FWD(CPL_, 3) else MCCNN_FUSED_FWD(CPL_, 2)
-  switch (cpl) {
-    case 8: MCCNN_FUSED_FWD_D(8); break;
-    case 4: MCCNN_FUSED_FWD_D(4); break;
-    case 2: MCCNN_FUSED_FWD_D(2); break;
-    default: MCCNN_FUSED_FWD_D(1); break;
+#define MCCNN_FUSED_FWD_D(CPL_, KT_) \
+  if (num_dims == 3) MCCNN_FUSED_FWD(CPL_, 3, KT_) else MCCNN_FUSED_FWD(CPL_, 2, KT_)
+  switch (kt * 16 + cpl) {
+    case 16 + 8: MCCNN_FUSED_FWD_D(8, 1); break;
+    case 16 + 4: MCCNN_FUSED_FWD_D(4, 1); break;
+    case 16 + 2: MCCNN_FUSED_FWD_D(2, 1); break;
+    case 16 + 1: MCCNN_FUSED_FWD_D(1, 1); break;
+    case 32 + 4: MCCNN_FUSED_FWD_D(4, 2); break;
+    case 32 + 2: MCCNN_FUSED_FWD_D(2, 2); break;
+    case 32 + 1: MCCNN_FUSED_FWD_D(1, 2); break;
+    case 64 + 2: MCCNN_FUSED_FWD_D(2, 4); break;
+    default: MCCNN_FUSED_FWD_D(1, 4); break;
   }
 #undef MCCNN_FUSED_FWD_D
 #undef MCCNN_FUSED_FWD
@@ -629,8 +676,9 @@ extern "C" int mccnn_mc_conv_project_grads(
   MCCNN_REQUIRE(!gathered || (point_ranges && pair_order),
                 "mc_conv_project_grads needs the transposed pair lists with a pair-row "
                 "workspace");
-  int rc = check_fused_args("mc_conv_project_grads", false, num_dims, num_features, num_basis, num_mlps,
-                            activation, num_neighbors, num_samples);
+  int rc = check_fused_args("mc_conv_project_grads", false, feature_grads_out == nullptr,
+                            num_dims, num_features, num_basis, num_mlps, activation,
+                            num_neighbors, num_samples);
   if (rc != MCCNN_OK) return rc;
   MCCNN_REQUIRE(num_pts >= 0 && num_pts * num_features < ((int64_t)1 << 30),
                 "mc_conv_project_grads expects a feature table of fewer than 2^30 elements");
@@ -660,7 +708,7 @@ extern "C" int mccnn_mc_conv_project_grads(
                      num_basis / num_mlps, activation};                                        \
     MCCNN_ACT_SWITCH(activation,                                                               \
                      rc = (launch_fused_backward<C_, D_, ACT>(                                 \
-                         s, num_samples, features, nb, ranges, prm, in_grads,                  \
+                         s, num_samples, features, nb, ranges, prm, num_basis, in_grads,       \
                          feature_grads_out, pair_rows, (float *)workspace, want_dfeat)));      \
   }
 #define MCCNN_FUSED_BWD_D(C_) \

@@ -377,7 +377,7 @@ class MCConv(torch.nn.Module):
         result is cut back.  None if the shape is out of reach."""
         d, c, f, l, h = (self._num_dims, self._num_features_in, self._num_features_out,
                          self._num_mlps, self._hidden)
-        if k != 16 or d not in (2, 3):
+        if k not in (16, 32, 64) or d not in (2, 3):
             return None
         pad = _layer_padding(c, f, l)
         if pad is None:

@@ -77,7 +77,10 @@ def test_layer_entry_points_reject_uncovered_shapes(lib):
     # K = 8 is not covered by the fused projection
     rc = lib.mccnn_mc_conv_project(None, 3, i64(10), None, 64, None, i64(10), None, i64(20), None,
                                    None, None, 8, 1, 0, None, None, None, None, None)
-    assert rc == 1 and b"K = 16" in lib.mccnn_last_error()
+    assert rc == 1 and b"K in {16,32,64}" in lib.mccnn_last_error()
+    assert lib.mccnn_mc_conv_project_supported(3, 48, 32) == 1
+    assert lib.mccnn_mc_conv_weight_grads_supported(3, 64, 64) == 1
+    assert lib.mccnn_mc_conv_supported(3, 64, 32) == 0          # no feature-gradient half there
     rc = lib.mccnn_kp_conv_project(None, 3, i64(10), None, 64, None, i64(10), None, i64(20), None,
                                    None, None, 17, None, 0, ctypes.c_float(1.0), None, None)
     assert rc == 1 and b"kernel points" in lib.mccnn_last_error()
