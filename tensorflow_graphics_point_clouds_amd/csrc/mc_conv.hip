@@ -210,30 +210,21 @@ __global__ void __launch_bounds__(256) kp_conv_project16_kernel(
                                &stages[threadIdx.x / kWave]);
 }
 
-// Persistent wavefronts stride over the centres.  Per tile of 16 pairs:
-//   dbasis^T [k x pair] by MFMA (reduction over channels), turned in registers
-//   into dz = dbasis * act'(z) / pdf and accumulated into per-lane partial sums
-//   of dW[d][k] = sum delta_d * dz and db[k] = sum dz (lane (pair, quarter) owns
-//   k = 4*quarter .. +3);
-//   dfeat [pair x channel] by MFMA with the recomputed basis as A operand,
-//   added to the feature gradient with fp32 atomics, or (pair_rows given)
-//   stored per pair for the atomic-free gather that follows.
-// At the end the partial sums are reduced over the 16 pair-lanes and the waves
-// of the block and written to partials[block][(D+1)][K].
-// kDB / kDF select the two halves (weight-gradient half, feature-gradient half);
-// launching them as two kernels keeps each under ~90 registers, which more than
-// pays for reading the upstream gradient twice.
-template <int C, int D, int kAct, bool kDB, bool kDF>
-__global__ void __launch_bounds__(256) mc_conv_project_grads16_kernel(
-    int64_t n_out, const float *__restrict__ feat, const int2 *__restrict__ nbrs,
-    const int *__restrict__ ranges, McParams<D> p, const float *__restrict__ in_grad,
-    float *__restrict__ dfeat, float *__restrict__ pair_rows, float *__restrict__ partials) {
+// Feature gradient by scatter, for callers that do not use the transposed
+// convolution: one wavefront per centre, per tile of 16 pairs the basis is
+// recomputed in registers and dfeat [pair x channel] = basis [pair x k] * G [k x
+// channel] comes from the matrix cores; it is added to the feature gradient with
+// fp32 atomics or (pair_rows given) stored per pair for the atomic-free gather
+// that follows.
+template <int C, int D, int kAct>
+__global__ void __launch_bounds__(256) mc_conv_feature_grads16_kernel(
+    int64_t n_out, const int2 *__restrict__ nbrs, const int *__restrict__ ranges, McParams<D> p,
+    const float *__restrict__ in_grad, float *__restrict__ dfeat,
+    float *__restrict__ pair_rows) {
   constexpr int K = kFusedK;
-  constexpr int kQuarterC = C / 4;
   constexpr int kTiles = C / 16;
-  __shared__ float red[kWavesPerBlock][(D + 1) * K];
   __shared__ float wlds[K * (D + 1)];     // column j: D weights then the bias
-  const int lane = lane_id(), wave = threadIdx.x / kWave;
+  const int lane = lane_id();
   const int quarter = lane >> 4, col = lane & 15;
   if (threadIdx.x < K) {
     float w[D], bias;
@@ -246,23 +237,11 @@ __global__ void __launch_bounds__(256) mc_conv_project_grads16_kernel(
   float ir[D];
 #pragma unroll
   for (int d = 0; d < D; ++d) ir[d] = p.inv_radii[d];
-  float dw[4][D], db[4];
-#pragma unroll
-  for (int r = 0; r < 4; ++r) {
-    db[r] = 0.0f;
-#pragma unroll
-    for (int d = 0; d < D; ++d) dw[r][d] = 0.0f;
-  }
   const int64_t total_waves = (int64_t)gridDim.x * kWavesPerBlock;
   for (int64_t centre = wave_slot(); centre < n_out; centre += total_waves) {
     const int a = centre > 0 ? ranges[centre - 1] : 0, b = ranges[centre];
     if (b <= a) continue;
     const float *gi = in_grad + centre * (int64_t)C * K;
-    float gk[kQuarterC];
-    if (kDB) {
-#pragma unroll
-      for (int s = 0; s < kQuarterC; ++s) gk[s] = gi[(quarter * kQuarterC + s) * K + col];
-    }
     float ctr[D];
 #pragma unroll
     for (int d = 0; d < D; ++d) ctr[d] = p.pout[centre * D + d];
@@ -271,15 +250,13 @@ __global__ void __launch_bounds__(256) mc_conv_project_grads16_kernel(
       const int cnt = b - m0 < 16 ? b - m0 : 16;
       const bool valid = col < cnt;
       const int idx = nbrs[m0 + (valid ? col : 0)].x;
-      FVec<kQuarterC> f;
-      if (kDB) f = load_vec<kQuarterC>(feat + (int64_t)idx * C + quarter * kQuarterC, valid);
       const float inv_pdf = valid ? 1.0f / p.pdf[m0 + col] : 0.0f;
       float delta[D];
 #pragma unroll
       for (int d = 0; d < D; ++d)
         delta[d] = valid ? (p.pin[(int64_t)idx * D + d] - ctr[d]) * ir[d] : 0.0f;
-      // for this lane's pair and its four basis columns: basis and act'/pdf
-      float basis4[4], dact4[4];
+      // this lane's pair and its four basis columns 4*quarter .. +3
+      float basis4[4];
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const float *wr = wlds + (4 * quarter + r) * (D + 1);
@@ -287,24 +264,9 @@ __global__ void __launch_bounds__(256) mc_conv_project_grads16_kernel(
 #pragma unroll
         for (int d = 0; d < D; ++d) z += delta[d] * wr[d];
         basis4[r] = valid ? act_fwd(kAct, z) * inv_pdf : 0.0f;
-        dact4[r] = act_bwd(kAct, z) * inv_pdf;
-      }
-      if (kDB) {
-        v4f acc = {0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-        for (int s = 0; s < kQuarterC; ++s)
-          acc = __builtin_amdgcn_mfma_f32_16x16x4f32(gk[s], f.v[s], acc, 0, 0, 0);
-        // acc[r] = dbasis[pair col][k = 4*quarter + r]
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const float dz = acc[r] * dact4[r];
-          db[r] += dz;
-#pragma unroll
-          for (int d = 0; d < D; ++d) dw[r][d] += delta[d] * dz;
-        }
       }
 #pragma unroll
-      for (int t = 0; t < (kDF ? kTiles : 0); ++t) {
+      for (int t = 0; t < kTiles; ++t) {
         // B operand of channel tile t: G[c = 16 t + col][k = 4*quarter + s] (L1 resident)
         const FVec<4> gt = load_vec<4>(gi + (16 * t + col) * K + 4 * quarter, true);
         v4f acc = {0.0f, 0.0f, 0.0f, 0.0f};
@@ -331,33 +293,6 @@ __global__ void __launch_bounds__(256) mc_conv_project_grads16_kernel(
         }
       }
     }
-  }
-  if (!kDB) return;
-  // reduce over the 16 pair-lanes of each quarter
-#pragma unroll
-  for (int r = 0; r < 4; ++r) {
-#pragma unroll
-    for (int off = 8; off > 0; off >>= 1) {
-      db[r] += __shfl_xor(db[r], off, kWave);
-#pragma unroll
-      for (int d = 0; d < D; ++d) dw[r][d] += __shfl_xor(dw[r][d], off, kWave);
-    }
-  }
-  if (col == 0) {
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      const int k = 4 * quarter + r;
-#pragma unroll
-      for (int d = 0; d < D; ++d) red[wave][d * K + k] = dw[r][d];
-      red[wave][D * K + k] = db[r];
-    }
-  }
-  __syncthreads();
-  if (threadIdx.x < (D + 1) * K) {
-    float s = 0.0f;
-#pragma unroll
-    for (int w = 0; w < kWavesPerBlock; ++w) s += red[w][threadIdx.x];
-    partials[(int64_t)blockIdx.x * (D + 1) * K + threadIdx.x] = s;
   }
 }
 
@@ -544,9 +479,9 @@ static int launch_fused_backward(hipStream_t s, int64_t num_samples, const float
       break;
   }
   if (want_dfeat)        // the feature half keeps no running sums: one wavefront per centre
-    hipLaunchKernelGGL((mc_conv_project_grads16_kernel<C, D, ACT, false, true>),
-                       dim3(wave_grid(num_samples)), dim3(256), 0, s, num_samples, features, nb,
-                       ranges, prm, in_grads, feature_grads_out, pair_rows, workspace);
+    hipLaunchKernelGGL((mc_conv_feature_grads16_kernel<C, D, ACT>),
+                       dim3(wave_grid(num_samples)), dim3(256), 0, s, num_samples, nb, ranges, prm,
+                       in_grads, feature_grads_out, pair_rows);
   return MCCNN_OK;
 }
 
