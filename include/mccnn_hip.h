@@ -449,9 +449,10 @@ int mccnn_mc_conv_project_grads(
  * followed by basis_proj in one kernel, the correlation weights
  *   kind 0: max(1 - d/sigma, 0),  kind 1: exp(-(d/(sigma/3))^2),
  *   d = || delta - kernel_points[k] ||,  delta = (p_in[nbr] - p_out[centre]) * inv_radii
- * evaluated in registers.  out [N_out, C, 16]; columns >= num_kernel_points are
- * zero (the padding the reference slices off).  out_rows as for
- * mccnn_mc_conv_project.  D in {2,3}, C in {16,32,64,128}, 1..16 kernel points.
+ * evaluated in registers.  out [N_out, C, 16] for up to 16 kernel points and
+ * [N_out, C, 32] for 17..32; columns >= num_kernel_points are zero (the padding
+ * the reference slices off).  out_rows as for mccnn_mc_conv_project.  D in
+ * {2,3}, C a multiple of 16 up to 512, 1..32 kernel points.
  * No counterpart among the reference's ops. */
 int mccnn_kp_conv_project(mccnn_stream_t stream, int num_dims, int64_t num_pts,
                           const float *points_in, int num_features,

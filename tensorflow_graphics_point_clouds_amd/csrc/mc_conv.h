@@ -68,20 +68,23 @@ struct MlpBasis {                  // act(delta . W[:, col] + b[col]) / pdf   (M
   }
 };
 
-template <int D, int kKind>
+template <int D, int kKind, int KT = 1>
 struct KpBasis {                   // kernel-point correlation (KPConv.py:29-57, 193-213)
-  float k[3], sigma;
-  bool live;                       // columns past the last kernel point are zero padding
+  float k[KT][3], sigma;
+  bool live[KT];                   // columns past the last kernel point are zero padding
   __device__ __forceinline__ KpBasis(const float *__restrict__ kernel_points, int num_kp,
                                      float sigma_) : sigma(sigma_) {
-    const int col = lane_id() & 15;
-    live = col < num_kp;
-    k[0] = k[1] = k[2] = 0.0f;
 #pragma unroll
-    for (int d = 0; d < D; ++d) k[d] = live ? kernel_points[col * D + d] : 0.0f;
+    for (int kt = 0; kt < KT; ++kt) {
+      const int col = 16 * kt + (lane_id() & 15);
+      live[kt] = col < num_kp;
+      k[kt][0] = k[kt][1] = k[kt][2] = 0.0f;
+#pragma unroll
+      for (int d = 0; d < D; ++d) k[kt][d] = live[kt] ? kernel_points[col * D + d] : 0.0f;
+    }
   }
-  __device__ __forceinline__ float operator()(const float4 &g, int = 0) const {
-    const float dx = g.x - k[0], dy = g.y - k[1], dz = g.z - k[2];
+  __device__ __forceinline__ float operator()(const float4 &g, int kt = 0) const {
+    const float dx = g.x - k[kt][0], dy = g.y - k[kt][1], dz = g.z - k[kt][2];
     const float dist = sqrtf(dx * dx + dy * dy + dz * dz);
     float wgt;
     if (kKind == 0) {
@@ -91,7 +94,7 @@ struct KpBasis {                   // kernel-point correlation (KPConv.py:29-57,
       const float q = dist / (sigma / 3.0f);
       wgt = expf(-(q * q));
     }
-    return live ? wgt * g.w : 0.0f;
+    return live[kt] ? wgt * g.w : 0.0f;
   }
 };
 

@@ -197,17 +197,18 @@ __global__ void __launch_bounds__(256) mc_conv_project16_kernel(
 }
 
 // The same projection with the kernel-point correlation of KPConv as basis
-// (KPConv.py:193-224: weights of up to 16 kernel points, zero padding beyond).
-template <int kCPL, int D, int kKind>
+// (KPConv.py:193-224: weights of up to 32 kernel points in one or two tiles of 16
+// columns, zero padding beyond the last point).
+template <int kCPL, int D, int kKind, int KT>
 __global__ void __launch_bounds__(256) kp_conv_project16_kernel(
     int64_t n_out, int C, int chunks, const float *__restrict__ feat,
     const int2 *__restrict__ nbrs, const int *__restrict__ ranges, McParams<D> p,
     const float *__restrict__ kernel_points, int num_kp, float sigma,
     const int *__restrict__ out_rows, float *__restrict__ out) {
   __shared__ PairStage stages[kWavesPerBlock];
-  const KpBasis<D, kKind> basis(kernel_points, num_kp, sigma);
-  project_run_body<kCPL, D, 1>(n_out, C, chunks, feat, nbrs, ranges, p, basis, out_rows, out,
-                               &stages[threadIdx.x / kWave]);
+  const KpBasis<D, kKind, KT> basis(kernel_points, num_kp, sigma);
+  project_run_body<kCPL, D, KT>(n_out, C, chunks, feat, nbrs, ranges, p, basis, out_rows, out,
+                                &stages[threadIdx.x / kWave]);
 }
 
 // Feature gradient by scatter, for callers that do not use the transposed
@@ -680,8 +681,8 @@ extern "C" int mccnn_kp_conv_project(mccnn_stream_t stream, int num_dims, int64_
   MCCNN_REQUIRE(project_supported(num_dims, num_features, kFusedK),
                 "kp_conv_project supports D in {2,3} and C in {16, 32, ..., 512} (got D=%d, C=%d); "
                 "use kp_basis + basis_proj for other shapes", num_dims, num_features);
-  MCCNN_REQUIRE(num_kernel_points > 0 && num_kernel_points <= kFusedK,
-                "kp_conv_project supports 1 to 16 kernel points (got %d)", num_kernel_points);
+  MCCNN_REQUIRE(num_kernel_points > 0 && num_kernel_points <= 2 * kFusedK,
+                "kp_conv_project supports 1 to 32 kernel points (got %d)", num_kernel_points);
   MCCNN_REQUIRE(kind == 0 || kind == 1, "kp_conv_project expects kind 0 (linear) or 1 (gaussian)");
   MCCNN_REQUIRE(sigma > 0.0f, "kp_conv_project expects a positive sigma");
   MCCNN_REQUIRE(num_neighbors >= 0 && num_neighbors < ((int64_t)1 << 31) && num_samples >= 0 &&
@@ -694,30 +695,35 @@ extern "C" int mccnn_kp_conv_project(mccnn_stream_t stream, int num_dims, int64_
                     (num_neighbors == 0 || (points_in && features && neighbors)),
                 "kp_conv_project received a null tensor");
   hipStream_t s = as_stream(stream);
+  // out is [N_out, C, 16] for up to 16 kernel points and [N_out, C, 32] beyond
+  const int kt = num_kernel_points > kFusedK ? 2 : 1;
   int cpl = 1;
-  for (int c = 8; c >= 1; c >>= 1)
+  for (int c = 8 / kt; c >= 1; c >>= 1)
     if (num_features % (16 * c) == 0) { cpl = c; break; }
   const int chunks = num_features / (16 * cpl);
   const dim3 grid(wave_grid((num_samples + kProjRun - 1) / kProjRun * chunks)), block(256);
   const int2 *nb = (const int2 *)neighbors;
-#define MCCNN_KP_FWD(CPL_, D_, KIND_)                                                          \
+#define MCCNN_KP_FWD(CPL_, D_, KIND_, KT_)                                                     \
   {                                                                                            \
     McParams<D_> prm{points_in, points_out, inv_radii, nullptr, nullptr, nullptr, 1, 0};       \
-    hipLaunchKernelGGL((kp_conv_project16_kernel<CPL_, D_, KIND_>), grid, block, 0, s,         \
+    hipLaunchKernelGGL((kp_conv_project16_kernel<CPL_, D_, KIND_, KT_>), grid, block, 0, s,    \
                        num_samples, num_features, chunks, features, nb, ranges, prm,           \
                        kernel_points, num_kernel_points, sigma, out_rows, out);                \
   }
-#define MCCNN_KP_FWD_D(CPL_)                                             \
-  if (num_dims == 3) {                                                   \
-    if (kind == 0) MCCNN_KP_FWD(CPL_, 3, 0) else MCCNN_KP_FWD(CPL_, 3, 1) \
-  } else {                                                               \
-    if (kind == 0) MCCNN_KP_FWD(CPL_, 2, 0) else MCCNN_KP_FWD(CPL_, 2, 1) \
+#define MCCNN_KP_FWD_D(CPL_, KT_)                                                  \
+  if (num_dims == 3) {                                                             \
+    if (kind == 0) MCCNN_KP_FWD(CPL_, 3, 0, KT_) else MCCNN_KP_FWD(CPL_, 3, 1, KT_) \
+  } else {                                                                         \
+    if (kind == 0) MCCNN_KP_FWD(CPL_, 2, 0, KT_) else MCCNN_KP_FWD(CPL_, 2, 1, KT_) \
   }
-  switch (cpl) {
-    case 8: MCCNN_KP_FWD_D(8); break;
-    case 4: MCCNN_KP_FWD_D(4); break;
-    case 2: MCCNN_KP_FWD_D(2); break;
-    default: MCCNN_KP_FWD_D(1); break;
+  switch (kt * 16 + cpl) {
+    case 16 + 8: MCCNN_KP_FWD_D(8, 1); break;
+    case 16 + 4: MCCNN_KP_FWD_D(4, 1); break;
+    case 16 + 2: MCCNN_KP_FWD_D(2, 1); break;
+    case 16 + 1: MCCNN_KP_FWD_D(1, 1); break;
+    case 32 + 4: MCCNN_KP_FWD_D(4, 2); break;
+    case 32 + 2: MCCNN_KP_FWD_D(2, 2); break;
+    default: MCCNN_KP_FWD_D(1, 2); break;
   }
 #undef MCCNN_KP_FWD_D
 #undef MCCNN_KP_FWD

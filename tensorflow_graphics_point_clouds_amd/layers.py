@@ -571,7 +571,10 @@ class PointConv(torch.nn.Module):
 
 
 def _padded_basis_count(num_kernel_points):
-    for k in (8, 16, 32, 64):
+    """Basis columns for a kernel of this many points (KPConv.py:199-213 pads to 8,
+    16, 32 or 64; 16 is the narrowest tile of the projection kernels, so kernels
+    of up to 8 points are padded to 16 here, with zero columns either way)."""
+    for k in (16, 32, 64):
         if num_kernel_points <= k:
             return k
     raise ValueError("at most 64 kernel points are supported")
@@ -661,7 +664,7 @@ def _kp_project(features, points_in, points_out, neighbors, ranges, inv_radii, k
     registers) when the shape is covered, else kp_basis followed by basis_proj."""
     kp, dims = kernel_points.shape
     c = features.shape[1]
-    if k == 16 and _lib.lib().mccnn_mc_conv_project_supported(cint(dims), cint(c), cint(16)):
+    if k in (16, 32) and _lib.lib().mccnn_mc_conv_project_supported(cint(dims), cint(c), cint(k)):
         out = torch.empty((ranges.shape[0], c, k), dtype=_F32, device=features.device)
         _lib.call("kp_conv_project", stream(), cint(dims), i64(features.shape[0]),
                   ptr(points_in, _F32), cint(c), ptr(features, _F32), i64(ranges.shape[0]),

@@ -82,7 +82,7 @@ def test_layer_entry_points_reject_uncovered_shapes(lib):
     assert lib.mccnn_mc_conv_weight_grads_supported(3, 64, 64) == 1
     assert lib.mccnn_mc_conv_supported(3, 64, 32) == 0          # no feature-gradient half there
     rc = lib.mccnn_kp_conv_project(None, 3, i64(10), None, 64, None, i64(10), None, i64(20), None,
-                                   None, None, 17, None, 0, ctypes.c_float(1.0), None, None)
+                                   None, None, 33, None, 0, ctypes.c_float(1.0), None, None)
     assert rc == 1 and b"kernel points" in lib.mccnn_last_error()
     rc = lib.mccnn_weight_grad_product(None, i64(10), 48, None, 1024, None, None, sz(0), None)
     assert rc == 1 and b"output rows" in lib.mccnn_last_error()

@@ -149,25 +149,32 @@ def test_pointconv_forward_backward(oracle, hidden, act):
     normwise(conv.pdf_biases_2.grad.cpu().numpy(), t["pb2"].grad.numpy(), tol=5e-5)
 
 
-@pytest.mark.parametrize("c_in,c_out,transposed", [(16, 24, True), (16, 24, False),
-                                                   (64, 32, True), (8, 16, True)])
+@pytest.mark.parametrize("c_in,c_out,transposed,kpn", [(16, 24, True, 15), (16, 24, False, 15),
+                                                       (64, 32, True, 15), (8, 16, True, 15),
+                                                       (16, 16, True, 5), (32, 8, True, 18),
+                                                       (16, 8, False, 18), (8, 8, True, 7)])
 @pytest.mark.parametrize("kind,influence", [("linear", None), ("gaussian", 0.3 * 0.15)])
-def test_kpconv_forward_backward(oracle, kind, influence, c_in, c_out, transposed):
+def test_kpconv_forward_backward(oracle, kind, influence, c_in, c_out, transposed, kpn):
+    """Rigid kernel-point convolution for the reference's kernel sizes (5 and 7 points
+    padded to 16 basis columns, 15 to 16, 18 to 32; KPConv.py:199-213)."""
     from tensorflow_graphics_point_clouds_amd import layers, pc, synthetic
     rng = np.random.default_rng(5)
     batch, radius = 2, 0.15
     pts, bids, ctr, cb, nbh = _setup(oracle, rng, batch=batch, radius=radius)
     feat = rng.standard_normal((len(pts), c_in)).astype(np.float32)
-    kp = synthetic.spherical_kernel_points(15, rotate=False) * 0.8      # * 0.75 inside the layer = 0.6
-    wts = (rng.standard_normal((15 * c_in, c_out)) * 0.1).astype(np.float32)
+    kp = synthetic.spherical_kernel_points(kpn, rotate=False) * 0.8     # * 0.75 inside the layer = 0.6
+    if kpn == 13:
+        kp = kp / 1.902
+    wts = (rng.standard_normal((kpn * c_in, c_out)) * 0.1).astype(np.float32)
     sigma = 1.0 if influence is None else influence / radius
     ids = nbh.original_neigh_ids
     radii = np.full(3, np.float32(radius), np.float32)
     diff = (pts[ids[:, 0]] - ctr[ids[:, 1]]) / radii
     basis, _ = oracle.kp_basis(diff, kp.astype(np.float64) * 0.75, sigma, kind)
-    padded = np.zeros((len(ids), 16), np.float32)
-    padded[:, :15] = basis
-    proj = oracle.basis_proj(padded, feat, ids, nbh.ranges)[:, :, :15]
+    kpad = 16 if kpn <= 16 else 32
+    padded = np.zeros((len(ids), kpad), np.float32)
+    padded[:, :kpn] = basis
+    proj = oracle.basis_proj(padded, feat, ids, nbh.ranges)[:, :, :kpn]
     expect = proj.reshape(len(ctr), -1) @ wts.astype(np.float64)
 
     conv = layers.KPConv(c_in, c_out, custom_kernel_points=kp, kp_interpolation=kind,
@@ -179,9 +186,9 @@ def test_kpconv_forward_backward(oracle, kind, influence, c_in, c_out, transpose
     normwise(out.detach().cpu().numpy(), expect, tol=2e-5)
     up = rng.standard_normal(expect.shape).astype(np.float32)
     out.backward(dev(up))
-    dproj = (up.astype(np.float64) @ wts.astype(np.float64).T).reshape(len(ctr), c_in, 15)
-    dpad = np.zeros((len(ctr), c_in, 16), np.float32)
-    dpad[:, :, :15] = dproj
+    dproj = (up.astype(np.float64) @ wts.astype(np.float64).T).reshape(len(ctr), c_in, kpn)
+    dpad = np.zeros((len(ctr), c_in, kpad), np.float32)
+    dpad[:, :, :kpn] = dproj
     _, dfeat = oracle.basis_proj_grads(padded, feat, ids, nbh.ranges, dpad)
     normwise(tfeat.grad.cpu().numpy(), dfeat, tol=2e-5)
     normwise(conv.weights.grad.cpu().numpy(), proj.reshape(len(ctr), -1).T @ up.astype(np.float64),
