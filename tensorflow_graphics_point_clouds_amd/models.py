@@ -46,13 +46,20 @@ class ConvBlock(torch.nn.Module):
 
     def forward(self, features, point_cloud_in, point_cloud_out, conv_radius, pool_radius=None,
                 training=None):
+        # the convolution and the pooling of a strided block look at the same pairs
+        # when their radii agree (modelnet40.py:373-379 passes the pooling radius twice)
+        shared = None
+        if self.pool is not None and pool_radius is not None and \
+                float(conv_radius) == float(pool_radius):
+            radii = pc._as_vector(conv_radius, 3, point_cloud_in._points.device)
+            shared = pc.Neighborhood(pc.Grid(point_cloud_in, radii), radii, point_cloud_out)
         res = self.reduce(self.act(self.norms[0](features, training)), point_cloud_in)
         res = self.conv(self.act(self.norms[1](res, training)), point_cloud_in, point_cloud_out,
-                        conv_radius)
+                        conv_radius, shared)
         res = self.expand(self.act(self.norms[2](res, training)), point_cloud_out)
         skip = features
         if self.pool is not None:
-            skip = self.pool(skip, point_cloud_in, point_cloud_out, pool_radius)
+            skip = self.pool(skip, point_cloud_in, point_cloud_out, pool_radius, shared)
         if self.skip_conv is not None:
             skip = self.skip_conv(self.act(self.skip_norm(skip, training)), point_cloud_out)
         return res + skip
