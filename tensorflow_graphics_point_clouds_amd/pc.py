@@ -208,7 +208,9 @@ class Grid:
     """Regular grid over a point cloud (pylib/pc/Grid.py:32-84): grid shape from
     the per-cloud bounding boxes, cell keys, stable descending sort, gathers."""
 
-    def __init__(self, point_cloud, cell_sizes):
+    def __init__(self, point_cloud, cell_sizes, aabb=None):
+        # `aabb` is accepted for the reference's signature; like the reference
+        # (Grid.py:42-44) the grid always takes the cloud's own bounding boxes
         L = _lib.lib()
         pc = point_cloud
         dev, n, d, b = pc._points.device, pc._points.shape[0], pc._dimension, pc._batch_size
