@@ -557,3 +557,27 @@ def test_object_level_adapters_match_the_callers(ops):
     feat = torch.randn((5000, 8), device="cuda")
     assert torch.equal(custom_ops.basis_proj(basis, feat, nbh),
                        ops.basis_proj(basis, feat, nbh._original_neigh_ids, ranges))
+
+
+def test_row_and_density_gathers(ops):
+    """The glue gathers the layers use: feature rows by int32 index (any row length
+    that is a multiple of 4) and per-pair densities from either column of a pair
+    table."""
+    from tensorflow_graphics_point_clouds_amd import _lib
+    from tensorflow_graphics_point_clouds_amd._lib import cint, i64, ptr, stream
+    gen = torch.Generator(device="cuda").manual_seed(0)
+    for n, c, m in ((1000, 4, 3000), (5000, 64, 777), (300, 132, 300), (7, 8, 0)):
+        x = torch.randn((n, c), device="cuda", generator=gen)
+        rows = torch.randint(0, n, (m,), device="cuda", generator=gen, dtype=torch.int32)
+        out = torch.empty((m, c), device="cuda")
+        _lib.call("gather_rows", stream(), i64(m), cint(c), ptr(x), ptr(rows), ptr(out))
+        assert torch.equal(out, x[rows.long()])
+    with pytest.raises(ValueError):
+        _lib.call("gather_rows", stream(), i64(4), cint(6), ptr(x), ptr(rows), ptr(out))
+    pairs = torch.randint(0, 500, (4000, 2), device="cuda", generator=gen, dtype=torch.int32)
+    pdf = torch.rand(500, device="cuda", generator=gen)
+    for column in (0, 1):
+        out = torch.empty(4000, device="cuda")
+        _lib.call("gather_pdf_column", stream(), i64(4000), ptr(pairs), cint(column), ptr(pdf),
+                  ptr(out))
+        assert torch.equal(out, pdf[pairs[:, column].long()])
