@@ -131,12 +131,18 @@ __global__ void aabb_init_kernel(int count, unsigned *mn, unsigned *mx) {
   }
 }
 
-// A wavefront walks a run of kAabbRun points.  While the 64 points of an
+// A wavefront walks a run of points (1024 for a large cloud, down to 64 for a small
+// one, so that a few thousand points still spread over many wavefronts).  While the 64 points of an
 // iteration belong to one cloud (the usual layout: clouds stored one after
 // another) the lanes keep running minima / maxima in registers; they are reduced
 // over the wavefront and sent as one atomic per dimension when the cloud changes
 // or the run ends.  Iterations that straddle two clouds use one atomic per lane.
 constexpr int kAabbRun = 1024;
+
+static int aabb_run(int64_t n) {
+  int64_t run = (n / 2048 + kWave - 1) / kWave * kWave;     // aim at ~2048 wavefronts
+  return (int)(run < kWave ? kWave : (run > kAabbRun ? kAabbRun : run));
+}
 
 template <int D>
 __device__ __forceinline__ void aabb_flush(int b, float *lo, float *hi, unsigned *mn,
@@ -159,11 +165,11 @@ __device__ __forceinline__ void aabb_flush(int b, float *lo, float *hi, unsigned
 
 template <int D>
 __global__ void __launch_bounds__(256) aabb_reduce_kernel(
-    int64_t n, const float *__restrict__ pts, const int *__restrict__ bids,
+    int64_t n, int run, const float *__restrict__ pts, const int *__restrict__ bids,
     unsigned *mn, unsigned *mx) {
   const int64_t wave = blockIdx.x * (int64_t)(blockDim.x / kWave) + threadIdx.x / kWave;
-  const int64_t first = wave * kAabbRun;
-  const int64_t last = first + kAabbRun < n ? first + kAabbRun : n;
+  const int64_t first = wave * run;
+  const int64_t last = first + run < n ? first + run : n;
   float lo[D], hi[D];
 #pragma unroll
   for (int d = 0; d < D; ++d) {
@@ -328,10 +334,11 @@ extern "C" int mccnn_grid_setup(mccnn_stream_t stream, int64_t num_pts, int num_
   MCCNN_LAUNCH_CHECK();
   if (num_pts > 0) {
     MCCNN_REQUIRE(points && batch_ids, "grid_setup received a null tensor");
+    const int run = aabb_run(num_pts);
     MCCNN_DIM_SWITCH(num_dims, hipLaunchKernelGGL(aabb_reduce_kernel<D>,
-                                                  dim3(blocks_for(num_pts, 4 * kAabbRun)),
+                                                  dim3(blocks_for(num_pts, 4 * run)),
                                                   dim3(256), 0,
-                                                  as_stream(stream), num_pts, points, batch_ids,
+                                                  as_stream(stream), num_pts, run, points, batch_ids,
                                                   (unsigned *)aabb_min_out,
                                                   (unsigned *)aabb_max_out));
     MCCNN_LAUNCH_CHECK();

@@ -8,6 +8,8 @@ import ctypes
 import enum
 import math
 
+import numpy as np
+
 import torch
 
 from . import _lib, tfg_custom_ops
@@ -24,11 +26,40 @@ class KDEMode(enum.Enum):
     no_pdf = 2
 
 
+_vector_cache = {}
+_vector_values = {}
+
+
 def _as_vector(value, dims, device):
-    t = torch.as_tensor(value, dtype=_F32).reshape(-1)
-    if t.numel() == 1:
-        t = t.repeat(dims)
-    return t.to(device).contiguous()
+    """`value` (a number, a sequence or a tensor) as a float32 [dims] tensor on
+    `device`.  Host numbers are uploaded once per (value, dims, device) and the
+    tensor is shared read-only afterwards: radii and cell sizes repeat in every
+    layer of a network."""
+    if isinstance(value, torch.Tensor):
+        t = value.to(dtype=_F32).reshape(-1)
+        if t.numel() == 1:
+            t = t.repeat(dims)
+        return t.to(device).contiguous()
+    host = np.asarray(value, dtype=np.float32).reshape(-1)
+    key = (host.tobytes(), int(dims), str(device))
+    t = _vector_cache.get(key)
+    if t is None:
+        t = torch.as_tensor(host)
+        if t.numel() == 1:
+            t = t.repeat(dims)
+        t = t.to(device).contiguous()
+        if len(_vector_cache) < 4096:
+            _vector_cache[key] = t
+            _vector_values[t.data_ptr()] = tuple(float(v) for v in t.tolist())
+    return t
+
+
+def _host_values(t):
+    """The entries of a small device vector as a tuple of floats; no device round
+    trip for the vectors `_as_vector` keeps."""
+    known = _vector_values.get(t.data_ptr())
+    return known if known is not None and len(known) == t.numel() else \
+        tuple(float(v) for v in t.tolist())
 
 
 class AABB:
@@ -256,7 +287,7 @@ class Grid:
         """The neighbourhood of the grid's sorted points among themselves for these
         radii, built once and shared (densities, grid-ordered view, same-cloud
         convolutions)."""
-        key = (tuple(float(r) for r in radii.tolist()), int(max_neighbors))
+        key = (_host_values(radii), int(max_neighbors))
         if key not in self._self_neighborhoods:
             self._self_neighborhoods[key] = Neighborhood(self, radii, None, max_neighbors)
         return self._self_neighborhoods[key]
