@@ -299,9 +299,10 @@ extern "C" int mccnn_find_neighbors_count(
   MCCNN_HIP_CHECK(hipMemcpyAsync(num_neighbors_out_host, w.total, sizeof(int64_t),
                                  hipMemcpyDeviceToHost, s));
   MCCNN_HIP_CHECK(hipStreamSynchronize(s));
-  MCCNN_REQUIRE(*num_neighbors_out_host < ((int64_t)1 << 31),
-                "FindNeighbors found %lld pairs; the int32 offsets of the op contract hold fewer "
-                "than 2^31",
+  // the scan saturates partial sums at 2^31 - 1, so a total from there on is a lower bound
+  MCCNN_REQUIRE(*num_neighbors_out_host < (((int64_t)1 << 31) - 1),
+                "FindNeighbors found at least %lld pairs; the int32 offsets of the op contract "
+                "hold fewer than 2^31 - 1",
                 (long long)*num_neighbors_out_host);
   return MCCNN_OK;
 }

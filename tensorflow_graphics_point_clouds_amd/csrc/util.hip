@@ -35,8 +35,11 @@ int fill_zero(hipStream_t stream, void *ptr, size_t bytes) {
 // ------------------------------------------------------------ prefix sum ----
 // Three launches, no inter-block waiting: (1) each block of kScanTile items
 // writes its sum, (2) one block scans the block sums, (3) each block rescans its
-// tile with the carried-in offset.  Totals stay below 2^31 (pair counts are
-// int32 in the op contract); the grand total is also stored as int64.
+// tile with the carried-in offset.  The scanned values are int32 (pair counts are
+// int32 in the op contract); tile sums and the grand total are formed in 64 bits
+// and a tile sum that does not fit saturates, so that a total of 2^31 - 1 or more
+// is always reported as at least 2^31 - 1 and the callers can refuse it instead
+// of working on wrapped offsets.
 
 constexpr int kScanThreads = 256;
 constexpr int kScanItems = 8;
@@ -61,28 +64,57 @@ __device__ __forceinline__ int block_exclusive_scan(int v, int *total) {
   return carry + incl - v;
 }
 
+constexpr long long kScanMax = 0x7fffffffLL;
+
+__device__ __forceinline__ int saturate_i32(long long v) {
+  return (int)(v > kScanMax ? kScanMax : v);
+}
+
+// 64-bit counterpart of block_exclusive_scan for the sums of whole tiles.
+__device__ __forceinline__ long long block_exclusive_scan_i64(long long v, long long *total) {
+  __shared__ long long wave_sums[kScanThreads / kWave];
+  const int lane = lane_id(), wave = threadIdx.x / kWave;
+  long long incl = v;
+#pragma unroll
+  for (int off = 1; off < kWave; off <<= 1) {
+    const long long t = __shfl_up(incl, off, kWave);
+    if (lane >= off) incl += t;
+  }
+  if (lane == kWave - 1) wave_sums[wave] = incl;
+  __syncthreads();
+  long long carry = 0, sum = 0;
+#pragma unroll
+  for (int w = 0; w < kScanThreads / kWave; ++w) {
+    if (w < wave) carry += wave_sums[w];
+    sum += wave_sums[w];
+  }
+  __syncthreads();
+  *total = sum;
+  return carry + incl - v;
+}
+
 __global__ void __launch_bounds__(kScanThreads) scan_tile_sums_kernel(
     int64_t n, const int *__restrict__ counts, int *__restrict__ block_sums) {
   const int64_t base = (int64_t)blockIdx.x * kScanTile + (int64_t)threadIdx.x * kScanItems;
-  int s = 0;
+  long long s = 0;
 #pragma unroll
   for (int k = 0; k < kScanItems; ++k)
     if (base + k < n) s += counts[base + k];
-  int total;
-  block_exclusive_scan(s, &total);
-  if (threadIdx.x == 0) block_sums[blockIdx.x] = total;
+  long long total;
+  block_exclusive_scan_i64(s, &total);
+  if (threadIdx.x == 0) block_sums[blockIdx.x] = saturate_i32(total);
 }
 
 // Single block: exclusive scan of block_sums[0..nb) in place, total to *total_dev.
 __global__ void __launch_bounds__(kScanThreads) scan_block_sums_kernel(int nb, int *block_sums,
                                                                        int64_t *total_dev) {
-  int carry = 0;
+  long long carry = 0;
   for (int base = 0; base < nb; base += kScanThreads) {
     const int i = base + threadIdx.x;
-    const int v = i < nb ? block_sums[i] : 0;
-    int total;
-    const int ex = block_exclusive_scan(v, &total);
-    if (i < nb) block_sums[i] = carry + ex;
+    const long long v = i < nb ? block_sums[i] : 0;
+    long long total;
+    const long long ex = block_exclusive_scan_i64(v, &total);
+    if (i < nb) block_sums[i] = saturate_i32(carry + ex);
     carry += total;
   }
   if (threadIdx.x == 0) *total_dev = carry;

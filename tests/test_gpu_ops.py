@@ -153,6 +153,22 @@ def test_neighbors_max_neighs_and_anisotropic_radii(ops, oracle):
         assert np.array_equal(nbrs.cpu().numpy(), nbh.neighbors)
 
 
+@pytest.mark.parametrize("n", [50000, 66000])
+def test_neighbors_refuses_pair_counts_beyond_int32(ops, oracle, n):
+    """Every point within reach of every other: n^2 pairs, 2.5e9 (past 2^31) and
+    4.36e9 (past 2^32, which a wrapped 32-bit total would report as 6.1e7).  The
+    offsets of the op contract are int32, so the op has to refuse, not wrap."""
+    rng = np.random.default_rng(n)
+    pts = (rng.random((n, 3)) * 0.1).astype(np.float32)
+    bids = np.zeros(n, np.int32)
+    g = oracle.Grid(pts, bids, 1, 1.0)
+    with pytest.raises(ValueError, match="pairs"):
+        _gpu_neighbors(ops, g, pts, bids, np.full(3, 1.0, np.float32))
+    # the library is usable afterwards
+    ranges, _ = _gpu_neighbors(ops, g, pts[:100], bids[:100], np.full(3, 1.0, np.float32))
+    assert np.array_equal(ranges.cpu().numpy(), n * np.arange(1, 101))
+
+
 def test_neighbors_clustered_cloud(ops, oracle):
     """Heavy-tailed neighbour counts (blobs + noise), the shape of the scene-scale
     configuration at 1/50 of its size."""
