@@ -312,6 +312,22 @@ def isolated_basis_proj(torch, pc, synthetic, tfg, _lib, radius=0.04, steps=5):
     # the same pairs with points and centres renumbered in grid-cell order
     view = nbh.sorted_view()
     run("_grid_order", view.table, view.ranges, feat[view.point_order].contiguous())
+    del basis, up, feat
+    # the density estimate and Poisson-disk sampling at the same radius (self neighbourhood)
+    self_nbh = pc.Neighborhood(grid, radius)
+    for timed in (False, True):
+        if timed:
+            _lib.start_timing()
+        for _ in range(steps if timed else 1):
+            self_nbh.compute_pdf(bandwidth=0.2)
+            sampled, _ = pc.sample(self_nbh, "poisson")
+    t = _lib.collect_timing()
+    ms = sum(t["compute_pdf"]) / steps
+    by = N * 4 * 3 + 8 * M + 4 * N + M * 4 * 3 + 4 * N
+    res["compute_pdf"] = {"ms": ms, "GBps": by / ms / 1e6, "frac_hbm_peak": by / ms / 1e6 / HBM_PEAK_GBS,
+                          "algorithmic_bytes": by}
+    res["poisson_disk_sampling"] = {"ms": (sum(t["sampling_count"]) + sum(t["sampling_fill"])) / steps,
+                                    "selected": int(sampled._points.shape[0])}
     return res
 
 
@@ -441,6 +457,12 @@ def main():
         result["basis_proj_isolated"] = isolated_basis_proj(torch, pc, synthetic, tfg_custom_ops,
                                                             _lib)
         torch.cuda.empty_cache()
+        # the other two radii of the dense case's sweep (about 7 and 180 pairs per point)
+        result["dense_radius_sweep"] = {}
+        for radius in (0.02, 0.06):
+            result["dense_radius_sweep"]["r=%.2f" % radius] = isolated_basis_proj(
+                torch, pc, synthetic, tfg_custom_ops, _lib, radius=radius, steps=3)
+            torch.cuda.empty_cache()
         result["per_op_dense_case"] = per_op_times(torch, pc, layers, synthetic, _lib)
         torch.cuda.empty_cache()
         result["kpconv_config5"] = kpconv_config5(torch, pc, layers, synthetic, _lib)

@@ -7,8 +7,7 @@
 // cell list and both outputs keep the sorted order (the reference compacts with
 // a global atomic counter and leaves the order to chance).  Poisson disk keeps
 // the reference's 2^D cell-parity launches; inside a launch one wavefront owns a
-// cell, visits its points in order and spreads each point's neighbour list over
-// its lanes.  Cell averages are summed serially in sorted order so that the
+// cell and decides its points in order (details at the kernel).  Cell averages are summed serially in sorted order so that the
 // result is bit-reproducible (later hierarchy levels derive integer keys from
 // these points).
 #include "common.h"
@@ -35,46 +34,67 @@ __global__ void __launch_bounds__(256) store_cell_starts_kernel(int64_t n,
     if (i == 0 || keys[i] != keys[i - 1]) first_idx[cell_scan[i] - 1] = (int)i;
 }
 
-// One wavefront per occupied cell whose index parity matches `call`
-// (bit d of call <-> parity of the cell index in dim d).
+// Parity class of every occupied cell: bit d = parity of the cell index in dim d.
 template <int D>
+__global__ void __launch_bounds__(256) cell_class_kernel(
+    const int64_t *__restrict__ num_cells_total /*device*/, const int64_t *__restrict__ keys,
+    const int *__restrict__ num_cells, const int *__restrict__ first_idx,
+    int *__restrict__ cell_class) {
+  const int64_t cells = *num_cells_total;
+  for (int64_t u = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; u < cells;
+       u += (int64_t)gridDim.x * blockDim.x) {
+    // decode the cell index of the key (batch digit dropped)
+    int64_t aux = keys[first_idx[u]];
+    int cls = 0;
+#pragma unroll
+    for (int d = D - 1; d >= 0; --d) {
+      const int nd = num_cells[d];
+      const int cd = (int)(aux % nd);
+      aux /= nd;
+      cls |= (cd & 1) << d;
+    }
+    cell_class[u] = cls;
+  }
+}
+
+// One wavefront per occupied cell of parity class `call`: it visits the cell's
+// points in ascending sorted index and spreads each point's neighbour list over its
+// lanes; a point is selected unless one of its neighbours already is.  (Cells of one
+// class are at least a cell apart, so only the wavefront's own selections can change
+// under it during a pass.  Sweeping a cell's whole pair stretch first, to leave only
+// a register-level pass for the order-dependent part, was measured and is not
+// faster: the passes are bound by the launch of a wavefront per cell and by the
+// latency of the sweep, not by the chain from point to point.)
 __global__ void __launch_bounds__(256) poisson_pass_kernel(
     int64_t n, int call, const int64_t *__restrict__ num_cells_total /*device*/,
-    const int64_t *__restrict__ keys, const int *__restrict__ num_cells,
-    const int2 *__restrict__ nbrs, const int *__restrict__ ranges,
-    const int *__restrict__ first_idx, int *used) {
+    const int *__restrict__ cell_class, const int2 *__restrict__ nbrs,
+    const int *__restrict__ ranges, const int *__restrict__ first_idx, int *used) {
   const int64_t cells = *num_cells_total;
   const int64_t u = __builtin_amdgcn_readfirstlane(
       (int)((blockIdx.x * (int64_t)blockDim.x + threadIdx.x) / kWave));
-  if (u >= cells) return;
+  if (u >= cells || cell_class[u] != call) return;
   const int lane = lane_id();
-  int64_t i = first_idx[u];
-  const int64_t key = keys[i];
-  // decode the cell index of the key (batch digit dropped)
-  int64_t aux = key;
-  bool valid = true;
-#pragma unroll
-  for (int d = D - 1; d >= 0; --d) {
-    const int nd = num_cells[d];
-    const int cd = (int)(aux % nd);
-    aux /= nd;
-    valid = valid && ((cd & 1) == ((call >> d) & 1));
-  }
-  if (!valid) return;
-  while (i < n && keys[i] == key) {
+  const int64_t cell_end = u + 1 < cells ? (int64_t)first_idx[u + 1] : n;
+  for (int64_t i = first_idx[u]; i < cell_end; ++i) {
     const int a = i > 0 ? ranges[i - 1] : 0, b = ranges[i];
     bool taken = false;
     for (int m = a + lane; m < b; m += kWave) {
       const int nb = nbrs[m].x;
-      taken = taken || __hip_atomic_load(&used[nb], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0;
+      taken = taken ||
+              __hip_atomic_load(&used[nb], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0;
     }
     if (!__any(taken)) {
-      if (lane == 0)
-        __hip_atomic_store(&used[i], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      // later points of this cell must observe the selection
-      __threadfence();
+      if (lane == 0) __hip_atomic_store(&used[i], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      // Later points of this cell must observe the selection.  They are visited by
+      // this same wavefront, and `used` is read and written past the per-CU cache
+      // (device-scope atomics), so it is enough that the store has reached L2 before
+      // the next loads are issued: a workgroup-scope fence.  A device-scope fence here
+      // also writes the whole L2 back, once per selected point; other wavefronts only
+      // need the selections in the next launch.
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
     }
-    ++i;
   }
 }
 
@@ -215,14 +235,17 @@ extern "C" int mccnn_sampling_count(mccnn_stream_t stream, int mode, int64_t num
   if (mode == 0) {
     rc = fill_zero(s, w.used, sizeof(int) * (size_t)num_pts);
     if (rc != MCCNN_OK) return rc;
-    // at most num_pts occupied cells; the kernel reads the true count on device
+    // at most num_pts occupied cells; the kernels read the true count on device.  The
+    // classes live in sel_scan, which is only filled after the passes.
+    MCCNN_DIM_SWITCH(num_dims, hipLaunchKernelGGL(cell_class_kernel<D>, dim3(grid), dim3(256), 0, s,
+                                                  w.num_cells_total, (const int64_t *)point_keys,
+                                                  num_cells, w.first_idx, w.sel_scan));
+    MCCNN_LAUNCH_CHECK();
     const unsigned wgrid = blocks_for(num_pts, 256 / kWave);
     for (int call = 0; call < (1 << num_dims); ++call) {
-      MCCNN_DIM_SWITCH(num_dims,
-                       hipLaunchKernelGGL(poisson_pass_kernel<D>, dim3(wgrid), dim3(256), 0, s,
-                                          num_pts, call, w.num_cells_total,
-                                          (const int64_t *)point_keys, num_cells,
-                                          (const int2 *)neighbors, ranges, w.first_idx, w.used));
+      hipLaunchKernelGGL(poisson_pass_kernel, dim3(wgrid), dim3(256), 0, s, num_pts, call,
+                         w.num_cells_total, w.sel_scan, (const int2 *)neighbors, ranges,
+                         w.first_idx, w.used);
       MCCNN_LAUNCH_CHECK();
     }
     hipLaunchKernelGGL(copy_i32_kernel, dim3(grid), dim3(256), 0, s, num_pts, w.used, w.sel_scan);
