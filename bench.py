@@ -341,6 +341,8 @@ def main():
                     help="run the product with the final weights inside the projection kernel")
     ap.add_argument("--no-cpu", action="store_true", help="skip the host-CPU baseline")
     ap.add_argument("--no-isolated", action="store_true", help="skip the isolated basis_proj case")
+    ap.add_argument("--no-sweep", action="store_true",
+                    help="skip the other two radii (0.02, 0.06) of the dense case")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run a 1 GiB device copy three times (reference point for the "
                          "FETCH_SIZE / WRITE_SIZE counters) and exit")
@@ -459,7 +461,7 @@ def main():
         torch.cuda.empty_cache()
         # the other two radii of the dense case's sweep (about 7 and 180 pairs per point)
         result["dense_radius_sweep"] = {}
-        for radius in (0.02, 0.06):
+        for radius in (() if args.no_sweep else (0.02, 0.06)):
             result["dense_radius_sweep"]["r=%.2f" % radius] = isolated_basis_proj(
                 torch, pc, synthetic, tfg_custom_ops, _lib, radius=radius, steps=3)
             torch.cuda.empty_cache()
