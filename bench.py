@@ -171,8 +171,10 @@ def cpu_baseline(synthetic, sample_points=60000):
 
 
 def kpconv_config5(torch, pc, layers, synthetic, _lib, steps=5):
-    """Rigid kernel-point convolution 128 -> 128, 15 kernel points (padded to 16),
-    linear correlation, fwd+bwd on the scene-scale geometry (configuration 5)."""
+    """Kernel-point convolution 128 -> 128, 15 kernel points (padded to 16), fwd+bwd
+    on the scene-scale geometry (configuration 5): rigid with the linear and the
+    Gaussian correlation (sigma = 0.3 r), and deformable (offsets from a rigid
+    convolution, scaled to a spread of 0.01 r) with its regularisation loss."""
     import numpy as np
     cfg = synthetic.config5()
     dev = lambda a: torch.as_tensor(np.ascontiguousarray(a)).cuda()
@@ -180,31 +182,50 @@ def kpconv_config5(torch, pc, layers, synthetic, _lib, steps=5):
     r = cfg["radius"]
     nbh = pc.Neighborhood(pc.Grid(cloud, r), r, cloud)
     N, M, C, CO = cloud._points.shape[0], nbh._neighbors.shape[0], cfg["c_in"], cfg["c_out"]
-    conv = layers.KPConv(C, CO, custom_kernel_points=cfg["kernel_points"] / 0.75,
-                         kp_interpolation="linear", seed=5)
     gen = torch.Generator(device="cuda").manual_seed(5)
     feats = torch.randn((N, C), device="cuda", generator=gen).requires_grad_(True)
     up = torch.randn((N, CO), device="cuda", generator=gen)
 
-    def step():
-        conv(feats, cloud, cloud, r, neighborhood=nbh).backward(up)
-        feats.grad = None
-        conv.weights.grad = None
+    def measure(conv, influence, regularised):
+        def step():
+            out = conv(feats, cloud, cloud, r, neighborhood=nbh, kernel_influence_dist=influence)
+            if regularised:
+                torch.autograd.backward([out, conv.regularization_loss()],
+                                        [up, torch.ones((), device="cuda")])
+            else:
+                out.backward(up)
+            feats.grad = None
+            for p in conv.parameters():
+                p.grad = None
 
-    for _ in range(2):
-        step()
-    torch.cuda.synchronize()
-    _lib.start_timing()
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        step()
-    torch.cuda.synchronize()
-    ms = (time.perf_counter() - t0) * 1e3 / steps
-    ops = {k.replace("_ordered", ""): round(sum(v) / steps, 3)
-           for k, v in _lib.collect_timing().items()}
-    return {"workload": "config 5: KPConv %d->%d, 15 kernel points, linear, radius %.2f, "
-                        "%d points, %d pairs, fwd+bwd" % (C, CO, r, N, M),
-            "ms_per_step": ms, "points_per_s": N / (ms * 1e-3), "ops_ms": ops}
+        for _ in range(2):
+            step()
+        torch.cuda.synchronize()
+        _lib.start_timing()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            step()
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - t0) * 1e3 / steps
+        ops = {k.replace("_ordered", ""): round(sum(v) / steps, 3)
+               for k, v in _lib.collect_timing().items()}
+        return {"ms_per_step": ms, "points_per_s": N / (ms * 1e-3), "ops_ms": ops}
+
+    kp = cfg["kernel_points"] / 0.75
+    res = {"workload": "config 5: KPConv %d->%d, 15 kernel points, radius %.2f, %d points, "
+                       "%d pairs, fwd+bwd" % (C, CO, r, N, M)}
+    res.update(measure(layers.KPConv(C, CO, custom_kernel_points=kp, kp_interpolation="linear",
+                                     seed=5), None, False))
+    res["gaussian"] = measure(layers.KPConv(C, CO, custom_kernel_points=kp,
+                                            kp_interpolation="gaussian", seed=5), 0.3 * r, False)
+    conv = layers.KPConv(C, CO, custom_kernel_points=kp, kp_interpolation="linear",
+                         deformable=True, seed=5)
+    with torch.no_grad():
+        conv.offset_weights.normal_(0.0, 1.0, generator=gen)
+        conv(feats, cloud, cloud, r, neighborhood=nbh)
+        conv.offset_weights.mul_(0.01 / float(conv._last[0].std()))
+    res["deformable_with_regularisation_loss"] = measure(conv, None, True)
+    return res
 
 
 def per_op_times(torch, pc, layers, synthetic, _lib, radius=0.04, reps=5):
