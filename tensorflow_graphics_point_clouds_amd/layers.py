@@ -819,8 +819,17 @@ class KPConv(torch.nn.Module):
 
         offsets = None
         if self.deformable:       # KPConv.py:317-392: offsets from a rigid convolution
-            rigid = _KPBasis.apply(None, *geometry, k, self._kind, sigma)
-            offsets = (project(rigid).reshape(-1, c * k) @ self._padded(self.offset_weights))
+            w_off = self._padded(self.offset_weights)
+            if self.transposed_grads and k in (16, 32):
+                # the rigid layer's kernels, output columns padded to a multiple of 16
+                cols = kp * d
+                w_off = torch.nn.functional.pad(w_off, (0, -cols % 16))
+                offsets = _KPConvRigidLayer.apply(w_off, features, neighborhood,
+                                                  torch.reciprocal(radii), self._kernel_points, k,
+                                                  self._kind, sigma)[:, :cols]
+            else:
+                rigid = _KPBasis.apply(None, *geometry, k, self._kind, sigma)
+                offsets = project(rigid).reshape(-1, c * k) @ w_off
             offsets = offsets.reshape(-1, kp, d).contiguous()
         self._last = (offsets, geometry, sigma)
         basis = _KPBasis.apply(offsets, *geometry, k, self._kind, sigma)
