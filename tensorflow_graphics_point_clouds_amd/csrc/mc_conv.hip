@@ -348,7 +348,8 @@ __global__ void __launch_bounds__(256) mc_conv_weight_grads16_kernel(
   // index order, so at any moment the device works on one compact window of the
   // (grid-ordered) centres and the feature rows of that window stay in L2.
   // (Giving each XCD its own contiguous eighth of the centres instead was measured
-  // on the scene-scale case, for this kernel and the projection: 12 % slower.)
+  // on the scene-scale case, for this kernel and the projection: 12 % slower; dealing
+  // groups of 4 to 64 consecutive blocks to the XCDs in turn: no different.)
   const int64_t first = wave_slot() * kGradRun;
   const int64_t last = first + kGradRun < n_out ? first + kGradRun : n_out;
   for (int64_t centre = first; centre < last; ++centre) {
