@@ -33,7 +33,7 @@ int fill_zero(hipStream_t stream, void *ptr, size_t bytes) {
 }
 
 // ------------------------------------------------------------ prefix sum ----
-// Three launches, no inter-block waiting: (1) each block of kScanTile items
+// Long inputs take three launches, no inter-block waiting: (1) each block of kScanTile items
 // writes its sum, (2) one block scans the block sums, (3) each block rescans its
 // tile with the carried-in offset.  The scanned values are int32 (pair counts are
 // int32 in the op contract); tile sums and the grand total are formed in 64 bits
@@ -139,11 +139,45 @@ __global__ void __launch_bounds__(kScanThreads) scan_apply_kernel(
   }
 }
 
+// Short inputs: one block walks the tiles in order and carries the running total,
+// one launch instead of three (small clouds are bound by launches, not by bytes).
+constexpr int64_t kScanSingleBlockMax = 16 * kScanTile;
+
+__global__ void __launch_bounds__(kScanThreads) scan_single_block_kernel(int64_t n, int *counts,
+                                                                         int64_t *total_dev) {
+  long long carry = 0;
+  for (int64_t tile = 0; tile < n; tile += kScanTile) {
+    const int64_t base = tile + (int64_t)threadIdx.x * kScanItems;
+    int v[kScanItems];
+    long long s = 0;
+#pragma unroll
+    for (int k = 0; k < kScanItems; ++k) {
+      v[k] = base + k < n ? counts[base + k] : 0;
+      s += v[k];
+    }
+    long long total;
+    long long run = carry + block_exclusive_scan_i64(s, &total);
+#pragma unroll
+    for (int k = 0; k < kScanItems; ++k) {
+      run += v[k];
+      if (base + k < n) counts[base + k] = saturate_i32(run);
+    }
+    carry += total;
+  }
+  if (threadIdx.x == 0) *total_dev = carry;
+}
+
 int inclusive_scan_i32(hipStream_t stream, int64_t n, int *counts, int *block_sums,
                        int64_t *total_dev) {
   const int nb = (int)((n + kScanTile - 1) / kScanTile);
   if (nb == 0) {
     return fill_zero(stream, total_dev, sizeof(int64_t));
+  }
+  if (n <= kScanSingleBlockMax) {
+    hipLaunchKernelGGL(scan_single_block_kernel, dim3(1), dim3(kScanThreads), 0, stream, n,
+                       counts, total_dev);
+    MCCNN_LAUNCH_CHECK();
+    return MCCNN_OK;
   }
   hipLaunchKernelGGL(scan_tile_sums_kernel, dim3(nb), dim3(kScanThreads), 0, stream, n, counts,
                      block_sums);
