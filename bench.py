@@ -165,9 +165,58 @@ def cpu_baseline(synthetic, sample_points=60000):
             break
     dt = (time.perf_counter() - t0) / reps
     cores = int(os.environ.get("OMP_NUM_THREADS", "0")) or len(os.sched_getaffinity(0))
+
+    # configuration 1, the case the reference's own CPU path is quoted on: 2 x 1024
+    # points, grid + neighbours + densities + one MCConv 8 -> 16 forward
+    c1 = synthetic.config1()
+    r1 = np.float32(c1["radius"])
+
+    def c1_step():
+        g1 = orc.Grid(c1["points"], c1["batch_ids"], c1["batch_size"], r1)
+        n1 = orc.Neighborhood(g1, r1, c1["points"], c1["batch_ids"])
+        return orc.mc_conv_forward(c1["features"], c1["points"], c1["points"], n1,
+                                   n1.pdf_per_pair(c1["bandwidth"]), c1["weights"], c1["biases"],
+                                   c1["final_weights"], r1)
+
+    c1_step()
+    t0 = time.perf_counter()
+    for _ in range(10):
+        c1_step()
+    c1_ms = (time.perf_counter() - t0) * 100.0
     return {"value": n / dt, "unit": "points/s", "cores": cores, "kind": "port",
             "sample": "one config-3 cloud cut to %d points (%d pairs), %d fwd+bwd passes of "
-                      "the C/OpenMP oracle with numpy GEMMs" % (n, len(ids), reps)}
+                      "the C/OpenMP oracle with numpy GEMMs" % (n, len(ids), reps),
+            "config1_forward_with_build_ms": c1_ms,
+            "config1_points_per_s": len(c1["points"]) / (c1_ms * 1e-3)}
+
+
+def config1_forward(torch, pc, layers, synthetic, steps=50):
+    """Configuration 1 on the GPU: 2 x 1024 points, grid + neighbours + densities +
+    one MCConv 8 -> 16 forward, everything rebuilt every step."""
+    import numpy as np
+    cfg = synthetic.config1()
+    dev = lambda a: torch.as_tensor(np.ascontiguousarray(a)).cuda()
+    pts, bids, feats = dev(cfg["points"]), dev(cfg["batch_ids"]), dev(cfg["features"])
+    conv = layers.MCConv(8, 16, 3, num_mlps=1, mlp_size=[16], non_linearity_type="relu",
+                         weights=dev(cfg["weights"]), biases=dev(cfg["biases"]),
+                         final_weights=dev(cfg["final_weights"]))
+
+    def step():
+        cloud = pc.PointCloud(pts, bids, cfg["batch_size"])
+        with torch.no_grad():
+            return conv(feats, cloud, cloud, cfg["radius"], bandwidth=cfg["bandwidth"])
+
+    for _ in range(5):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / steps
+    return {"workload": "config 1: 2 x 1024 points, r=0.1, MCConv 8->16, K=16, forward only, "
+                        "grid, neighbourhood and densities rebuilt every step",
+            "ms_per_step": ms, "points_per_s": int(pts.shape[0]) / (ms * 1e-3)}
 
 
 def kpconv_config5(torch, pc, layers, synthetic, _lib, steps=5):
@@ -226,6 +275,55 @@ def kpconv_config5(torch, pc, layers, synthetic, _lib, steps=5):
         conv.offset_weights.mul_(0.01 / float(conv._last[0].std()))
     res["deformable_with_regularisation_loss"] = measure(conv, None, True)
     return res
+
+
+def config2_network(torch, pc, layers, synthetic, steps=20):
+    """Configuration 2: 16 x 1024 points on random primitives, cell-average hierarchy
+    at radii 0.1 / 0.2 / 0.4, one Monte-Carlo convolution per level (3 -> 64 -> 128 ->
+    256, convolution radius 1.5 x the level's), fwd+bwd; once with the hierarchy,
+    grids, neighbourhoods and densities rebuilt every step, once with them reused."""
+    import numpy as np
+    cfg = synthetic.config2()
+    dev = lambda a: torch.as_tensor(np.ascontiguousarray(a)).cuda()
+    pts, bids, batch = dev(cfg["points"]), dev(cfg["batch_ids"]), cfg["batch_size"]
+    widths = cfg["channels"]
+    convs = [layers.MCConv(widths[i], widths[i + 1], 3, num_mlps=1, mlp_size=[16],
+                           non_linearity_type="leaky_relu", seed=i) for i in range(3)]
+    params = [p for c in convs for p in c.parameters()]
+    state = {}
+
+    def step(build):
+        if build or "hier" not in state:
+            state["hier"] = pc.PointHierarchy(pc.PointCloud(pts, bids, batch), cfg["radii"],
+                                              "cell average")
+            state["nbh"] = [None] * 3
+        hier, feat = state["hier"], pts
+        for level, r in enumerate(cfg["radii"]):
+            feat = torch.relu(convs[level](feat, hier[level], hier[level + 1], 1.5 * r,
+                                           bandwidth=0.2, neighborhood=state["nbh"][level]))
+            if not build:
+                state["nbh"][level] = convs[level].last_neighborhood
+        feat.sum().backward()
+        for p in params:
+            p.grad = None
+
+    def timed(build):
+        for _ in range(3):
+            step(build)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            step(build)
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e3 / steps
+
+    n = int(pts.shape[0])
+    with_build = timed(True)
+    reused = timed(False)
+    return {"workload": "config 2: 16 x 1024 points, 3-level cell-average hierarchy, MCConv "
+                        "3->64->128->256, fwd+bwd",
+            "ms_per_step_with_build": with_build, "points_per_s_with_build": n / (with_build * 1e-3),
+            "ms_per_step_prebuilt": reused, "points_per_s_prebuilt": n / (reused * 1e-3)}
 
 
 def per_op_times(torch, pc, layers, synthetic, _lib, radius=0.04, reps=5):
@@ -489,6 +587,8 @@ def main():
         result["per_op_dense_case"] = per_op_times(torch, pc, layers, synthetic, _lib)
         torch.cuda.empty_cache()
         result["kpconv_config5"] = kpconv_config5(torch, pc, layers, synthetic, _lib)
+        result["config2_network"] = config2_network(torch, pc, layers, synthetic)
+        result["config1_forward"] = config1_forward(torch, pc, layers, synthetic)
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(synthetic)
     else:
