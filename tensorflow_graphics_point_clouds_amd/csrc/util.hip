@@ -71,8 +71,9 @@ __device__ __forceinline__ int saturate_i32(long long v) {
 }
 
 // 64-bit counterpart of block_exclusive_scan for the sums of whole tiles.
+template <int kThreads = kScanThreads>
 __device__ __forceinline__ long long block_exclusive_scan_i64(long long v, long long *total) {
-  __shared__ long long wave_sums[kScanThreads / kWave];
+  __shared__ long long wave_sums[kThreads / kWave];
   const int lane = lane_id(), wave = threadIdx.x / kWave;
   long long incl = v;
 #pragma unroll
@@ -84,7 +85,7 @@ __device__ __forceinline__ long long block_exclusive_scan_i64(long long v, long 
   __syncthreads();
   long long carry = 0, sum = 0;
 #pragma unroll
-  for (int w = 0; w < kScanThreads / kWave; ++w) {
+  for (int w = 0; w < kThreads / kWave; ++w) {
     if (w < wave) carry += wave_sums[w];
     sum += wave_sums[w];
   }
@@ -141,12 +142,14 @@ __global__ void __launch_bounds__(kScanThreads) scan_apply_kernel(
 
 // Short inputs: one block walks the tiles in order and carries the running total,
 // one launch instead of three (small clouds are bound by launches, not by bytes).
-constexpr int64_t kScanSingleBlockMax = 16 * kScanTile;
+constexpr int kScanSingleThreads = 1024;
+constexpr int kScanSingleTile = kScanSingleThreads * kScanItems;
+constexpr int64_t kScanSingleBlockMax = 4 * kScanSingleTile;
 
-__global__ void __launch_bounds__(kScanThreads) scan_single_block_kernel(int64_t n, int *counts,
-                                                                         int64_t *total_dev) {
+__global__ void __launch_bounds__(kScanSingleThreads) scan_single_block_kernel(
+    int64_t n, int *counts, int64_t *total_dev) {
   long long carry = 0;
-  for (int64_t tile = 0; tile < n; tile += kScanTile) {
+  for (int64_t tile = 0; tile < n; tile += kScanSingleTile) {
     const int64_t base = tile + (int64_t)threadIdx.x * kScanItems;
     int v[kScanItems];
     long long s = 0;
@@ -156,7 +159,7 @@ __global__ void __launch_bounds__(kScanThreads) scan_single_block_kernel(int64_t
       s += v[k];
     }
     long long total;
-    long long run = carry + block_exclusive_scan_i64(s, &total);
+    long long run = carry + block_exclusive_scan_i64<kScanSingleThreads>(s, &total);
 #pragma unroll
     for (int k = 0; k < kScanItems; ++k) {
       run += v[k];
@@ -174,7 +177,7 @@ int inclusive_scan_i32(hipStream_t stream, int64_t n, int *counts, int *block_su
     return fill_zero(stream, total_dev, sizeof(int64_t));
   }
   if (n <= kScanSingleBlockMax) {
-    hipLaunchKernelGGL(scan_single_block_kernel, dim3(1), dim3(kScanThreads), 0, stream, n,
+    hipLaunchKernelGGL(scan_single_block_kernel, dim3(1), dim3(kScanSingleThreads), 0, stream, n,
                        counts, total_dev);
     MCCNN_LAUNCH_CHECK();
     return MCCNN_OK;
