@@ -92,6 +92,10 @@ __global__ void __launch_bounds__(256) poisson_pass_kernel(
       // also writes the whole L2 back, once per selected point; other wavefronts only
       // need the selections in the next launch.
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+      // (the compiler relies on the per-CU cache serving a workgroup's accesses in
+      // order and emits no wait for this scope; wait for the store's acknowledgement
+      // anyway, it costs one round trip per selected point)
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       __builtin_amdgcn_wave_barrier();
       __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
     }
