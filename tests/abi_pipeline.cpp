@@ -5,7 +5,7 @@
 // here).  Integer outputs must agree exactly, floats within 1e-5 of the magnitude
 // sum.  Prints one line per stage and exits non-zero on the first mismatch.
 //
-// Built by tests/Makefile (from __graft_entry__.build()); run by tests/test_abi_cpp_pipeline.py.
+// Built by tests/Makefile (from __graft_entry__.build()); run by tests/test_zz_abi_cpp_pipeline.py.
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
