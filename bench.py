@@ -462,6 +462,9 @@ def main():
     ap.add_argument("--no-isolated", action="store_true", help="skip the isolated basis_proj case")
     ap.add_argument("--no-sweep", action="store_true",
                     help="skip the other two radii (0.02, 0.06) of the dense case")
+    ap.add_argument("--small-configs", action="store_true",
+                    help="also time configurations 1 (2 x 1024 points, forward) and 2 (16 x 1024 "
+                         "points, three-level network, fwd+bwd)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run a 1 GiB device copy three times (reference point for the "
                          "FETCH_SIZE / WRITE_SIZE counters) and exit")
@@ -587,6 +590,9 @@ def main():
         result["per_op_dense_case"] = per_op_times(torch, pc, layers, synthetic, _lib)
         torch.cuda.empty_cache()
         result["kpconv_config5"] = kpconv_config5(torch, pc, layers, synthetic, _lib)
+    if args.small_configs:
+        # (not in the default run: these launch the layer's kernels on tiny shapes, which
+        # would blur the per-kernel averages of a profile of the default command)
         result["config2_network"] = config2_network(torch, pc, layers, synthetic)
         result["config1_forward"] = config1_forward(torch, pc, layers, synthetic)
     if not args.no_cpu:
