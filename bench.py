@@ -326,6 +326,39 @@ def config2_network(torch, pc, layers, synthetic, steps=20):
             "ms_per_step_prebuilt": reused, "points_per_s_prebuilt": n / (reused * 1e-3)}
 
 
+def pointconv_config3(torch, pc, layers, synthetic, _lib, steps=5):
+    """PointConv 64 -> 64 with 32 hidden units (the reference's default) on the clouds
+    of configuration 3, fwd+bwd, neighbourhood and densities prebuilt."""
+    cfg, cloud = build_scene(torch, pc, synthetic, 1.0)
+    r = cfg["radius"]
+    nbh = pc.Neighborhood(pc.Grid(cloud, r), r, cloud)
+    n = int(cloud._points.shape[0])
+    conv = layers.PointConv(64, 64, 3, size_hidden=32)
+    gen = torch.Generator(device="cuda").manual_seed(6)
+    feats = torch.randn((n, 64), device="cuda", generator=gen).requires_grad_(True)
+    up = torch.randn((n, 64), device="cuda", generator=gen)
+
+    def step():
+        conv(feats, cloud, cloud, r, neighborhood=nbh).backward(up)
+        feats.grad = None
+        for p in conv.parameters():
+            p.grad = None
+
+    for _ in range(2):
+        step()
+    torch.cuda.synchronize()
+    _lib.start_timing()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / steps
+    ops = {k: round(sum(v) / steps, 3) for k, v in _lib.collect_timing().items()}
+    return {"workload": "PointConv 64->64, 32 hidden units, radius %.2f, %d points, %d pairs, "
+                        "fwd+bwd" % (r, n, int(nbh._neighbors.shape[0])),
+            "ms_per_step": ms, "points_per_s": n / (ms * 1e-3), "ops_ms": ops}
+
+
 def per_op_times(torch, pc, layers, synthetic, _lib, radius=0.04, reps=5):
     """Every op of the path on the dense case (4 x 200k uniform points, radius
     0.04): average milliseconds from HIP events around each C-ABI call, with
@@ -462,9 +495,10 @@ def main():
     ap.add_argument("--no-isolated", action="store_true", help="skip the isolated basis_proj case")
     ap.add_argument("--no-sweep", action="store_true",
                     help="skip the other two radii (0.02, 0.06) of the dense case")
-    ap.add_argument("--small-configs", action="store_true",
+    ap.add_argument("--extra-configs", action="store_true",
                     help="also time configurations 1 (2 x 1024 points, forward) and 2 (16 x 1024 "
-                         "points, three-level network, fwd+bwd)")
+                         "points, three-level network, fwd+bwd) and PointConv on the scene-scale "
+                         "clouds")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run a 1 GiB device copy three times (reference point for the "
                          "FETCH_SIZE / WRITE_SIZE counters) and exit")
@@ -590,11 +624,12 @@ def main():
         result["per_op_dense_case"] = per_op_times(torch, pc, layers, synthetic, _lib)
         torch.cuda.empty_cache()
         result["kpconv_config5"] = kpconv_config5(torch, pc, layers, synthetic, _lib)
-    if args.small_configs:
+    if args.extra_configs:
         # (not in the default run: these launch the layer's kernels on tiny shapes, which
         # would blur the per-kernel averages of a profile of the default command)
         result["config2_network"] = config2_network(torch, pc, layers, synthetic)
         result["config1_forward"] = config1_forward(torch, pc, layers, synthetic)
+        result["pointconv_config3"] = pointconv_config3(torch, pc, layers, synthetic, _lib)
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(synthetic)
     else:

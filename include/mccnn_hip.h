@@ -445,6 +445,47 @@ int mccnn_mc_conv_project_grads(
     float *pair_rows_workspace, float *feature_grads_out,
     float *weight_grads_out, float *bias_grads_out);
 
+/* The weights-only backward of the fused projection that also returns the gradient
+ * with respect to every pair's scale 1/pdf[m]:
+ *   pair_scale_grads_out [K/16, M]: slab s, pair m = sum over the basis columns
+ *   16 s .. 16 s + 15 of dbasis[m, k] * act(z[m, k])
+ * (the slabs are summed by the consumer).  A layer whose per-pair density is itself
+ * a function of trainable parameters (PointConv.py:176-190) needs it; shapes as
+ * for mccnn_mc_conv_weight_grads_supported.  No counterpart among the reference's
+ * ops. */
+int mccnn_mc_conv_weight_and_scale_grads(
+    mccnn_stream_t stream, int num_dims, int64_t num_pts, const float *points_in,
+    int num_features, const float *features, int64_t num_samples,
+    const float *points_out, int64_t num_neighbors, const int32_t *neighbors,
+    const int32_t *ranges, const float *inv_radii, int num_basis, int num_mlps,
+    int activation, const float *weights, const float *biases, const float *pdf,
+    const float *in_grads, void *workspace, size_t workspace_bytes,
+    float *weight_grads_out, float *bias_grads_out, float *pair_scale_grads_out);
+
+/* Density transform of PointConv (pylib/pc/layers/PointConv.py:176-190), per pair:
+ *   rel = pdf[point] / max_pdf[centre],
+ *   density_out[m] = biases_2 + sum_j weights_2[j] * relu(rel * weights_1[j] + biases_1[j]),
+ * 16 hidden units.  neighbors[m][point_column] indexes pdf, the other column
+ * max_pdf (point_column 1 serves a transposed pair table).  density_out takes the
+ * place of pdf in the projection entry points above.  _grads turns the pair scale
+ * gradients of mccnn_mc_conv_weight_and_scale_grads into param_grads_out [49]:
+ * weights_1 [16], biases_1 [16], weights_2 [16], biases_2.  The reference forms
+ * the [M, 16] hidden layer with TensorFlow ops. */
+int mccnn_pointconv_density(mccnn_stream_t stream, int64_t num_neighbors,
+                            const int32_t *neighbors, int point_column,
+                            const float *pdf, const float *max_pdf,
+                            const float *weights_1, const float *biases_1,
+                            const float *weights_2, const float *biases_2,
+                            float *density_out);
+size_t mccnn_pointconv_density_grads_workspace_bytes(int64_t num_neighbors);
+int mccnn_pointconv_density_grads(
+    mccnn_stream_t stream, int64_t num_neighbors, const int32_t *neighbors,
+    int point_column, const float *pdf, const float *max_pdf,
+    const float *weights_1, const float *biases_1, const float *weights_2,
+    const float *biases_2, const float *density, int num_slabs,
+    const float *pair_scale_grads, void *workspace, size_t workspace_bytes,
+    float *param_grads_out);
+
 /* Rigid kernel-point convolution projection (KPConv.py:193-224): kp_basis
  * followed by basis_proj in one kernel, the correlation weights
  *   kind 0: max(1 - d/sigma, 0),  kind 1: exp(-(d/(sigma/3))^2),

@@ -316,7 +316,7 @@ template <int C, int D, int kAct, int KT>
 __global__ void __launch_bounds__(256) mc_conv_weight_grads16_kernel(
     int64_t n_out, const float *__restrict__ feat, const int2 *__restrict__ nbrs,
     const int *__restrict__ ranges, McParams<D> p, const float *__restrict__ in_grad,
-    float *__restrict__ partials) {
+    float *__restrict__ partials, float *__restrict__ pair_sums, int64_t pair_stride) {
   constexpr int K = kFusedK;               // a block works on basis columns k0 .. k0 + 15
   constexpr int num_basis = kFusedK * KT;  // of the KT * 16 the layer has
   constexpr int kQuarterC = C / 4;
@@ -326,6 +326,7 @@ __global__ void __launch_bounds__(256) mc_conv_weight_grads16_kernel(
   const int lane = lane_id(), wave = threadIdx.x / kWave;
   const int quarter = lane >> 4, col = lane & 15;
   const int k0 = blockIdx.y * K;
+  if (pair_sums) pair_sums += (int64_t)blockIdx.y * pair_stride;   // [K / 16][M]
   if (threadIdx.x < K) {
     float w[3] = {0.0f, 0.0f, 0.0f}, bias;
     load_weight_column<D>(p, k0 + threadIdx.x, w, &bias);
@@ -393,6 +394,7 @@ __global__ void __launch_bounds__(256) mc_conv_weight_grads16_kernel(
         for (int s = 0; s < kQuarterC; ++s)
           acc = __builtin_amdgcn_mfma_f32_16x16x4f32(gk[s], f.v[s], acc, 0, 0, 0);
         // acc[r] = dbasis[pair col][k = 4*quarter + r]
+        float along = 0.0f;                 // sum_k dbasis * act(z) over this lane's columns
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           const float4 wr = wlds[4 * quarter + r];
@@ -402,6 +404,13 @@ __global__ void __launch_bounds__(256) mc_conv_weight_grads16_kernel(
           dw[r][0] += geo.x * dz;
           dw[r][1] += geo.y * dz;
           if (D > 2) dw[r][2] += geo.z * dz;
+          if (pair_sums) along += acc[r] * act_fwd(kAct, z);
+        }
+        if (pair_sums) {
+          // the gradient with respect to the pair's scale 1/pdf, over the block's 16 columns
+          along += __shfl_xor(along, 16, kWave);
+          along += __shfl_xor(along, 32, kWave);
+          if (quarter == 0 && 16 * t + col < cnt) pair_sums[m0 + 16 * t + col] = along;
         }
         f = fn;
       }
@@ -466,20 +475,24 @@ template <int C, int D, int ACT>
 static int launch_fused_backward(hipStream_t s, int64_t num_samples, const float *features,
                                  const int2 *nb, const int *ranges, const McParams<D> &prm,
                                  int num_basis, const float *in_grads, float *feature_grads_out,
-                                 float *pair_rows, float *workspace, bool want_dfeat) {
+                                 float *pair_rows, float *workspace, bool want_dfeat,
+                                 float *pair_sums, int64_t num_neighbors) {
   const dim3 grid((unsigned)grad_blocks(num_samples), (unsigned)(num_basis / kFusedK));
   switch (num_basis / kFusedK) {
     case 1:
       hipLaunchKernelGGL((mc_conv_weight_grads16_kernel<C, D, ACT, 1>), grid, dim3(256), 0, s,
-                         num_samples, features, nb, ranges, prm, in_grads, workspace);
+                         num_samples, features, nb, ranges, prm, in_grads, workspace, pair_sums,
+                         num_neighbors);
       break;
     case 2:
       hipLaunchKernelGGL((mc_conv_weight_grads16_kernel<C, D, ACT, 2>), grid, dim3(256), 0, s,
-                         num_samples, features, nb, ranges, prm, in_grads, workspace);
+                         num_samples, features, nb, ranges, prm, in_grads, workspace, pair_sums,
+                         num_neighbors);
       break;
     default:
       hipLaunchKernelGGL((mc_conv_weight_grads16_kernel<C, D, ACT, 4>), grid, dim3(256), 0, s,
-                         num_samples, features, nb, ranges, prm, in_grads, workspace);
+                         num_samples, features, nb, ranges, prm, in_grads, workspace, pair_sums,
+                         num_neighbors);
       break;
   }
   if (want_dfeat)        // the feature half keeps no running sums: one wavefront per centre
@@ -601,7 +614,7 @@ extern "C" size_t mccnn_mc_conv_project_grads_workspace_bytes(int num_dims, int 
   return align256(sizeof(float) * (size_t)grad_blocks(num_samples) * (num_dims + 1) * num_basis);
 }
 
-extern "C" int mccnn_mc_conv_project_grads(
+static int project_grads(
     mccnn_stream_t stream, int num_dims, int64_t num_pts, const float *points_in,
     int num_features, const float *features, int64_t num_samples, const float *points_out,
     int64_t num_neighbors, const int32_t *neighbors, const int32_t *ranges,
@@ -609,7 +622,7 @@ extern "C" int mccnn_mc_conv_project_grads(
     const float *biases, const float *pdf, const float *in_grads, void *workspace,
     size_t workspace_bytes, const int32_t *point_ranges, const int32_t *pair_order,
     float *pair_rows_workspace, float *feature_grads_out, float *weight_grads_out,
-    float *bias_grads_out) {
+    float *bias_grads_out, float *pair_sums) {
   float *pair_rows = pair_rows_workspace;
   const bool gathered = pair_rows != nullptr;
   MCCNN_REQUIRE(!gathered || (point_ranges && pair_order),
@@ -648,7 +661,8 @@ extern "C" int mccnn_mc_conv_project_grads(
     MCCNN_ACT_SWITCH(activation,                                                               \
                      rc = (launch_fused_backward<C_, D_, ACT>(                                 \
                          s, num_samples, features, nb, ranges, prm, num_basis, in_grads,       \
-                         feature_grads_out, pair_rows, (float *)workspace, want_dfeat)));      \
+                         feature_grads_out, pair_rows, (float *)workspace, want_dfeat,         \
+                         pair_sums, num_neighbors)));                                          \
   }
 #define MCCNN_FUSED_BWD_D(C_) \
   if (num_dims == 3) MCCNN_FUSED_BWD(C_, 3) else MCCNN_FUSED_BWD(C_, 2)
@@ -671,6 +685,39 @@ extern "C" int mccnn_mc_conv_project_grads(
     return launch_dfeat_gather(s, num_pts, num_features, point_ranges, pair_order, pair_rows,
                                feature_grads_out);
   return MCCNN_OK;
+}
+
+extern "C" int mccnn_mc_conv_project_grads(
+    mccnn_stream_t stream, int num_dims, int64_t num_pts, const float *points_in,
+    int num_features, const float *features, int64_t num_samples, const float *points_out,
+    int64_t num_neighbors, const int32_t *neighbors, const int32_t *ranges,
+    const float *inv_radii, int num_basis, int num_mlps, int activation, const float *weights,
+    const float *biases, const float *pdf, const float *in_grads, void *workspace,
+    size_t workspace_bytes, const int32_t *point_ranges, const int32_t *pair_order,
+    float *pair_rows_workspace, float *feature_grads_out, float *weight_grads_out,
+    float *bias_grads_out) {
+  return project_grads(stream, num_dims, num_pts, points_in, num_features, features, num_samples,
+                       points_out, num_neighbors, neighbors, ranges, inv_radii, num_basis,
+                       num_mlps, activation, weights, biases, pdf, in_grads, workspace,
+                       workspace_bytes, point_ranges, pair_order, pair_rows_workspace,
+                       feature_grads_out, weight_grads_out, bias_grads_out, nullptr);
+}
+
+extern "C" int mccnn_mc_conv_weight_and_scale_grads(
+    mccnn_stream_t stream, int num_dims, int64_t num_pts, const float *points_in,
+    int num_features, const float *features, int64_t num_samples, const float *points_out,
+    int64_t num_neighbors, const int32_t *neighbors, const int32_t *ranges,
+    const float *inv_radii, int num_basis, int num_mlps, int activation, const float *weights,
+    const float *biases, const float *pdf, const float *in_grads, void *workspace,
+    size_t workspace_bytes, float *weight_grads_out, float *bias_grads_out,
+    float *pair_scale_grads_out) {
+  MCCNN_REQUIRE(pair_scale_grads_out || num_neighbors == 0,
+                "mc_conv_weight_and_scale_grads received a null output");
+  return project_grads(stream, num_dims, num_pts, points_in, num_features, features, num_samples,
+                       points_out, num_neighbors, neighbors, ranges, inv_radii, num_basis,
+                       num_mlps, activation, weights, biases, pdf, in_grads, workspace,
+                       workspace_bytes, nullptr, nullptr, nullptr, nullptr, weight_grads_out,
+                       bias_grads_out, pair_scale_grads_out);
 }
 
 extern "C" int mccnn_kp_conv_project(mccnn_stream_t stream, int num_dims, int64_t num_pts,

@@ -489,6 +489,100 @@ def _layer_padding(c, f, num_mlps):
     return c_pad, g_pad
 
 
+class _PointConvLayer(torch.autograd.Function):
+    """PointConv (PointConv.py:143-202) on the neighbourhood's grid-ordered view with
+    the kernels of the Monte-Carlo convolution: the transformed density of a pair,
+        y = mlp(pdf[point] / max pdf of the centre's neighbourhood),
+    is computed once per pair (forward and transposed order) and takes the place
+    of the density in the fused projection, which runs on the unscaled offsets
+    (unit radii).  Backward as for the Monte-Carlo convolution (transposed
+    convolution for the features, no scatter); the gradient of the four density
+    parameters comes from the per-pair gradient of the scale 1/y that the
+    kernel-MLP backward returns beside the weight gradients."""
+
+    @staticmethod
+    def forward(ctx, weights, biases, final_weights, pw1, pb1, pw2, pb2, features,
+                neighborhood, act):
+        view = neighborhood.sorted_view()
+        dev = features.device
+        per_point = neighborhood._pdf_per_point.detach()
+        m, dims = view.table.shape[0], weights.shape[1]
+        max_pdf = torch.empty((view.ranges.shape[0], 1), dtype=_F32, device=dev)
+        _lib.call("local_pool", stream(), cint(0), i64(per_point.shape[0]), cint(1),
+                  ptr(per_point, _F32), i64(m), ptr(view.table, _I32),
+                  i64(view.ranges.shape[0]), ptr(view.ranges, _I32), ptr(max_pdf))
+        mlp = [t.detach().reshape(-1).contiguous() for t in (pw1, pb1, pw2, pb2)]
+
+        def density(table, point_column):
+            out = torch.empty(m, dtype=_F32, device=dev)
+            _lib.call("pointconv_density", stream(), i64(m), ptr(table, _I32), cint(point_column),
+                      ptr(per_point, _F32), ptr(max_pdf, _F32), ptr(mlp[0], _F32),
+                      ptr(mlp[1], _F32), ptr(mlp[2], _F32), ptr(mlp[3], _F32), ptr(out))
+            return out
+
+        y = density(view.table, 0)
+        y_t = density(view.table_t, 1)
+        ones = torch.ones(dims, dtype=_F32, device=dev)
+        feats = _gather_rows(features, view.point_rows)
+        proj = _mc_project(weights, biases, feats, view.points_in, view.points_out, view.table,
+                           view.ranges, ones, y, act, view.centre_rows)
+        with _lib.region("gemm_out"):
+            out = proj.reshape(proj.shape[0], -1) @ final_weights[0]
+        ctx.save_for_backward(weights, biases, final_weights, feats, features, per_point, max_pdf,
+                              y, y_t, ones, *mlp)
+        ctx.neighborhood, ctx.act = neighborhood, act
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        (weights, biases, final_weights, feats, features, per_point, max_pdf, y, y_t, ones,
+         w1, b1, w2, b2) = ctx.saved_tensors
+        view = ctx.neighborhood.sorted_view()
+        dev = feats.device
+        _, dims, k = weights.shape
+        n, c, m = view.ranges.shape[0], feats.shape[1], view.table.shape[0]
+        dense = final_weights[0]                                      # [C*K, F]
+        f = dense.shape[1]
+        if view.centre_order is not None:
+            dout = _gather_rows(dout, view.centre_rows)
+        else:
+            dout = dout.contiguous()
+        # kernel-MLP gradients and, per pair, the gradient of the scale 1/y
+        dproj = _projection_grad_product(dout, dense)
+        L = _lib.lib()
+        ws = _lib.workspace(L.mccnn_mc_conv_project_grads_workspace_bytes(
+            cint(dims), cint(k), i64(n)), dev)
+        dw, db = torch.empty_like(weights), torch.empty_like(biases)
+        slabs = k // 16
+        scale_grads = torch.empty((slabs, m), dtype=_F32, device=dev)
+        _lib.call("mc_conv_weight_and_scale_grads", stream(), cint(dims), i64(feats.shape[0]),
+                  ptr(view.points_in, _F32), cint(c), ptr(feats, _F32), i64(n),
+                  ptr(view.points_out, _F32), i64(m), ptr(view.table, _I32),
+                  ptr(view.ranges, _I32), ptr(ones, _F32), cint(k), cint(1), cint(ctx.act),
+                  ptr(weights, _F32), ptr(biases, _F32), ptr(y, _F32), ptr(dproj, _F32),
+                  ptr(ws), _lib.csize(ws.numel()), ptr(dw), ptr(db), ptr(scale_grads))
+        del dproj
+        ws2 = _lib.workspace(L.mccnn_pointconv_density_grads_workspace_bytes(i64(m)), dev)
+        dmlp = torch.empty(49, dtype=_F32, device=dev)
+        _lib.call("pointconv_density_grads", stream(), i64(m), ptr(view.table, _I32), cint(0),
+                  ptr(per_point, _F32), ptr(max_pdf, _F32), ptr(w1, _F32), ptr(b1, _F32),
+                  ptr(w2, _F32), ptr(b2, _F32), ptr(y, _F32), cint(slabs),
+                  ptr(scale_grads, _F32), ptr(ws2), _lib.csize(ws2.numel()), ptr(dmlp))
+        # feature and final-weight gradients from the transposed convolution
+        q = _mc_project(weights, biases, dout, view.points_out, view.points_in, view.table_t,
+                        view.ranges_t, -ones, y_t, ctx.act, view.point_rows)
+        q = q.reshape(q.shape[0], f * k)
+        dfeat = None
+        if ctx.needs_input_grad[7]:
+            w_t = dense.reshape(c, k, f).permute(2, 1, 0).reshape(f * k, c)
+            with _lib.region("gemm_dfeat"):
+                dfeat = q @ w_t
+        ddense = _weight_grad_product(features, q).reshape(c, f, k).permute(0, 2, 1)
+        dfinal = ddense.reshape(1, c * k, f)
+        return (dw, db, dfinal, dmlp[0:16].reshape(1, 16), dmlp[16:32].reshape(1, 16),
+                dmlp[32:48].reshape(16, 1), dmlp[48:49].reshape(1, 1), dfeat, None, None)
+
+
 class PointConv(torch.nn.Module):
     """PointConv-style Monte-Carlo convolution (pylib/pc/layers/PointConv.py:34-292):
     one kernel MLP with a single hidden layer on the unscaled point offsets, the
@@ -497,8 +591,9 @@ class PointConv(torch.nn.Module):
 
     def __init__(self, num_features_in, num_features_out, num_dims, size_hidden=32,
                  non_linearity_type="relu", device="cuda", seed=0, weights=None, biases=None,
-                 final_weights=None, pdf_weights=None, pdf_biases=None):
+                 final_weights=None, pdf_weights=None, pdf_biases=None, fused=True):
         super().__init__()
+        self.fused = fused
         if size_hidden not in (8, 16, 32):
             raise ValueError("size_hidden must be 8, 16 or 32")
         self._num_features_in, self._num_features_out = num_features_in, num_features_out
@@ -533,6 +628,29 @@ class PointConv(torch.nn.Module):
                              bandwidth)
         return point_cloud_out.format_output(out, return_sorted, return_padded)
 
+    def _convolve_on_view(self, features, neighborhood, bandwidth):
+        """The fused path on the grid-ordered view (channels zero-padded as for the
+        Monte-Carlo convolution); None if the shape is out of its reach."""
+        d, c, f, h = (self._num_dims, self._num_features_in, self._num_features_out,
+                      self._size_hidden)
+        pad = _layer_padding(c, f, 1)
+        if not self.fused or h not in (16, 32) or d not in (2, 3) or pad is None:
+            return None
+        if neighborhood.point_pdf(bandwidth=bandwidth, mode=pc.KDEMode.constant) is None:
+            return None
+        c_pad, f_pad = pad
+        final = self.final_weights.reshape(1, c * h, f)
+        if c_pad != c or f_pad != f:
+            final = torch.nn.functional.pad(final.reshape(1, c, h, f),
+                                            (0, f_pad - f, 0, 0, 0, c_pad - c))
+            final = final.reshape(1, c_pad * h, f_pad)
+            features = torch.nn.functional.pad(features, (0, c_pad - c))
+        out = _PointConvLayer.apply(self.weights.reshape(1, d, h), self.biases.reshape(1, h),
+                                    final, self.pdf_weights_1, self.pdf_biases_1,
+                                    self.pdf_weights_2, self.pdf_biases_2,
+                                    features.contiguous(), neighborhood, self._act)
+        return out[:, :f] if f_pad != f else out
+
     def _convolve(self, features, point_cloud_in, point_cloud_out, radius, neighborhood,
                   bandwidth):
         d, dev = self._num_dims, features.device
@@ -550,6 +668,9 @@ class PointConv(torch.nn.Module):
                 point_cloud_out._points[ids[:, 1].long()]
             hidden = _activate(diff @ self.weights + self.biases, self._act)
         else:
+            out = self._convolve_on_view(features, neighborhood, bandwidth)
+            if out is not None:
+                return out
             pdf = neighborhood.get_pdf(bandwidth=bandwidth, mode=pc.KDEMode.constant)
             # hidden layer on the unscaled offsets (PointConv.py:268-272): unit radii, unit pdf
             ones_d = torch.ones(d, dtype=_F32, device=dev)
