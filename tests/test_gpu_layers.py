@@ -152,6 +152,48 @@ def test_pointconv_forward_backward(oracle, hidden, act, fused):
     normwise(conv.pdf_biases_2.grad.cpu().numpy(), t["pb2"].grad.numpy(), tol=5e-5)
 
 
+@pytest.mark.parametrize("column", [0, 1])
+def test_pointconv_density_transform_and_parameter_gradients(column):
+    """The per-pair density transform of PointConv (PointConv.py:176-190) and the
+    gradients of its 49 parameters against float64 torch autograd, for a pair table
+    read in either orientation; two slabs of scale gradients."""
+    from tensorflow_graphics_point_clouds_amd import _lib
+    from tensorflow_graphics_point_clouds_amd._lib import cint, csize, i64, ptr, stream
+    gen = torch.Generator(device="cuda").manual_seed(column)
+    m, n_pts, n_ctr = 70001, 900, 400
+    pairs = torch.stack((torch.randint(0, n_pts, (m,), device="cuda", generator=gen),
+                         torch.randint(0, n_ctr, (m,), device="cuda", generator=gen)), 1).int()
+    if column == 1:
+        pairs = pairs.flip(1).contiguous()
+    pdf = torch.rand(n_pts, device="cuda", generator=gen) + 0.1
+    mx = torch.rand(n_ctr, device="cuda", generator=gen) + 1.0
+    par = [torch.randn(s, device="cuda", generator=gen) for s in (16, 16, 16, 1)]
+    par[3] += 3.0
+    y = torch.empty(m, device="cuda")
+    _lib.call("pointconv_density", stream(), i64(m), ptr(pairs), cint(column), ptr(pdf), ptr(mx),
+              ptr(par[0]), ptr(par[1]), ptr(par[2]), ptr(par[3]), ptr(y))
+    ref = [p.double().cpu().requires_grad_(True) for p in par]
+    pt, ctr = pairs[:, column].long().cpu(), pairs[:, 1 - column].long().cpu()
+    rel = (pdf.double().cpu()[pt] / mx.double().cpu()[ctr]).reshape(-1, 1)
+    yr = torch.relu(rel * ref[0] + ref[1]) @ ref[2] + ref[3]
+    normwise(y.cpu().numpy(), yr.detach().numpy(), tol=1e-5)
+    # gradient of sum_m t[m] / y[m] for two slabs of scale gradients t
+    t = torch.randn((2, m), device="cuda", generator=gen)
+    L = _lib.lib()
+    ws = _lib.workspace(L.mccnn_pointconv_density_grads_workspace_bytes(i64(m)), y.device)
+    grads = torch.empty(49, device="cuda")
+    _lib.call("pointconv_density_grads", stream(), i64(m), ptr(pairs), cint(column), ptr(pdf),
+              ptr(mx), ptr(par[0]), ptr(par[1]), ptr(par[2]), ptr(par[3]), ptr(y), cint(2),
+              ptr(t), ptr(ws), csize(ws.numel()), ptr(grads))
+    (t.double().cpu().sum(0) / yr).sum().backward()
+    expect = torch.cat([r.grad.reshape(-1) for r in ref]).numpy()
+    scale = torch.cat([(t.double().cpu().sum(0).abs() / yr.detach() ** 2).sum().reshape(1)] * 49)
+    assert np.abs(grads.cpu().numpy() - expect).max() <= 1e-5 * float(scale[0])
+    with pytest.raises(ValueError):
+        _lib.call("pointconv_density", stream(), i64(m), ptr(pairs), cint(2), ptr(pdf), ptr(mx),
+                  ptr(par[0]), ptr(par[1]), ptr(par[2]), ptr(par[3]), ptr(y))
+
+
 @pytest.mark.parametrize("c_in,c_out,transposed,kpn", [(16, 24, True, 15), (16, 24, False, 15),
                                                        (64, 32, True, 15), (8, 16, True, 15),
                                                        (16, 16, True, 5), (32, 8, True, 18),
