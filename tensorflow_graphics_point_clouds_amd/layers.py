@@ -634,18 +634,24 @@ class PointConv(torch.nn.Module):
         d, c, f, h = (self._num_dims, self._num_features_in, self._num_features_out,
                       self._size_hidden)
         pad = _layer_padding(c, f, 1)
-        if not self.fused or h not in (16, 32) or d not in (2, 3) or pad is None:
+        if not self.fused or d not in (2, 3) or pad is None:
             return None
         if neighborhood.point_pdf(bandwidth=bandwidth, mode=pc.KDEMode.constant) is None:
             return None
         c_pad, f_pad = pad
+        h_pad = max(h, 16)       # 8 hidden units: zero columns (every activation maps 0 to 0)
+        weights, biases = self.weights, self.biases
         final = self.final_weights.reshape(1, c * h, f)
-        if c_pad != c or f_pad != f:
+        if h_pad != h:
+            weights = torch.nn.functional.pad(weights, (0, h_pad - h))
+            biases = torch.nn.functional.pad(biases, (0, h_pad - h))
+        if c_pad != c or f_pad != f or h_pad != h:
             final = torch.nn.functional.pad(final.reshape(1, c, h, f),
-                                            (0, f_pad - f, 0, 0, 0, c_pad - c))
-            final = final.reshape(1, c_pad * h, f_pad)
+                                            (0, f_pad - f, 0, h_pad - h, 0, c_pad - c))
+            final = final.reshape(1, c_pad * h_pad, f_pad)
             features = torch.nn.functional.pad(features, (0, c_pad - c))
-        out = _PointConvLayer.apply(self.weights.reshape(1, d, h), self.biases.reshape(1, h),
+        h = h_pad
+        out = _PointConvLayer.apply(weights.reshape(1, d, h), biases.reshape(1, h),
                                     final, self.pdf_weights_1, self.pdf_biases_1,
                                     self.pdf_weights_2, self.pdf_biases_2,
                                     features.contiguous(), neighborhood, self._act)

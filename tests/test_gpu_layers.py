@@ -98,7 +98,7 @@ def test_mcconv_forward_backward(oracle, c_in, c_out, hidden, num_mlps, act, fus
     normwise(conv.biases.grad.cpu().numpy(), tb.grad.numpy(), tol=2e-5)
 
 
-@pytest.mark.parametrize("hidden,act,fused", [(8, "relu", True), (16, "elu", True),
+@pytest.mark.parametrize("hidden,act,fused", [(8, "relu", True), (8, "elu", False), (16, "elu", True),
                                               (32, "leaky_relu", True), (32, "leaky_relu", False)])
 def test_pointconv_forward_backward(oracle, hidden, act, fused):
     """PointConv against the numpy expressions of point_conv_test.py:75-117 evaluated
