@@ -65,6 +65,19 @@ def test_invalid_arguments_return_status_not_abort(lib):
     assert rc == 1 and b"batch size" in lib.mccnn_last_error()
 
 
+def test_pointconv_density_entry_points_validate_before_the_device(lib):
+    i64, sz = ctypes.c_int64, ctypes.c_size_t
+    rc = lib.mccnn_pointconv_density(None, i64(5), None, 2, None, None, None, None, None, None, None)
+    assert rc == 1 and b"point_column" in lib.mccnn_last_error()
+    assert lib.mccnn_pointconv_density(None, i64(0), None, 0, None, None, None, None, None, None,
+                                       None) == 0
+    rc = lib.mccnn_pointconv_density_grads(None, i64(5), None, 0, None, None, None, None, None, None,
+                                           None, 5, None, None, sz(0), None)
+    assert rc == 1 and b"slabs" in lib.mccnn_last_error()
+    lib.mccnn_pointconv_density_grads_workspace_bytes.restype = sz
+    assert lib.mccnn_pointconv_density_grads_workspace_bytes(i64(10 ** 6)) >= 49 * 4
+
+
 def test_layer_entry_points_reject_uncovered_shapes(lib):
     i64, sz = ctypes.c_int64, ctypes.c_size_t
     assert lib.mccnn_mc_conv_supported(3, 64, 16) == 1 and lib.mccnn_mc_conv_supported(3, 24, 16) == 0
