@@ -13,6 +13,10 @@
 //           a ballot prefix inside the 16-lane group, so the pairs of a centre
 //           come out in ascending sorted-point index without atomics or a sort.
 // Offsets are enumerated so that the slices of a centre ascend in index.
+// (Keeping the count pass's hit masks for the fill pass, so that it need not load
+// and test the candidates again, was measured: what the count pass loses by
+// storing them is what the fill pass gains, and crowded centres, whose masks do
+// not fit a fixed budget, pay for both.)
 // Compiled with -ffp-contract=off (the distance test decides integer output).
 #include "common.h"
 #include "fill.h"
