@@ -560,6 +560,63 @@ def test_mcconv_layer_at_full_scene_size():
         normwise(dfeat[j].cpu().numpy(), expect.cpu().numpy(), tol=2e-5)
 
 
+def test_mcconv_step_replays_from_a_captured_graph():
+    """With its neighbourhood built, a Monte-Carlo convolution enqueues kernels and
+    library products only: forward + backward recorded in a HIP graph, replayed on
+    changed features with eager steps in between; outputs and every gradient equal
+    the eager ones bit for bit (the layer path has no atomics)."""
+    from tensorflow_graphics_point_clouds_amd import layers, pc
+    gen = torch.Generator(device="cuda").manual_seed(3)
+    n = 4000
+    pts = torch.rand((n, 3), device="cuda", generator=gen)
+    bids = (torch.arange(n, device="cuda") % 2).int()
+    cloud = pc.PointCloud(pts, bids, 2)
+    conv = layers.MCConv(32, 48, 3, num_mlps=1, mlp_size=[16], seed=4)
+    feat = torch.randn((n, 32), device="cuda", generator=gen).requires_grad_(True)
+    up = torch.randn((n, 48), device="cuda", generator=gen)
+    nbh = pc.Neighborhood(pc.Grid(cloud, 0.12), 0.12, cloud)
+    params = list(conv.parameters())
+
+    def step():
+        feat.grad = None
+        for p in params:
+            p.grad = None
+        out = conv(feat, cloud, cloud, 0.12, neighborhood=nbh)
+        out.backward(up)
+        return out
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(3):
+            step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    feat.grad = None
+    for p in params:
+        p.grad = None
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = conv(feat, cloud, cloud, 0.12, neighborhood=nbh)
+        out.backward(up)
+    captured = [out, feat.grad] + [p.grad for p in params]
+    for rep in range(3):
+        with torch.no_grad():
+            feat.copy_(torch.randn((n, 32), device="cuda", generator=gen))
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [t.clone() for t in captured]
+        eager_out = step()
+        torch.cuda.synchronize()
+        eager = [eager_out, feat.grad] + [p.grad for p in params]
+        for a, b in zip(got, eager):
+            assert torch.equal(a, b), rep
+        # the eager step re-created the gradient tensors; point the graph's at fresh zeros
+        feat.grad = captured[1]
+        for p, g in zip(params, captured[2:]):
+            p.grad = g
+
+
 @pytest.mark.parametrize("mlp_size,num_mlps,act", [([8, 16], 1, "relu"), ([4, 8, 8], 2, "elu")])
 def test_mcconv_with_deeper_kernel_mlp(oracle, mlp_size, num_mlps, act):
     """Kernel MLPs of several layers (MCConv.py:163-171): forward and all gradients
