@@ -183,11 +183,11 @@ extern "C" int mccnn_weight_grad_product(mccnn_stream_t stream, int64_t num_pts,
                     mccnn_weight_grad_product_workspace_bytes(num_rows_out, num_cols_out),
                 "weight_grad_product workspace too small");
   hipStream_t s = as_stream(stream);
-  // slices of the point range, each reduced on its own: at least 512 points per slice, so that a
-  // small cloud does not pay for summing a thousand empty partials
+  // slices of the point range, each reduced on its own: at least 128 points per slice, so that a
+  // small cloud does not pay for summing a thousand empty partials and still fills the device
   const int C = num_rows_out, R = num_cols_out;
   int slices = tn_slices(R);
-  const int64_t by_size = (num_pts + 511) / 512;
+  const int64_t by_size = (num_pts + 127) / 128;
   if (slices > by_size) slices = by_size < 1 ? 1 : (int)by_size;
   const dim3 grid((R / 256) * slices), block(256);
   float *partials = (float *)workspace;
