@@ -560,6 +560,82 @@ def test_mcconv_layer_at_full_scene_size():
         normwise(dfeat[j].cpu().numpy(), expect.cpu().numpy(), tol=2e-5)
 
 
+@pytest.mark.parametrize("layer", ["mcconv", "kpconv", "pointconv"])
+def test_fused_layers_in_two_dimensions(layer):
+    """The three convolutions on planar clouds (D = 2 takes its own instantiation of
+    every fused kernel): outputs and gradients against float64 torch autograd of the
+    reference expressions on the layer's own pair table and densities."""
+    from tensorflow_graphics_point_clouds_amd import layers, pc
+    rng = np.random.default_rng(21)
+    n, n_out, batch, radius, c_in, c_out = 2600, 700, 2, 0.07, 16, 32
+    pts = rng.random((n, 2)).astype(np.float32)
+    bids = np.sort(rng.integers(0, batch, n)).astype(np.int32)
+    ctr = rng.random((n_out, 2)).astype(np.float32)
+    cb = np.sort(rng.integers(0, batch, n_out)).astype(np.int32)
+    feat = rng.standard_normal((n, c_in)).astype(np.float32)
+    cin, cout = pc.PointCloud(dev(pts), dev(bids), batch), pc.PointCloud(dev(ctr), dev(cb), batch)
+    if layer == "mcconv":
+        conv = layers.MCConv(c_in, c_out, 2, num_mlps=1, mlp_size=[16],
+                             non_linearity_type="leaky_relu", seed=1)
+    elif layer == "kpconv":
+        ang = np.linspace(0, 2 * np.pi, 6, endpoint=False)
+        kp = np.concatenate([np.zeros((1, 2)), 0.8 * np.stack([np.cos(ang), np.sin(ang)], 1)])
+        conv = layers.KPConv(c_in, c_out, num_kernel_points=7, num_dims=2,
+                             custom_kernel_points=kp.astype(np.float32), seed=2)
+    else:
+        conv = layers.PointConv(c_in, c_out, 2, size_hidden=16, seed=3)
+        with torch.no_grad():      # a density MLP away from its kinks and from zero
+            conv.pdf_weights_1.abs_().add_(0.2)
+            conv.pdf_weights_2.abs_().add_(0.2)
+            conv.pdf_biases_2.fill_(0.5)
+    tfeat = dev(feat).requires_grad_(True)
+    out = conv(tfeat, cin, cout, radius)
+    up = rng.standard_normal(out.shape).astype(np.float32)
+    out.backward(dev(up))
+
+    nb = conv.last_neighborhood
+    ids = nb._original_neigh_ids.cpu().long()
+    f64 = lambda t: t.detach().cpu().double()
+    x = torch.tensor(feat.astype(np.float64), requires_grad=True)
+    delta = torch.tensor((pts[ids[:, 0]] - ctr[ids[:, 1]]).astype(np.float64))
+    ref_params = {}
+
+    def leaf(name, t):
+        ref_params[name] = f64(t).requires_grad_(True)
+        return ref_params[name]
+
+    if layer == "mcconv":
+        pdf = f64(nb.get_pdf()).reshape(-1, 1)
+        hid = torch.nn.functional.leaky_relu(
+            (delta / radius) @ leaf("weights", conv.weights)[0] + leaf("biases", conv.biases)[0], 0.2)
+        basis = hid / pdf
+        final = leaf("final_weights", conv.final_weights)[0]
+    elif layer == "kpconv":
+        kpt = torch.tensor(kp * 0.75)
+        dist = ((delta / radius)[:, None, :] - kpt[None]).norm(dim=2)
+        basis = torch.relu(1.0 - dist)
+        final = leaf("weights", conv.weights)
+    else:
+        pdf = f64(nb.get_pdf())
+        mx = torch.zeros(n_out, dtype=torch.float64).scatter_reduce(0, ids[:, 1], pdf, "amax",
+                                                                    include_self=False)
+        rel = (pdf / mx[ids[:, 1]]).reshape(-1, 1)
+        y = torch.relu(rel @ leaf("pdf_weights_1", conv.pdf_weights_1) +
+                       leaf("pdf_biases_1", conv.pdf_biases_1)) @ \
+            leaf("pdf_weights_2", conv.pdf_weights_2) + leaf("pdf_biases_2", conv.pdf_biases_2)
+        basis = torch.relu(delta @ leaf("weights", conv.weights) + leaf("biases", conv.biases)) / y
+        final = leaf("final_weights", conv.final_weights)
+    per_pair = x[ids[:, 0]][:, :, None] * basis[:, None, :]
+    proj = torch.zeros(n_out, c_in, basis.shape[1], dtype=torch.float64).index_add(
+        0, ids[:, 1], per_pair)
+    ref = proj.reshape(n_out, -1) @ final.reshape(-1, c_out)
+    normwise(out.detach().cpu().numpy(), ref.detach().numpy(), tol=2e-5)
+    (ref * torch.tensor(up.astype(np.float64))).sum().backward()
+    normwise(tfeat.grad.cpu().numpy(), x.grad.numpy(), tol=2e-5)
+    for name, t in ref_params.items():
+        normwise(getattr(conv, name).grad.cpu().numpy(), t.grad.numpy(), tol=5e-5)
+
+
 def test_mcconv_step_replays_from_a_captured_graph():
     """With its neighbourhood built, a Monte-Carlo convolution enqueues kernels and
     library products only: forward + backward recorded in a HIP graph, replayed on
