@@ -381,7 +381,9 @@ class Neighborhood:
     """Neighbour pairs of the centres `point_cloud_sample` (default: the grid's
     own sorted points) inside `grid` (pylib/pc/Neighborhood.py:218-311)."""
 
-    def __init__(self, grid, radius, point_cloud_sample=None, max_neighbors=0):
+    def __init__(self, grid, radius, point_cloud_sample=None, max_neighbors=0, lazy=False):
+        """`lazy` puts the search off until the pair table is first read (a cell-average
+        hierarchy keeps a neighbourhood per level that it never reads itself)."""
         d = grid._point_cloud._dimension
         dev = grid._sorted_points.device
         self._radii = _as_vector(radius, d, dev)
@@ -407,11 +409,8 @@ class Neighborhood:
             # only); it is built when somebody asks for it, which the layers on the
             # grid-ordered view never do.
             self._self_neighborhood = grid.self_neighborhood(self._radii, max_neighbors)
-        else:
-            self._ranges, self._table = tfg_custom_ops.find_neighbors(
-                s._points, s._batch_ids, grid._sorted_points, grid._sorted_keys, grid.get_DS(),
-                grid._num_cells, grid._scaled_aabb_min, grid._inv_cell_sizes, self._inv_radii,
-                max_neighbors)
+        elif not lazy:
+            self._search()
         self._pdf = None
         self._pdf_per_point = None
         self._pdf_args = None
@@ -422,7 +421,16 @@ class Neighborhood:
         self._sorted_view = None
         self._transposed = None
 
+    def _search(self):
+        s, grid = self._point_cloud_sampled, self._grid
+        self._ranges, self._table = tfg_custom_ops.find_neighbors(
+            s._points, s._batch_ids, grid._sorted_points, grid._sorted_keys, grid.get_DS(),
+            grid._num_cells, grid._scaled_aabb_min, grid._inv_cell_sizes, self._inv_radii,
+            self.max_neighbors)
+
     def _regroup(self):
+        if self._self_neighborhood is None:      # a search that was put off
+            return self._search()
         own, grid = self._self_neighborhood, self._grid
         n = self._point_cloud_sampled._points.shape[0]
         dev = own._neighbors.device
@@ -553,9 +561,16 @@ def sample(neighborhood, sample_mode="poisson"):
     """pylib/pc/sampling.py:123-150 -> (PointCloud, original indices or None)."""
     mode = _SAMPLE_MODES[sample_mode.lower()]
     g = neighborhood._grid
+    if mode == 1:
+        # cell averages read the keys only: no reason to run the neighbour search that
+        # the (lazily built) pair table of `neighborhood` would cost
+        dev = g._sorted_points.device
+        pairs = torch.empty((0, 2), dtype=_I32, device=dev)
+        ranges = torch.zeros(g._sorted_points.shape[0], dtype=_I32, device=dev)
+    else:
+        pairs, ranges = neighborhood._neighbors, neighborhood._samples_neigh_ranges
     pts, bids, idx = tfg_custom_ops.sampling(
-        g._sorted_points, g._sorted_batch_ids, g._sorted_keys, g._num_cells,
-        neighborhood._neighbors, neighborhood._samples_neigh_ranges, mode)
+        g._sorted_points, g._sorted_batch_ids, g._sorted_keys, g._num_cells, pairs, ranges, mode)
     original = None
     if mode == 0:
         original = torch.empty_like(idx)
@@ -585,7 +600,7 @@ def cell_average_sampling(point_cloud, cell_sizes=None, grid=None):
     if grid is None:
         grid = Grid(point_cloud, _as_vector(cell_sizes, point_cloud._dimension,
                                             point_cloud._points.device))
-    return sample(Neighborhood(grid, grid._cell_sizes), "average")[0]
+    return sample(Neighborhood(grid, grid._cell_sizes, lazy=True), "average")[0]
 
 
 class PointHierarchy:
@@ -601,7 +616,7 @@ class PointHierarchy:
             cs = _as_vector(cs, point_cloud._dimension, point_cloud._points.device)
             self._cell_sizes.append(cs)
             grid = Grid(cur, cs)
-            nbh = Neighborhood(grid, cs)
+            nbh = Neighborhood(grid, cs, lazy=_SAMPLE_MODES[sample_mode.lower()] == 1)
             cur, idx = sample(nbh, sample_mode)
             self._neighborhoods.append(nbh)
             self._point_clouds.append(cur)
