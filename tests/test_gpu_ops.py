@@ -575,6 +575,40 @@ def test_object_level_adapters_match_the_callers(ops):
                        ops.basis_proj(basis, feat, nbh._original_neigh_ids, ranges))
 
 
+def test_pipeline_on_the_reference_sample_cloud(ops, oracle):
+    """Real data instead of uniform noise: the first 256 points of the reference's
+    sample scan (positions; the normals serve as features), radius 0.05: keys, sort,
+    grid table and pairs bit-exact, densities and the projection within 1e-5."""
+    import os
+    from tensorflow_graphics_point_clouds_amd import pc
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden",
+                        "shrec15_cloud0_first256.txt")
+    data = np.loadtxt(path, delimiter=",", dtype=np.float32)
+    pts, normals = np.ascontiguousarray(data[:, :3]), np.ascontiguousarray(data[:, 3:6])
+    bids = np.zeros(len(pts), np.int32)
+    radius = np.float32(0.05)
+    g = oracle.Grid(pts, bids, 1, radius)
+    nbh = oracle.Neighborhood(g, radius, pts, bids)
+    cloud = pc.PointCloud(dev(pts), dev(bids), 1)
+    grid = pc.Grid(cloud, float(radius))
+    got = pc.Neighborhood(grid, float(radius), cloud)
+    assert np.array_equal(grid._sorted_keys.cpu().numpy(), g.sorted_keys)
+    assert np.array_equal(grid._sorted_indices.cpu().numpy(), g.sorted_indices)
+    assert np.array_equal(grid.get_DS().cpu().numpy(), g.get_ds())
+    assert np.array_equal(got._samples_neigh_ranges.cpu().numpy(), nbh.ranges)
+    assert np.array_equal(got._neighbors.cpu().numpy(), nbh.neighbors)
+    assert np.array_equal(got._original_neigh_ids.cpu().numpy(), nbh.original_neigh_ids)
+    assert len(nbh.neighbors) > 2 * len(pts)          # the radius reaches beyond the point itself
+    pdf = nbh.pdf_per_pair(0.2)
+    np.testing.assert_allclose(got.get_pdf(bandwidth=0.2).cpu().numpy(), pdf, rtol=1e-5)
+    rng = np.random.default_rng(0)
+    basis = rng.random((len(nbh.neighbors), 16)).astype(np.float32)
+    feat = np.concatenate([normals, np.ones((len(pts), 1), np.float32)], axis=1)   # C = 4
+    out = ops.basis_proj(dev(basis), dev(feat), got._original_neigh_ids, got._samples_neigh_ranges)
+    expect, mag = oracle.basis_proj(basis, feat, nbh.original_neigh_ids, nbh.ranges, with_magnitude=True)
+    assert_rel(out.cpu().numpy(), expect, mag)
+
+
 def test_ops_without_a_host_round_trip_replay_from_a_captured_graph(ops):
     """The entry points that size no output enqueue kernels only (zero-fills are
     kernels too), so a caller may capture them: basis_proj with both gradients and
