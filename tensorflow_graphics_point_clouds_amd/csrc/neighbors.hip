@@ -16,7 +16,9 @@
 // (Keeping the count pass's hit masks for the fill pass, so that it need not load
 // and test the candidates again, was measured: what the count pass loses by
 // storing them is what the fill pass gains, and crowded centres, whose masks do
-// not fit a fixed budget, pay for both.)
+// not fit a fixed budget, pay for both.  Letting the count pass find its slices
+// itself, 9 of a group's 16 lanes searching, saves a launch and was no faster
+// either.)
 // Compiled with -ffp-contract=off (the distance test decides integer output).
 #include "common.h"
 #include "fill.h"
