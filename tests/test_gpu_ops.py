@@ -609,6 +609,55 @@ def test_pipeline_on_the_reference_sample_cloud(ops, oracle):
     assert_rel(out.cpu().numpy(), expect, mag)
 
 
+def test_two_host_threads_on_their_own_streams(ops, oracle):
+    """The library keeps no state between calls (error text and the pinned size
+    word are per thread, workspaces per call): two host threads, each on its own
+    stream, build grids and neighbourhoods and project at the same time and get
+    what the oracle gets."""
+    import threading
+    from tensorflow_graphics_point_clouds_amd import pc
+    jobs = []
+    for seed in (1, 2):
+        rng = np.random.default_rng(seed)
+        pts, bids = _cloud(rng, 3, 20000 + 3000 * seed, 3)
+        radius = np.float32(0.04 + 0.01 * seed)
+        g = oracle.Grid(pts, bids, 3, radius)
+        nbh = oracle.Neighborhood(g, radius, pts, bids)
+        basis = rng.random((len(nbh.neighbors), 16)).astype(np.float32)
+        feat = rng.standard_normal((len(pts), 16)).astype(np.float32)
+        expect, mag = oracle.basis_proj(basis, feat, nbh.original_neigh_ids, nbh.ranges,
+                                        with_magnitude=True)
+        jobs.append(dict(pts=dev(pts), bids=dev(bids), radius=float(radius), nbh=nbh,
+                         basis=dev(basis), feat=dev(feat), expect=expect, mag=mag, out=None,
+                         error=None))
+    torch.cuda.synchronize()
+
+    def work(job):
+        try:
+            stream = torch.cuda.Stream()
+            with torch.cuda.stream(stream):
+                for _ in range(3):
+                    cloud = pc.PointCloud(job["pts"], job["bids"], 3)
+                    got = pc.Neighborhood(pc.Grid(cloud, job["radius"]), job["radius"], cloud)
+                    out = ops.basis_proj(job["basis"], job["feat"], got._original_neigh_ids,
+                                         got._samples_neigh_ranges)
+                stream.synchronize()
+            job["out"] = (got._neighbors.cpu().numpy(), out.cpu().numpy())
+        except Exception as exc:                      # surfaced by the main thread
+            job["error"] = exc
+
+    threads = [threading.Thread(target=work, args=(job,)) for job in jobs]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    for job in jobs:
+        assert job["error"] is None, job["error"]
+        pairs, out = job["out"]
+        assert np.array_equal(pairs, job["nbh"].neighbors)
+        assert_rel(out, job["expect"], job["mag"])
+
+
 def test_ops_without_a_host_round_trip_replay_from_a_captured_graph(ops):
     """The entry points that size no output enqueue kernels only (zero-fills are
     kernels too), so a caller may capture them: basis_proj with both gradients and
