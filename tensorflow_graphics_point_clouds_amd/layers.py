@@ -455,13 +455,24 @@ def _differentiable_pdf(neighborhood, bandwidth):
     grid = neighborhood._grid
     points = grid._point_cloud._points
     d, dev = points.shape[1], points.device
+    mode = pc.KDEMode.constant
+    if neighborhood._pdf_args is not None:       # the settings of an earlier compute_pdf
+        bandwidth, mode = neighborhood._pdf_args
+    nb = neighborhood._neighbors
+    if mode == pc.KDEMode.no_pdf:
+        return torch.ones(nb.shape[0], dtype=_F32, device=dev)
     own = neighborhood if neighborhood._equal_samples else \
         grid.self_neighborhood(neighborhood._radii)
     per_point = tfg_custom_ops.compute_pdf_with_pt_grads(
         points[grid._sorted_indices.long()], own._neighbors, own._samples_neigh_ranges,
         torch.reciprocal(pc._as_vector(bandwidth, d, dev)), own._inv_radii,
-        pc.KDEMode.constant.value, symmetric=own._equal_samples and own.max_neighbors == 0)
-    return per_point[neighborhood._neighbors[:, 0].long()]
+        mode.value, symmetric=own._equal_samples and own.max_neighbors == 0)
+    pdf = per_point[nb[:, 0].long()]
+    if neighborhood._pdf_normalize:              # Neighborhood.py:288-293
+        ends = neighborhood._samples_neigh_ranges.long()
+        counts = (ends - torch.cat([ends.new_zeros(1), ends[:-1]])).to(_F32)
+        pdf = pdf / counts[nb[:, 1].long()]
+    return pdf
 
 
 def _moving(*clouds):

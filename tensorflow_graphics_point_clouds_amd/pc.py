@@ -361,7 +361,9 @@ class _SortedView:
     def pair_pdf(self, nbh):
         """Per-pair densities of `table` and `table_t` (the neighbour point's)."""
         per_point = nbh._pdf_per_point
-        key = None if per_point is None else (per_point.data_ptr(), per_point._version)
+        # compute_pdf bumps the generation: a key made of the density tensor's address
+        # could match a later tensor that the allocator put in the same place
+        key = nbh._pdf_generation
         if self.pdf is None or key != self._pdf_key:
             m, dev = self.table.shape[0], self.table.device
             if per_point is None:
@@ -373,6 +375,14 @@ class _SortedView:
                 for out, table, column in ((self.pdf, self.table, 0), (self.pdf_t, self.table_t, 1)):
                     _lib.call("gather_pdf_column", stream(), i64(m), ptr(table, _I32), cint(column),
                               ptr(per_point, _F32), ptr(out))
+                if nbh._pdf_normalize:
+                    # Neighborhood.py:288-293: divided by the size of the pair's
+                    # neighbourhood, i.e. the pair count of its centre (column 1 of
+                    # `table`, column 0 of `table_t`)
+                    ends = self.ranges.long()
+                    counts = (ends - torch.cat([ends.new_zeros(1), ends[:-1]])).to(_F32)
+                    self.pdf = self.pdf / counts[self.table[:, 1].long()]
+                    self.pdf_t = self.pdf_t / counts[self.table_t[:, 0].long()]
             self._pdf_key = key
         return self.pdf, self.pdf_t
 
@@ -415,6 +425,7 @@ class Neighborhood:
         self._pdf_per_point = None
         self._pdf_args = None
         self._pdf_normalize = False
+        self._pdf_generation = 0
         # optional visiting order of the centres for the projection kernels
         self._centre_order = None
         self._transposed_pairs = None
@@ -517,6 +528,7 @@ class Neighborhood:
         self._pdf = None
         self._pdf_args = (bandwidth, mode)
         self._pdf_normalize = bool(normalize)
+        self._pdf_generation += 1
         if mode == KDEMode.no_pdf:
             self._pdf_per_point = None
             return

@@ -1,0 +1,488 @@
+"""The benchmark configurations as parity cases on the GPU.
+
+* configuration 1 (2 x 1024 points, MCConv 8 -> 16) against the oracle, end to end;
+* neighbourhoods with normalised densities through the fused and the unfused layer;
+* configuration 5 (kernel-point convolution 128 -> 128, 15 points, clustered clouds) at a
+  reduced size against the oracle / float64 autograd and at its real size through sampled
+  rows in float64 and properties of the whole tensors;
+* configuration 4 (4 x 200k uniform points, C = 128, K = 32) at its real size, where the
+  element offsets of the projection and of the basis pass 2^31, and its Poisson-disk
+  sampling at 800k points.
+
+Float tolerance: |got - expect| <= 1e-5 * mag elementwise, where mag is the same sum
+taken over the absolute values of its terms, unless a test states otherwise."""
+import numpy as np
+import pytest
+
+torch = pytest.importorskip("torch")
+
+pytestmark = pytest.mark.gpu
+
+REL = 1e-5
+
+
+def dev(a):
+    return torch.as_tensor(np.ascontiguousarray(a)).cuda().contiguous()
+
+
+def assert_rel(got, expect, mag, tol=REL):
+    got, expect, mag = (np.asarray(a, np.float64) for a in (got, expect, mag))
+    err = np.abs(got - expect)
+    bad = err > tol * mag + 1e-30
+    assert not bad.any(), "max err/mag = %g at %d of %d entries" % (
+        (err / np.maximum(mag, 1e-300)).max(), int(bad.sum()), err.size)
+
+
+def assert_rel_t(got, expect, mag, tol=REL):
+    """The same bound on device tensors (float64 expect / mag)."""
+    err = (got.double() - expect).abs()
+    bad = err > tol * mag + 1e-30
+    assert not bool(bad.any()), "max err/mag = %g at %d of %d entries" % (
+        float((err / mag.clamp(min=1e-300)).max()), int(bad.sum()), err.numel())
+
+
+# ------------------------------------------------------------ configuration 1 ----
+
+def test_config1_mcconv_layer_matches_oracle(oracle):
+    """2 x 1024 uniform points, 8 -> 16 channels, radius 0.1, bandwidth 0.2, ReLU kernel
+    of 16 units: pair table bit-exact, densities and output against the oracle, and the
+    gradients against float64 autograd on the oracle's pairs."""
+    from tensorflow_graphics_point_clouds_amd import layers, pc, synthetic
+    cfg = synthetic.config1()
+    cloud = pc.PointCloud(dev(cfg["points"]), dev(cfg["batch_ids"]), cfg["batch_size"])
+    conv = layers.MCConv(8, 16, 3, num_mlps=1, mlp_size=[16], non_linearity_type="relu",
+                         weights=dev(cfg["weights"]), biases=dev(cfg["biases"]),
+                         final_weights=dev(cfg["final_weights"]))
+    feats = dev(cfg["features"]).requires_grad_(True)
+    out = conv(feats, cloud, cloud, cfg["radius"], bandwidth=cfg["bandwidth"])
+    r = np.float32(cfg["radius"])
+    g = oracle.Grid(cfg["points"], cfg["batch_ids"], cfg["batch_size"], r)
+    nbh = oracle.Neighborhood(g, r, cfg["points"], cfg["batch_ids"])
+    got = conv.last_neighborhood
+    assert np.array_equal(got._samples_neigh_ranges.cpu().numpy(), nbh.ranges)
+    assert np.array_equal(got._neighbors.cpu().numpy(), nbh.neighbors)
+    assert np.array_equal(got._original_neigh_ids.cpu().numpy(), nbh.original_neigh_ids)
+    pdf = nbh.pdf_per_pair(cfg["bandwidth"])
+    np.testing.assert_allclose(got.get_pdf().cpu().numpy(), pdf, rtol=REL)
+    expect, basis, proj = oracle.mc_conv_forward(
+        cfg["features"], cfg["points"], cfg["points"], nbh, pdf, cfg["weights"], cfg["biases"],
+        cfg["final_weights"], r)
+    _, pmag = oracle.basis_proj(np.abs(basis).astype(np.float32), np.abs(cfg["features"]),
+                                nbh.original_neigh_ids, nbh.ranges, with_magnitude=True)
+    mag = pmag.reshape(len(expect), -1) @ np.abs(cfg["final_weights"][0]).astype(np.float64)
+    assert_rel(out.detach().cpu().numpy(), expect, mag)
+
+    rng = np.random.default_rng(1)
+    up = rng.standard_normal(expect.shape).astype(np.float32)
+    out.backward(dev(up))
+    ids = torch.tensor(nbh.original_neigh_ids).long()
+    tw = torch.tensor(cfg["weights"].astype(np.float64), requires_grad=True)
+    tb = torch.tensor(cfg["biases"].astype(np.float64), requires_grad=True)
+    two = torch.tensor(cfg["final_weights"].astype(np.float64), requires_grad=True)
+    tf = torch.tensor(cfg["features"].astype(np.float64), requires_grad=True)
+    radii = np.full(3, r, np.float32)
+    diff = torch.tensor(((cfg["points"][ids[:, 0]] - cfg["points"][ids[:, 1]]) / radii)
+                        .astype(np.float64))
+    bas = torch.relu(diff @ tw[0] + tb[0]) / torch.tensor(pdf).reshape(-1, 1)
+    pj = torch.zeros(len(expect), 8, 16, dtype=torch.float64).index_add(
+        0, ids[:, 1], tf[ids[:, 0]][:, :, None] * bas[:, None, :])
+    ref = pj.reshape(len(expect), -1) @ two[0]
+    (ref * torch.tensor(up.astype(np.float64))).sum().backward()
+    for got_g, ref_g in ((feats.grad, tf.grad), (conv.final_weights.grad, two.grad),
+                         (conv.weights.grad, tw.grad), (conv.biases.grad, tb.grad)):
+        e = ref_g.numpy()
+        assert np.abs(got_g.cpu().numpy() - e).max() <= REL * np.abs(e).max()
+
+
+# ---------------------------------------------------------- normalised densities ----
+
+@pytest.mark.parametrize("same_cloud", [True, False])
+def test_layers_use_the_normalised_density_of_the_neighbourhood(oracle, same_cloud):
+    """Neighborhood.compute_pdf(normalize=True) (Neighborhood.py:288-293) divides a pair's
+    density by the pair count of its centre; the layer on the grid-ordered view and the
+    composed path must both use it (MCConv.py:261 reads the cached get_pdf())."""
+    from tensorflow_graphics_point_clouds_amd import layers, pc, synthetic
+    rng = np.random.default_rng(9)
+    n, n_out, batch, radius, c_in, c_out = 2500, 600, 2, 0.17, 16, 32
+    pts = rng.random((n, 3)).astype(np.float32)
+    bids = np.sort(rng.integers(0, batch, n)).astype(np.int32)
+    if same_cloud:
+        ctr, cb = pts, bids
+    else:
+        ctr = rng.random((n_out, 3)).astype(np.float32)
+        cb = np.sort(rng.integers(0, batch, n_out)).astype(np.int32)
+    feat = rng.standard_normal((n, c_in)).astype(np.float32)
+    w, b, wo = synthetic.mcconv_weights(rng, 3, c_in, c_out, 16, 1)
+    g = oracle.Grid(pts, bids, batch, np.float32(radius))
+    nbh = oracle.Neighborhood(g, np.float32(radius), ctr, cb)
+    counts = np.diff(np.concatenate([[0], nbh.ranges])).astype(np.float64)
+    pdf = nbh.pdf_per_pair(0.25) / counts[nbh.neighbors[:, 1]]
+    plain = nbh.pdf_per_pair(0.25)
+    assert np.abs(pdf - plain).max() > 0.1 * np.abs(plain).max()      # the flag matters
+    expect, _, _ = oracle.mc_conv_forward(feat, pts, ctr, nbh, pdf, w, b, wo,
+                                          np.float32(radius), "leaky_relu")
+    up = rng.standard_normal(expect.shape).astype(np.float32)
+    cin = pc.PointCloud(dev(pts), dev(bids), batch)
+    cout = cin if same_cloud else pc.PointCloud(dev(ctr), dev(cb), batch)
+    grads = []
+    for fused in (True, False):
+        tnb = pc.Neighborhood(pc.Grid(cin, radius), radius, cout)
+        tnb.compute_pdf(bandwidth=0.25, normalize=True)
+        conv = layers.MCConv(c_in, c_out, 3, num_mlps=1, mlp_size=[16],
+                             non_linearity_type="leaky_relu", weights=dev(w), biases=dev(b),
+                             final_weights=dev(wo), fused=fused)
+        tfeat = dev(feat).requires_grad_(True)
+        out = conv(tfeat, cin, cout, radius, neighborhood=tnb, bandwidth=0.25)
+        np.testing.assert_allclose(tnb.get_pdf().cpu().numpy(), pdf, rtol=REL)
+        got = out.detach().cpu().numpy()
+        assert np.abs(got - expect).max() <= REL * np.abs(expect).max()
+        out.backward(dev(up))
+        grads.append([t.grad.cpu().numpy() for t in (tfeat, conv.weights, conv.final_weights)])
+        # a second density estimate replaces the first one on the view as well
+        tnb.compute_pdf(bandwidth=0.25, normalize=False)
+        with torch.no_grad():
+            again = conv(dev(feat), cin, cout, radius, neighborhood=tnb).cpu().numpy()
+        e2, _, _ = oracle.mc_conv_forward(feat, pts, ctr, nbh, plain, w, b, wo,
+                                          np.float32(radius), "leaky_relu")
+        assert np.abs(again - e2).max() <= REL * np.abs(e2).max()
+    for a, e in zip(*grads):
+        assert np.abs(a - e).max() <= 2e-5 * np.abs(e).max()
+    # PointConv divides by the neighbourhood's largest density: the normalisation cancels
+    outs = []
+    for normalize in (True, False):
+        tnb = pc.Neighborhood(pc.Grid(cin, radius), radius, cout)
+        tnb.compute_pdf(bandwidth=0.25, normalize=normalize)
+        pconv = layers.PointConv(c_in, c_out, 3, size_hidden=16, seed=4)
+        with torch.no_grad():
+            outs.append(pconv(dev(feat), cin, cout, radius, neighborhood=tnb, bandwidth=0.25))
+    assert float((outs[0] - outs[1]).abs().max()) <= REL * float(outs[1].abs().max())
+
+
+# ------------------------------------------------------------ configuration 5 ----
+
+def _config5_small(oracle, radius):
+    from tensorflow_graphics_point_clouds_amd import synthetic
+    cfg = synthetic.config5(scale=0.02)
+    pts, bids, batch = cfg["points"], cfg["batch_ids"], cfg["batch_size"]
+    g = oracle.Grid(pts, bids, batch, np.float32(radius))
+    nbh = oracle.Neighborhood(g, np.float32(radius), pts, bids)
+    return cfg, pts, bids, batch, nbh
+
+
+@pytest.mark.parametrize("kind,influence_factor", [("linear", None), ("gaussian", 0.3)])
+def test_config5_kpconv_matches_oracle_at_reduced_size(oracle, kind, influence_factor):
+    """Kernel-point convolution 128 -> 128 with 15 kernel points at 0.6 r on the clustered
+    clouds (1/50 of the points, radius widened to 0.5 so that a centre keeps ~20
+    neighbours, up to ~100): linear correlation (sigma = 1) and Gaussian with an
+    influence distance of 0.3 r (KPConv.py:165-232, 283-288).  Output, feature gradient
+    and weight gradient against the oracle's float64 basis projection."""
+    from tensorflow_graphics_point_clouds_amd import layers, pc, synthetic
+    radius, c, kpn, kpad = 0.5, 128, 15, 16
+    cfg, pts, bids, batch, nbh = _config5_small(oracle, radius)
+    n = len(pts)
+    rng = np.random.default_rng(55)
+    feat = rng.standard_normal((n, c)).astype(np.float32)
+    kp = synthetic.spherical_kernel_points(15, rotate=False) * 0.8       # * 0.75 inside = 0.6
+    np.testing.assert_allclose(kp * 0.75, cfg["kernel_points"], rtol=1e-6)
+    wts = (rng.standard_normal((kpn * c, c)) * np.sqrt(2.0 / (kpn * c + c))).astype(np.float32)
+    influence = None if influence_factor is None else influence_factor * radius
+    sigma = 1.0 if influence is None else influence / radius
+    ids = nbh.original_neigh_ids
+    counts = np.diff(np.concatenate([[0], nbh.ranges]))
+    assert counts.mean() > 15 and counts.max() > 80
+    diff = (pts[ids[:, 0]] - pts[ids[:, 1]]) / np.full(3, np.float32(radius), np.float32)
+    basis, _ = oracle.kp_basis(diff, kp.astype(np.float64) * 0.75, sigma, kind)
+    padded = np.zeros((len(ids), kpad), np.float32)
+    padded[:, :kpn] = basis
+    proj, pmag = oracle.basis_proj(padded, feat, ids, nbh.ranges, with_magnitude=True)
+    proj, pmag = proj[:, :, :kpn].reshape(n, -1), pmag[:, :, :kpn].reshape(n, -1)
+    w64 = wts.astype(np.float64)
+    expect, mag = proj @ w64, pmag @ np.abs(w64)
+
+    cloud = pc.PointCloud(dev(pts), dev(bids), batch)
+    conv = layers.KPConv(c, c, custom_kernel_points=kp, kp_interpolation=kind, weights=dev(wts))
+    tfeat = dev(feat).requires_grad_(True)
+    out = conv(tfeat, cloud, cloud, radius, kernel_influence_dist=influence)
+    assert np.array_equal(conv.last_neighborhood._original_neigh_ids.cpu().numpy(), ids)
+    assert_rel(out.detach().cpu().numpy(), expect, mag)
+
+    up = rng.standard_normal(expect.shape).astype(np.float32)
+    out.backward(dev(up))
+    up64 = up.astype(np.float64)
+    dpad = np.zeros((n, c, kpad), np.float32)
+    dmag = np.zeros((n, c, kpad), np.float32)
+    dpad[:, :, :kpn] = (up64 @ w64.T).reshape(n, c, kpn)
+    dmag[:, :, :kpn] = (np.abs(up64) @ np.abs(w64).T).reshape(n, c, kpn)
+    _, dfeat = oracle.basis_proj_grads(padded, feat, ids, nbh.ranges, dpad)
+    _, fmag = oracle.basis_proj_grads(padded, feat, ids, nbh.ranges, dmag)
+    # dpad is rounded to float32 before the oracle sums it: 2^-24 of the magnitude
+    assert_rel(tfeat.grad.cpu().numpy(), dfeat, fmag, tol=REL + 1e-7)
+    assert_rel(conv.weights.grad.cpu().numpy(), proj.T @ up64, pmag.T @ np.abs(up64))
+
+
+@pytest.mark.parametrize("kind", ["linear", "gaussian"])
+def test_config5_deformable_kpconv_matches_float64_autograd(oracle, kind):
+    """Deformable variant of the same layer (KPConv.py:317-429) at the reduced size:
+    offsets predicted by a rigid convolution with weights scaled so that they come out
+    near N(0, 0.01) in units of the radius, the deformed convolution and the
+    regularisation loss; all gradients against float64 autograd (run on the device, the
+    [M, C, K] intermediate holds 0.4 G doubles) on the oracle's pair table."""
+    from tensorflow_graphics_point_clouds_amd import layers, pc, synthetic
+    radius, c, kpn = 0.4, 128, 15
+    cfg, pts, bids, batch, nbh = _config5_small(oracle, radius)
+    n = len(pts)
+    rng = np.random.default_rng(56)
+    feat = rng.standard_normal((n, c)).astype(np.float32)
+    kp = synthetic.spherical_kernel_points(15, rotate=False) * 0.8
+    wts = (rng.standard_normal((kpn * c, c)) * np.sqrt(2.0 / (kpn * c + c))).astype(np.float32)
+    woff = (rng.standard_normal((kpn * c, kpn * 3)) * 1e-4).astype(np.float32)
+    influence = 0.5 * radius
+    sigma = influence / radius
+    f64 = dict(dtype=torch.float64, device="cuda")
+    ids = torch.tensor(nbh.original_neigh_ids).long().cuda()
+    radii = np.full(3, np.float32(radius), np.float32)
+    o = nbh.original_neigh_ids
+    delta = torch.tensor(((pts[o[:, 0]] - pts[o[:, 1]]) / radii).astype(np.float64)).cuda()
+    tkp = torch.tensor(kp.astype(np.float64) * 0.75).cuda()
+
+    def weight(dist):
+        if kind == "linear":
+            return torch.relu(1 - dist / sigma)
+        return torch.exp(-(dist / (sigma / 3)) ** 2)
+
+    tf = torch.tensor(feat.astype(np.float64), device="cuda", requires_grad=True)
+    tw = torch.tensor(wts.astype(np.float64), device="cuda", requires_grad=True)
+    two = torch.tensor(woff.astype(np.float64), device="cuda", requires_grad=True)
+
+    def project(basis, f):
+        return torch.zeros(n, c, kpn, **f64).index_add(
+            0, ids[:, 1], f[ids[:, 0]][:, :, None] * basis[:, None, :])
+
+    rigid = weight((delta[:, None, :] - tkp[None]).norm(dim=2))
+    off = (project(rigid, tf).reshape(n, -1) @ two).reshape(n, kpn, 3)
+    assert 0.003 < float(off.std()) < 0.03
+    dist = (delta[:, None, :] - (tkp[None] + off[ids[:, 1]])).norm(dim=2)
+    deformed = weight(dist)
+    ref_out = project(deformed, tf).reshape(n, -1) @ tw
+    with torch.no_grad():
+        out_mag = project(deformed, tf.abs()).reshape(n, -1) @ tw.abs()
+    fit = torch.full((n, kpn), float("inf"), **f64).scatter_reduce(
+        0, ids[:, 1][:, None].expand(-1, kpn), (dist / sigma) ** 2, "amin")
+    kpd = tkp[None] + off
+    kd = (kpd[:, None] - kpd[:, :, None] + 1e-300).norm(dim=3)
+    rep = weight(kd) * (1 - torch.eye(kpn, **f64))[None]
+    ref_loss = fit.sum() + rep.sum()
+
+    cloud = pc.PointCloud(dev(pts), dev(bids), batch)
+    conv = layers.KPConv(c, c, custom_kernel_points=kp, kp_interpolation=kind, weights=dev(wts),
+                         deformable=True, offset_weights=dev(woff))
+    tfeat = dev(feat).requires_grad_(True)
+    out = conv(tfeat, cloud, cloud, radius, kernel_influence_dist=influence)
+    loss = conv.regularization_loss()
+    assert_rel_t(out.detach(), ref_out.detach(), out_mag, tol=2e-5)
+    np.testing.assert_allclose(float(loss.detach()), float(ref_loss.detach()), rtol=REL)
+
+    up = torch.tensor(rng.standard_normal((n, c)).astype(np.float32)).cuda()
+    (out * up).sum().backward(retain_graph=True)
+    (ref_out * up.double()).sum().backward(retain_graph=True)
+
+    def normwise(got, expect, tol):
+        err = float((got.double() - expect).abs().max())
+        assert err <= tol * float(expect.abs().max()), err / float(expect.abs().max())
+
+    normwise(tfeat.grad, tf.grad, 2e-5)
+    normwise(conv.weights.grad, tw.grad, 2e-5)
+    normwise(conv.offset_weights.grad, two.grad, 2e-5)
+    for t in (tfeat, conv.weights, conv.offset_weights, tf, tw, two):
+        t.grad = None
+    loss.backward()
+    ref_loss.backward()
+    normwise(conv.offset_weights.grad, two.grad, 2e-5)
+    normwise(tfeat.grad, tf.grad, 2e-5)
+
+
+def test_config5_kpconv_at_full_scene_size():
+    """Configuration 5 at its real size (8 clouds, ~0.8 M points, ~30 M pairs, 128 -> 128,
+    15 kernel points at 0.6 r; linear and Gaussian with sigma = 0.3 r): sampled rows of
+    the output and of the feature gradient in float64 on the layer's own pair table
+    (whose integer parity is pinned elsewhere), linearity in the features, and the
+    adjoint identities <up, conv(x)> == <dfeat, x> == <dW, W>."""
+    from tensorflow_graphics_point_clouds_amd import layers, pc, synthetic
+    cfg = synthetic.config5()
+    cloud = pc.PointCloud(dev(cfg["points"]), dev(cfg["batch_ids"]), cfg["batch_size"])
+    radius, c, kpn = cfg["radius"], 128, 15
+    n = cloud._points.shape[0]
+    kp = synthetic.spherical_kernel_points(15, rotate=False) * 0.8
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    x = torch.randn((n, c), device="cuda", generator=gen).requires_grad_(True)
+    y = torch.randn((n, c), device="cuda", generator=gen)
+    up = torch.randn((n, c), device="cuda", generator=gen)
+    pts = cloud._points.double()
+    tkp = torch.as_tensor(kp.astype(np.float64) * 0.75).cuda()
+    nbh = None
+    for kind, influence in (("linear", None), ("gaussian", 0.3 * radius)):
+        sigma = 1.0 if influence is None else influence / radius
+        conv = layers.KPConv(c, c, custom_kernel_points=kp, kp_interpolation=kind, seed=2)
+        x.grad = None
+        out = conv(x, cloud, cloud, radius, neighborhood=nbh, kernel_influence_dist=influence)
+        nbh = conv.last_neighborhood
+        out.backward(up)
+        dfeat, dw = x.grad, conv.weights.grad
+        with torch.no_grad():
+            out_y = conv(y, cloud, cloud, radius, neighborhood=nbh,
+                         kernel_influence_dist=influence)
+            out_xy = conv(x.detach() + 2 * y, cloud, cloud, radius, neighborhood=nbh,
+                          kernel_influence_dist=influence)
+            assert float((out_xy - (out + 2 * out_y)).abs().max()) <= \
+                2e-5 * float(out_xy.abs().max())
+        terms = up.double() * out.detach().double()
+        lhs, scale = float(terms.sum()), float(terms.abs().sum())
+        assert abs(lhs - float((dfeat.double() * x.detach().double()).sum())) <= REL * scale
+        assert abs(lhs - float((dw.double() * conv.weights.detach().double()).sum())) <= REL * scale
+
+        ids = nbh._original_neigh_ids.long()
+        ranges = nbh._samples_neigh_ranges.long()
+        w3 = conv.weights.detach().double().reshape(c, kpn, c)          # [C, KP, F]
+        rng = np.random.default_rng(0)
+        picks = torch.as_tensor(rng.choice(n, 120, replace=False), device="cuda")
+        starts = torch.where(picks > 0, ranges[(picks - 1).clamp(min=0)], torch.zeros_like(picks))
+
+        def basis_of(seg):
+            diff = (pts[ids[seg, 0]] - pts[ids[seg, 1]]) / radius
+            dist = (diff[:, None, :] - tkp[None]).norm(dim=2)
+            if kind == "linear":
+                return torch.relu(1 - dist / sigma)
+            return torch.exp(-(dist / (sigma / 3)) ** 2)
+
+        xs, ups = x.detach().double(), up.double()
+        pair_key = ids[:, 0] * n + ids[:, 1]
+        order = torch.argsort(pair_key)
+        sorted_key = pair_key[order]
+        for centre, a, e in zip(picks.tolist(), starts.tolist(), ranges[picks].tolist()):
+            seg = torch.arange(a, e, device="cuda")
+            assert bool((ids[seg, 1] == centre).all())
+            bas = basis_of(seg)
+            proj = torch.einsum("mc,mk->ck", xs[ids[seg, 0]], bas)
+            pmag = torch.einsum("mc,mk->ck", xs[ids[seg, 0]].abs(), bas)
+            expect = torch.einsum("ck,ckf->f", proj, w3)
+            mag = torch.einsum("ck,ckf->f", pmag, w3.abs())
+            assert_rel_t(out[centre].detach(), expect, mag)
+            # feature gradient of point `centre`: the pairs (centre, i); the self-
+            # neighbourhood is symmetric, so the i are the points of its own segment
+            centres = ids[seg, 0]
+            tseg = order[torch.searchsorted(sorted_key, centre * n + centres)]
+            assert bool((ids[tseg, 0] == centre).all()) and bool((ids[tseg, 1] == centres).all())
+            bt = basis_of(tseg)
+            dproj = torch.einsum("mf,ckf->mck", ups[centres], w3)
+            dmag = torch.einsum("mf,ckf->mck", ups[centres].abs(), w3.abs())
+            assert_rel_t(dfeat[centre], torch.einsum("mck,mk->c", dproj, bt),
+                         torch.einsum("mck,mk->c", dmag, bt))
+
+
+# ------------------------------------------------------------ configuration 4 ----
+
+def _chunked_dot(a, b, chunk=1 << 27):
+    """(sum a*b, sum |a*b|) in float64 over flat views, a slice at a time."""
+    a, b = a.reshape(-1), b.reshape(-1)
+    s = t = 0.0
+    for lo in range(0, a.numel(), chunk):
+        p = a[lo:lo + chunk].double() * b[lo:lo + chunk].double()
+        s += float(p.sum())
+        t += float(p.abs().sum())
+    return s, t
+
+
+@pytest.mark.parametrize("radius", [0.04, 0.06])
+def test_config4_basis_proj_beyond_int32_element_offsets(radius):
+    """Dense configuration at its real size: 4 x 200k uniform points, C = 128, K = 32.
+    The projection holds N*C*K = 3.28e9 elements (offsets pass 2^31 from centre 524 288
+    on); at radius 0.06 the basis and its gradient hold M*K = 4.35e9.  Rows beyond
+    element 2^31 of the projection, of the basis gradient and rows of the feature
+    gradient are recomputed in float64 on the device from the GPU's own pair table, and
+    <up, proj> == <dbasis, basis> == <dfeat, feat> over the whole tensors."""
+    from tensorflow_graphics_point_clouds_amd import pc, synthetic, tfg_custom_ops as ops
+    cfg = synthetic.config4()
+    c, k = cfg["c_in"], cfg["basis"]
+    cloud = pc.PointCloud(dev(cfg["points"]), dev(cfg["batch_ids"]), cfg["batch_size"])
+    nbh = pc.Neighborhood(pc.Grid(cloud, radius), radius)
+    ids, ranges = nbh._original_neigh_ids, nbh._samples_neigh_ranges
+    n, m = ranges.shape[0], ids.shape[0]
+    assert n * c * k > 2 ** 31
+    if radius == 0.06:
+        assert m * k > 2 ** 32
+    gen = torch.Generator(device="cuda").manual_seed(4)
+    basis = torch.rand((m, k), device="cuda", generator=gen)
+    feat = torch.randn((n, c), device="cuda", generator=gen)
+    out = ops._basis_proj_raw(basis, feat, ids, ranges)
+    up = torch.randn(out.shape, device="cuda", generator=gen)
+    dbasis, dfeat = ops.basis_proj_grads(basis, feat, ids, ranges, up)
+    torch.cuda.synchronize()
+
+    first_beyond = 2 ** 31 // (c * k)                    # first centre whose row starts past 2^31
+    rng = np.random.default_rng(int(radius * 100))
+    picks = np.concatenate([rng.integers(first_beyond, n, 40), [first_beyond, n - 1],
+                            rng.integers(0, first_beyond, 8)])
+    ends = ranges.long()
+    idl = ids.long()
+    for centre in picks.tolist():
+        a = int(ends[centre - 1]) if centre > 0 else 0
+        e = int(ends[centre])
+        assert bool((idl[a:e, 1] == centre).all())
+        f = feat[idl[a:e, 0]].double()
+        b = basis[a:e].double()
+        assert_rel_t(out[centre], torch.einsum("mc,mk->ck", f, b),
+                     torch.einsum("mc,mk->ck", f.abs(), b))
+        g = up[centre].double()
+        assert_rel_t(dbasis[a:e], torch.einsum("ck,mc->mk", g, f),
+                     torch.einsum("ck,mc->mk", g.abs(), f.abs()))
+    # the last rows of the basis gradient (beyond element 2^32 at radius 0.06)
+    assert (m - 1) * k > (2 ** 32 if radius == 0.06 else 2 ** 30)
+    # feature gradient of sampled points: all pairs whose neighbour is that point
+    order = torch.argsort(idl[:, 0], stable=True)
+    sorted_pt = idl[order, 0]
+    js = torch.as_tensor(rng.integers(0, n, 24), device="cuda")
+    los, his = torch.searchsorted(sorted_pt, js).tolist(), torch.searchsorted(sorted_pt, js + 1).tolist()
+    for j, lo, hi in zip(js.tolist(), los, his):
+        rows = order[lo:hi]
+        g = up[idl[rows, 1]].double()                                  # [len, C, K]
+        b = basis[rows].double()
+        assert_rel_t(dfeat[j], torch.einsum("mck,mk->c", g, b),
+                     torch.einsum("mck,mk->c", g.abs(), b))
+    lhs, scale = _chunked_dot(up, out)
+    rb, _ = _chunked_dot(dbasis, basis)
+    rf, _ = _chunked_dot(dfeat, feat)
+    assert abs(lhs - rb) <= REL * scale and abs(lhs - rf) <= REL * scale
+
+
+@pytest.mark.parametrize("radius", [0.04, 0.06])
+def test_config4_poisson_disk_sampling_at_full_size(radius):
+    """Poisson-disk sampling of the 4 x 200k uniform clouds: no two selected points of a
+    cloud lie within the radius of each other, and every point has a selected point of
+    its cloud within the radius (the sample is maximal).  Checked by brute force on the
+    device with the same float32 expression as the neighbour test, one rounding per
+    operation: sum_d ((a_d - b_d) / r)^2 < 1."""
+    from tensorflow_graphics_point_clouds_amd import pc, synthetic
+    cfg = synthetic.config4()
+    cloud = pc.PointCloud(dev(cfg["points"]), dev(cfg["batch_ids"]), cfg["batch_size"])
+    sampled, sel = pc.poisson_disk_sampling(cloud, radius, return_ids=True)
+    sel = sel.long()
+    assert torch.equal(sampled._points, cloud._points[sel])
+    assert torch.equal(sampled._batch_ids, cloud._batch_ids[sel])
+    assert int(torch.unique(sel).numel()) == sel.numel()
+    inv_r = torch.reciprocal(torch.full((3,), radius, dtype=torch.float32, device="cuda"))
+    for b in range(cfg["batch_size"]):
+        pts = cloud._points[cloud._batch_ids == b]
+        chosen = sampled._points[sampled._batch_ids == b]
+        assert 0 < chosen.shape[0] < pts.shape[0]
+
+        def within(block):                       # [rows, S] bool
+            d = (block[:, None, :] - chosen[None, :, :]) * inv_r
+            sq = d * d
+            return (sq[..., 0] + sq[..., 1]) + sq[..., 2] < 1.0
+
+        step = max(1, (1 << 26) // chosen.shape[0])
+        for lo in range(0, pts.shape[0], step):
+            assert bool(within(pts[lo:lo + step]).any(dim=1).all())          # maximal
+        for lo in range(0, chosen.shape[0], step):
+            hits = within(chosen[lo:lo + step]).sum(dim=1)
+            assert bool((hits == 1).all())                                   # itself only

@@ -256,3 +256,87 @@ def test_pooling_matches_loops(oracle):
     for b in range(2):
         np.testing.assert_allclose(gm[b], feat[g.batch_ids == b].max(axis=0))
         np.testing.assert_allclose(ga[b], feat[g.batch_ids == b].astype(np.float64).mean(axis=0))
+
+
+@pytest.mark.parametrize("kind", ["linear", "gaussian"])
+@pytest.mark.parametrize("with_offsets", [False, True])
+def test_kp_basis_matches_per_pair_loop(oracle, kind, with_offsets):
+    """kernel_point_conv_test.py:61-98 computes the correlation of a pair with a kernel
+    point as max(1 - |d - kp| / sigma, 0); KPConv.py:29-57 adds the Gaussian
+    exp(-(dist / (sigma/3))^2), KPConv.py:369-375 the per-centre offsets added to the
+    kernel points.  Scalar loops over pairs and kernel points, written with math.* only."""
+    import math
+    rng = np.random.default_rng(71)
+    m, k, d, sigma = 37, 5, 3, 0.8
+    diff = (rng.random((m, d)) * 2 - 1).astype(np.float32)
+    kp = (rng.random((k, d)) * 1.2 - 0.6).astype(np.float32)
+    off = (0.1 * rng.standard_normal((m, k, d))).astype(np.float32) if with_offsets else None
+    got, dist = oracle.kp_basis(diff, kp, sigma, kind, off)
+    assert got.shape == (m, k) and dist.shape == (m, k)
+    for p in range(m):
+        for q in range(k):
+            centre = [float(kp[q, a]) + (float(off[p, q, a]) if with_offsets else 0.0)
+                      for a in range(d)]
+            r = math.sqrt(sum((float(diff[p, a]) - centre[a]) ** 2 for a in range(d)))
+            if kind == "linear":
+                expect = max(1.0 - r / sigma, 0.0)
+            else:
+                expect = math.exp(-(r / (sigma / 3.0)) ** 2)
+            assert abs(dist[p, q] - r) <= 1e-12
+            assert abs(got[p, q] - expect) <= 1e-12
+
+
+def test_kp_basis_closed_form_cases(oracle):
+    """A pair that sits on a kernel point has weight 1 in both correlations; at a
+    distance of sigma the linear weight is 0 and the Gaussian one exp(-9); beyond sigma
+    the linear weight stays 0; a distance of sigma/3 gives 2/3 and exp(-1)."""
+    sigma = 0.5
+    kp = np.array([[0.0, 0.0, 0.0], [0.3, -0.4, 0.0]])
+    diff = np.array([[0.0, 0.0, 0.0],            # on kernel point 0, 0.5 = sigma from 1
+                     [0.3, -0.4, 0.0],           # on kernel point 1
+                     [0.0, 0.0, 0.9],            # beyond sigma from both
+                     [0.0, 0.0, sigma / 3]])     # sigma/3 from kernel point 0
+    lin, dist = oracle.kp_basis(diff, kp, sigma, "linear")
+    gau, _ = oracle.kp_basis(diff, kp, sigma, "gaussian")
+    np.testing.assert_allclose(dist[0], [0.0, 0.5], atol=1e-15)
+    np.testing.assert_allclose(lin[0], [1.0, 0.0], atol=1e-15)
+    np.testing.assert_allclose(gau[0], [1.0, np.exp(-9.0)], rtol=1e-12)
+    np.testing.assert_allclose(lin[1], [0.0, 1.0], atol=1e-15)
+    np.testing.assert_allclose(gau[1], [np.exp(-9.0), 1.0], rtol=1e-12)
+    assert np.all(lin[2] == 0.0)
+    np.testing.assert_allclose(lin[3, 0], 2.0 / 3.0, rtol=1e-12)
+    np.testing.assert_allclose(gau[3, 0], np.exp(-1.0), rtol=1e-12)
+    # an offset that moves kernel point 1 onto the pair gives weight 1 again
+    off = np.zeros((4, 2, 3))
+    off[2, 1] = np.array([0.0, 0.0, 0.9]) - kp[1]
+    lin_o, _ = oracle.kp_basis(diff, kp, sigma, "linear", off)
+    assert lin_o[2, 1] == 1.0 and lin_o[2, 0] == 0.0
+
+
+@pytest.mark.parametrize("activation", ["relu", "leaky_relu", "elu"])
+def test_mc_basis_activations_hand_values(oracle, activation):
+    """MCConv.py:27-31, 163-171: basis = act(d W + b) / pdf with relu, leaky relu
+    (slope 0.2, TensorFlow's default) or ELU, one column block per kernel MLP.  The
+    pre-activations are chosen by hand (-2, -0.5, 0, 0.25, 3) so every branch is hit."""
+    import math
+    z = [-2.0, -0.5, 0.0, 0.25, 3.0]
+    # d = (1, 0): column h of the first weight row is the pre-activation; second MLP
+    # sees the same values through the bias with a zero weight
+    w = np.zeros((2, 2, 5))
+    b = np.zeros((2, 1, 5))
+    w[0, 0] = z
+    b[1, 0] = z[::-1]
+    diff = np.array([[1.0, 0.0], [1.0, 7.0]])
+    pdf = np.array([2.0, 0.5])
+    act = {"relu": lambda x: max(x, 0.0),
+           "leaky_relu": lambda x: x if x > 0 else 0.2 * x,
+           "elu": lambda x: x if x > 0 else math.exp(x) - 1.0}[activation]
+    got = oracle.mc_basis(diff, pdf, w, b, activation)
+    assert got.shape == (2, 10)
+    for p in range(2):
+        expect = [act(v) / pdf[p] for v in z] + [act(v) / pdf[p] for v in z[::-1]]
+        np.testing.assert_allclose(got[p], expect, rtol=1e-14, atol=0)
+    if activation == "leaky_relu":
+        assert got[0, 0] == -0.4 / 2.0 and got[0, 1] == -0.1 / 2.0
+    if activation == "elu":
+        np.testing.assert_allclose(got[1, 0], (math.exp(-2.0) - 1.0) / 0.5, rtol=1e-14)
