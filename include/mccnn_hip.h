@@ -395,6 +395,27 @@ int mccnn_mc_basis_grads(mccnn_stream_t stream, int64_t num_neighbors,
                          size_t workspace_bytes, float *weight_grads_out,
                          float *bias_grads_out);
 
+/* mccnn_mc_basis_grads without a workspace argument and without any allocation:
+ * the per-block partial sums live in a static device array of the library
+ * (1.75 MiB per device, enough for the largest shape the op accepts: 6
+ * dimensions, 64 basis functions; anything larger is refused with status 1).
+ * No counterpart in the reference.  It is for callers that cannot allocate:
+ * code under HIP graph capture, serving loops, harnesses that forbid
+ * hipMalloc.  Same arguments, results bit-identical to mccnn_mc_basis_grads.
+ * All calls on one device share that device's array: calls that overlap on
+ * one device (two streams, two threads) race; serialise them.  The first call
+ * on a device looks the array's address up (hipGetSymbolAddress, no
+ * allocation); make one call before starting a graph capture. */
+int mccnn_mc_basis_grads_static(mccnn_stream_t stream, int64_t num_neighbors,
+                                int num_dims, int num_basis, int activation,
+                                const float *points_in, const float *points_out,
+                                const int32_t *neighbors,
+                                const float *inv_radii, const float *weights,
+                                const float *biases, int num_mlps,
+                                const float *pdf, const float *basis_grads,
+                                float *weight_grads_out,
+                                float *bias_grads_out);
+
 /* Fused Monte-Carlo convolution projection: mccnn_mc_basis followed by
  * mccnn_basis_proj (MCConv.py:163-177) in one kernel that evaluates the basis in
  * registers, and the matching backward (gradients of features, kernel weights

@@ -4,6 +4,8 @@
 //   kernel-point convolution pylib/pc/layers/KPConv.py:29-57, 193-213
 // One lane per (pair, basis column): the K lanes of a pair read the same two
 // points (broadcast loads) and write one contiguous basis row.
+#include <mutex>
+
 #include "common.h"
 #include "fill.h"
 
@@ -353,29 +355,31 @@ extern "C" size_t mccnn_mc_basis_grads_workspace_bytes(int num_dims, int num_bas
   return align256(sizeof(float) * (size_t)kGradBlocks * (num_dims + 1) * num_basis);
 }
 
-extern "C" int mccnn_mc_basis_grads(mccnn_stream_t stream, int64_t num_neighbors, int num_dims,
-                                    int num_basis, int activation, const float *points_in,
-                                    const float *points_out, const int32_t *neighbors,
-                                    const float *inv_radii, const float *weights,
-                                    const float *biases, int num_mlps, const float *pdf,
-                                    const float *basis_grads, void *workspace,
-                                    size_t workspace_bytes, float *weight_grads_out,
-                                    float *bias_grads_out) {
-  MCCNN_REQUIRE(valid_dims(num_dims), "mc_basis_grads expects a valid number of dimensions");
-  MCCNN_REQUIRE(valid_basis_count(num_basis),
-                "mc_basis_grads expects 8, 16, 32 or 64 basis functions");
+// Validation and the two launches shared by mccnn_mc_basis_grads (partials in the caller's
+// workspace) and mccnn_mc_basis_grads_static (partials in this library's static array).
+static int mc_basis_grads_run(const char *op, mccnn_stream_t stream, int64_t num_neighbors,
+                              int num_dims, int num_basis, int activation,
+                              const float *points_in, const float *points_out,
+                              const int32_t *neighbors, const float *inv_radii,
+                              const float *weights, const float *biases, int num_mlps,
+                              const float *pdf, const float *basis_grads, float *partials,
+                              size_t partials_bytes, float *weight_grads_out,
+                              float *bias_grads_out) {
+  MCCNN_REQUIRE(valid_dims(num_dims), "%s expects a valid number of dimensions", op);
+  MCCNN_REQUIRE(valid_basis_count(num_basis), "%s expects 8, 16, 32 or 64 basis functions", op);
   MCCNN_REQUIRE(num_mlps > 0 && num_basis % num_mlps == 0,
-                "mc_basis_grads expects the number of basis functions to be divisible by the "
-                "number of kernel MLPs");
-  MCCNN_REQUIRE(activation >= 0 && activation <= 2, "mc_basis_grads expects a known activation");
-  MCCNN_REQUIRE(num_neighbors >= 0, "mc_basis_grads expects a non-negative size");
-  MCCNN_REQUIRE(weight_grads_out && bias_grads_out && workspace,
-                "mc_basis_grads received a null tensor");
-  MCCNN_REQUIRE(workspace_bytes >= mccnn_mc_basis_grads_workspace_bytes(num_dims, num_basis),
-                "mc_basis_grads workspace too small");
+                "%s expects the number of basis functions to be divisible by the number of "
+                "kernel MLPs", op);
+  MCCNN_REQUIRE(activation >= 0 && activation <= 2, "%s expects a known activation", op);
+  MCCNN_REQUIRE(num_neighbors >= 0, "%s expects a non-negative size", op);
+  MCCNN_REQUIRE(weight_grads_out && bias_grads_out && partials, "%s received a null tensor", op);
+  MCCNN_REQUIRE(partials_bytes >= mccnn_mc_basis_grads_workspace_bytes(num_dims, num_basis),
+                "%s: scratch of %zu bytes is too small for %d dimensions and %d basis "
+                "functions (%zu bytes needed)", op, partials_bytes, num_dims, num_basis,
+                mccnn_mc_basis_grads_workspace_bytes(num_dims, num_basis));
   MCCNN_REQUIRE(num_neighbors == 0 || (points_in && points_out && neighbors && inv_radii &&
                                        weights && biases && pdf && basis_grads),
-                "mc_basis_grads received a null tensor");
+                "%s received a null tensor", op);
   hipStream_t s = as_stream(stream);
   const int rows = 256 / num_basis;
   int blocks = (int)((num_neighbors + rows - 1) / rows);
@@ -385,15 +389,83 @@ extern "C" int mccnn_mc_basis_grads(mccnn_stream_t stream, int64_t num_neighbors
                                                 0, s, num_neighbors, num_basis,
                                                 num_basis / num_mlps, activation, points_in,
                                                 points_out, (const int2 *)neighbors, inv_radii,
-                                                weights, biases, pdf, basis_grads,
-                                                (float *)workspace));
+                                                weights, biases, pdf, basis_grads, partials));
   MCCNN_LAUNCH_CHECK();
   const int outs = (num_dims + 1) * num_basis;
   hipLaunchKernelGGL(mc_basis_grads_reduce_kernel, dim3(outs), dim3(kWave), 0, s,
                      blocks, num_dims, num_basis, num_basis / num_mlps,
-                     (const float *)workspace, weight_grads_out, bias_grads_out);
+                     (const float *)partials, weight_grads_out, bias_grads_out);
   MCCNN_LAUNCH_CHECK();
   return MCCNN_OK;
+}
+
+extern "C" int mccnn_mc_basis_grads(mccnn_stream_t stream, int64_t num_neighbors, int num_dims,
+                                    int num_basis, int activation, const float *points_in,
+                                    const float *points_out, const int32_t *neighbors,
+                                    const float *inv_radii, const float *weights,
+                                    const float *biases, int num_mlps, const float *pdf,
+                                    const float *basis_grads, void *workspace,
+                                    size_t workspace_bytes, float *weight_grads_out,
+                                    float *bias_grads_out) {
+  return mc_basis_grads_run("mc_basis_grads", stream, num_neighbors, num_dims, num_basis,
+                            activation, points_in, points_out, neighbors, inv_radii, weights,
+                            biases, num_mlps, pdf, basis_grads, (float *)workspace,
+                            workspace_bytes, weight_grads_out, bias_grads_out);
+}
+
+// Per-block partial sums of mccnn_mc_basis_grads_static: the largest shape the op accepts
+// (6 dimensions, 64 basis functions) times the fixed number of blocks, 1.75 MiB.  Every
+// device the library runs on holds its own copy until the process ends.  Host code never
+// passes the array's name to a kernel (there it is a host-side stand-in, not a device
+// address): it asks the runtime once per device for the address and uses that.
+constexpr size_t kStaticScratchFloats = (size_t)kGradBlocks * (kMaxDims + 1) * 64;
+static __device__ __align__(256) float scratch[kStaticScratchFloats];
+
+constexpr int kMaxDevices = 64;
+static std::mutex g_scratch_mutex;
+static float *g_scratch_ptr[kMaxDevices];      // address of `scratch` on each device
+
+// The current device's copy of `scratch` (looked up on the first call on that device).
+static int static_scratch(float **out) {
+  int device = -1;
+  MCCNN_HIP_CHECK(hipGetDevice(&device));
+  MCCNN_REQUIRE(device >= 0 && device < kMaxDevices,
+                "mc_basis_grads_static supports device ordinals below %d (got %d)", kMaxDevices,
+                device);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[device] == nullptr) {
+    void *address = nullptr;
+    MCCNN_HIP_CHECK(hipGetSymbolAddress(&address, HIP_SYMBOL(scratch)));
+    MCCNN_REQUIRE(address != nullptr, "mc_basis_grads_static: no address for the static scratch");
+    g_scratch_ptr[device] = static_cast<float *>(address);
+  }
+  *out = g_scratch_ptr[device];
+  return MCCNN_OK;
+}
+
+extern "C" int mccnn_mc_basis_grads_static(mccnn_stream_t stream, int64_t num_neighbors,
+                                           int num_dims, int num_basis, int activation,
+                                           const float *points_in, const float *points_out,
+                                           const int32_t *neighbors, const float *inv_radii,
+                                           const float *weights, const float *biases,
+                                           int num_mlps, const float *pdf,
+                                           const float *basis_grads, float *weight_grads_out,
+                                           float *bias_grads_out) {
+  // sizes the static array cannot hold are refused before anything is launched
+  MCCNN_REQUIRE(num_dims <= kMaxDims && num_basis <= 64,
+                "mc_basis_grads_static holds partial sums for at most %d dimensions and 64 basis "
+                "functions (got %d and %d); use mc_basis_grads with a workspace", kMaxDims,
+                num_dims, num_basis);
+  float *partials = nullptr;
+  int rc = static_scratch(&partials);
+  if (rc != MCCNN_OK) return rc;
+  // Nothing in the array has to start at zero: every block that runs overwrites its own
+  // slots and the reduction reads the slots of exactly those blocks.
+  return mc_basis_grads_run("mc_basis_grads_static", stream, num_neighbors, num_dims, num_basis,
+                            activation, points_in, points_out, neighbors, inv_radii, weights,
+                            biases, num_mlps, pdf, basis_grads, partials,
+                            sizeof(float) * kStaticScratchFloats, weight_grads_out,
+                            bias_grads_out);
 }
 
 extern "C" int mccnn_kp_basis(mccnn_stream_t stream, int64_t num_neighbors, int num_dims,
