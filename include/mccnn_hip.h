@@ -530,16 +530,15 @@ int mccnn_kp_conv_project(mccnn_stream_t stream, int num_dims, int64_t num_pts,
  * with proj as produced by mccnn_mc_conv_project; the projection is handed from
  * the matrix-core accumulators to the final product through LDS and reaches HBM
  * only when proj_out [N_out, C, K] is not NULL.  final_weights is the dense
- * [C*K, F] matrix (several kernel MLPs: their [C*H, F/L] blocks placed on the
- * block diagonal).  workspace holds the weights re-ordered for the kernel
- * (mccnn_mc_conv_layer_workspace_bytes).  Covered shapes
- * (mccnn_mc_conv_layer_supported): D in {2,3}, K = 16, C and F in
- * {16,32,64,128}.  No counterpart among the reference's ops, which run the
- * projection and tf.matmul separately. */
+ * [C*K, F] matrix, kept in registers by every block for the whole launch.
+ * out_rows (optional, a permutation of 0..N_out-1) names the row of out (and of
+ * proj_out) that centre i is written to.  Covered shapes
+ * (mccnn_mc_conv_layer_supported): D in {2,3}, K = 16, C in {16,32,64}, F in
+ * {16,32,64,128}, C*K*F <= 65536.  Results are bit-reproducible.  No
+ * counterpart among the reference's ops, which run the projection and
+ * tf.matmul separately. */
 int mccnn_mc_conv_layer_supported(int num_dims, int num_features, int num_basis,
                                   int num_out_features);
-size_t mccnn_mc_conv_layer_workspace_bytes(int num_features, int num_basis,
-                                           int num_out_features);
 int mccnn_mc_conv_layer(mccnn_stream_t stream, int num_dims, int64_t num_pts,
                         const float *points_in, int num_features,
                         const float *features, int64_t num_samples,
@@ -548,8 +547,34 @@ int mccnn_mc_conv_layer(mccnn_stream_t stream, int num_dims, int64_t num_pts,
                         const float *inv_radii, int num_basis, int num_mlps,
                         int activation, const float *weights, const float *biases,
                         const float *pdf, int num_out_features,
-                        const float *final_weights, void *workspace,
-                        size_t workspace_bytes, float *proj_out, float *out);
+                        const float *final_weights, const int32_t *out_rows,
+                        float *proj_out, float *out);
+
+/* The same for the rigid kernel-point convolution (KPConv.py:165-232): the
+ * projection of mccnn_kp_conv_project (up to 16 kernel points, 16 basis columns,
+ * the columns past the last kernel point zero) times final_weights [C*16, F].
+ * Shapes as for mccnn_mc_conv_layer. */
+int mccnn_kp_conv_layer(mccnn_stream_t stream, int num_dims, int64_t num_pts,
+                        const float *points_in, int num_features,
+                        const float *features, int64_t num_samples,
+                        const float *points_out, int64_t num_neighbors,
+                        const int32_t *neighbors, const int32_t *ranges,
+                        const float *inv_radii, int num_kernel_points,
+                        const float *kernel_points, int kind, float sigma,
+                        int num_out_features, const float *final_weights,
+                        const int32_t *out_rows, float *proj_out, float *out);
+
+/* out[out_rows[n] or n, :] = x[n, :] * w: the product of a layer with its final
+ * weights (the tf.matmul of MCConv.py:187 / KPConv.py:226-230) for x [N, R] in
+ * HBM and w [R, F].  One block per compute unit keeps all of w in registers and
+ * streams x through LDS tiles of 16 rows, reading it exactly once; sums in a
+ * fixed order (bit-reproducible).  Supported: R in {256, 512, 1024}, F in {16,
+ * 32, 64, 128}, R*F <= 65536.  No counterpart among the reference's ops
+ * (TensorFlow's matmul). */
+int mccnn_final_product_supported(int num_cols_in, int num_cols_out);
+int mccnn_final_product(mccnn_stream_t stream, int64_t num_rows, int num_cols_in,
+                        const float *x, int num_cols_out, const float *w,
+                        const int32_t *out_rows, float *out);
 
 /* out[c, r] = sum_n x[n, c] * y[n, r]: the gradient of a layer's final weights
  * (the backward of the tf.matmul of MCConv.py:187 / KPConv.py:226-230), a product

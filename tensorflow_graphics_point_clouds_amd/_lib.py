@@ -45,7 +45,6 @@ def lib():
         handle.mccnn_last_error.restype = ctypes.c_char_p
         for name in ("mccnn_find_neighbors_workspace_bytes",
                      "mccnn_mc_basis_grads_workspace_bytes",
-                     "mccnn_mc_conv_layer_workspace_bytes",
                      "mccnn_mc_conv_project_grads_workspace_bytes",
                      "mccnn_pointconv_density_grads_workspace_bytes",
                      "mccnn_reorder_neighbors_workspace_bytes",

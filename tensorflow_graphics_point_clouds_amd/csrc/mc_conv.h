@@ -99,10 +99,10 @@ struct KpBasis {                   // kernel-point correlation (KPConv.py:29-57,
 };
 
 // acc[j] += projection of the pairs [a, b) of one centre for the channels
-// col*kCPL + j of the 16*kCPL-channel chunk starting at feat_base.  Rows are
-// row_bytes apart; every byte offset fits 32 bits (checked by the host).  p.pdf
-// may be null (weight 1).
-template <int kCPL, int D, class Basis>
+// col*kCPL + j (kStrided: col + 16*j) of the 16*kCPL-channel chunk starting at
+// feat_base.  Rows are row_bytes apart; every byte offset fits 32 bits (checked by
+// the host).  p.pdf may be null (weight 1).
+template <int kCPL, int D, class Basis, bool kStrided = false>
 __device__ __forceinline__ void project_pairs(const char *__restrict__ feat_base,
                                               unsigned row_bytes, const int2 *__restrict__ nbrs,
                                               int a, int b, const McParams<D> &p,
@@ -112,7 +112,7 @@ __device__ __forceinline__ void project_pairs(const char *__restrict__ feat_base
   float ir[D];
 #pragma unroll
   for (int d = 0; d < D; ++d) ir[d] = p.inv_radii[d];
-  const unsigned lane_off = col * kCPL * 4;
+  const unsigned lane_off = kStrided ? col * 4 : col * kCPL * 4;
   for (int m0 = a; m0 < b; m0 += kWave) {
     const int cnt = b - m0 < kWave ? b - m0 : kWave;
     float4 g = {0.0f, 0.0f, 0.0f, 0.0f};
@@ -142,7 +142,13 @@ __device__ __forceinline__ void project_pairs(const char *__restrict__ feat_base
         const int n = 4 * (t + u) + quarter;
         const float4 gn = stage->geo[n];
         const unsigned rn = stage->row[n];
-        f[u] = load_vec<kCPL>(reinterpret_cast<const float *>(feat_base + rn + lane_off), true);
+        if constexpr (kStrided) {
+#pragma unroll
+          for (int j = 0; j < kCPL; ++j)
+            f[u].v[j] = *reinterpret_cast<const float *>(feat_base + rn + lane_off + j * 64);
+        } else {
+          f[u] = load_vec<kCPL>(reinterpret_cast<const float *>(feat_base + rn + lane_off), true);
+        }
         w[u] = basis(gn);
       }
 #pragma unroll

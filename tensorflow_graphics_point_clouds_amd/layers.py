@@ -115,14 +115,11 @@ def _mc_project(weights, biases, features, points_in, points_out, neighbors, ran
 
 
 def _mc_layer(weights, biases, features, points_in, points_out, neighbors, ranges, inv_radii,
-              pdf, act, dense_weights, want_proj=False):
-    """Fused projection + product with the dense [C*K, F] final weights."""
+              pdf, act, dense_weights, out_rows=None, want_proj=False):
+    """Fused projection + product with the dense [C*K, F] final weights; rows of the
+    result (and of the projection, if asked for) go to `out_rows`."""
     num_mlps, dims, hidden = weights.shape
     k, c, f = num_mlps * hidden, features.shape[1], dense_weights.shape[1]
-    L = _lib.lib()
-    L.mccnn_mc_conv_layer_workspace_bytes.restype = _lib.csize
-    ws = _lib.workspace(L.mccnn_mc_conv_layer_workspace_bytes(cint(c), cint(k), cint(f)),
-                        features.device)
     out = torch.empty((ranges.shape[0], f), dtype=_F32, device=features.device)
     proj = None
     if want_proj:
@@ -132,8 +129,7 @@ def _mc_layer(weights, biases, features, points_in, points_out, neighbors, range
               ptr(points_out, _F32), i64(neighbors.shape[0]), ptr(neighbors, _I32),
               ptr(ranges, _I32), ptr(inv_radii, _F32), cint(k), cint(num_mlps), cint(act),
               ptr(weights, _F32), ptr(biases, _F32), ptr(pdf, _F32), cint(f),
-              ptr(dense_weights.contiguous(), _F32), ptr(ws), _lib.csize(ws.numel()), ptr(proj),
-              ptr(out))
+              ptr(dense_weights.contiguous(), _F32), ptr(out_rows), ptr(proj), ptr(out))
     return out, proj
 
 
@@ -175,6 +171,18 @@ def _projection_grad_product(x, w):
     return out
 
 
+def _final_product(x, w):
+    """x w for x [N, R] and the final weights w [R, F]."""
+    r, f = w.shape
+    if not _lib.lib().mccnn_final_product_supported(cint(r), cint(f)):
+        with _lib.region("gemm_final"):
+            return x @ w
+    out = torch.empty((x.shape[0], f), dtype=_F32, device=x.device)
+    _lib.call("final_product", stream(), i64(x.shape[0]), cint(r), ptr(x, _F32), cint(f),
+              ptr(w.contiguous(), _F32), ptr(None), ptr(out))
+    return out
+
+
 def _dense_final_weights(final_weights, c):
     """[L, C*H, G] per-MLP blocks -> dense [C*(L*H), L*G] with zero off-diagonal blocks."""
     l, ch, g = final_weights.shape
@@ -211,17 +219,14 @@ class _MCConvLayer(torch.autograd.Function):
         dense = _dense_final_weights(final_weights, features.shape[1])
         if fuse_final:
             out, _ = _mc_layer(weights, biases, feats, view.points_in, view.points_out,
-                               view.table, view.ranges, inv_radii, pdf, act, dense)
-            if view.centre_order is not None:
-                with _lib.region("permute_rows"):
-                    out = torch.empty_like(out).index_copy_(0, view.centre_order, out)
+                               view.table, view.ranges, inv_radii, pdf, act, dense,
+                               view.centre_rows)
         else:
             # rows of the projection go straight to the centres' original positions
             proj = _mc_project(weights, biases, feats, view.points_in, view.points_out,
                                view.table, view.ranges, inv_radii, pdf, act,
                                view.centre_rows)
-            with _lib.region("gemm_out"):
-                out = proj.reshape(proj.shape[0], -1) @ dense
+            out = _final_product(proj.reshape(proj.shape[0], -1), dense)
         ctx.save_for_backward(weights, biases, final_weights, feats, features, inv_radii)
         ctx.neighborhood, ctx.act, ctx.fuse_final = neighborhood, act, fuse_final
         return out
@@ -259,18 +264,16 @@ class _MCConvLayer(torch.autograd.Function):
         w2 = dense.reshape(c, k, f).permute(2, 1, 0).reshape(f * k, c)
         neg = -inv_radii
         if ctx.fuse_final:
+            # rows of Q and of dfeat go straight to the points' original positions
             dfeat, q = _mc_layer(weights, biases, dout, view.points_out, view.points_in,
                                  view.table_t, view.ranges_t, neg, pdf_t, ctx.act, w2,
-                                 want_proj=True)
-            with _lib.region("permute_rows"):
-                dfeat = torch.empty_like(dfeat).index_copy_(0, view.point_order, dfeat)
-            ddense = _weight_grad_product(feats, q.reshape(feats.shape[0], f * k))
+                                 view.point_rows, want_proj=True)
+            ddense = _weight_grad_product(features, q.reshape(features.shape[0], f * k))
         else:
             # rows of Q (and so of dfeat) go straight to the points' original positions
             q = _mc_project(weights, biases, dout, view.points_out, view.points_in,
                             view.table_t, view.ranges_t, neg, pdf_t, ctx.act, view.point_rows)
-            with _lib.region("gemm_dfeat"):
-                dfeat = q.reshape(q.shape[0], f * k) @ w2
+            dfeat = _final_product(q.reshape(q.shape[0], f * k), w2)
             ddense = _weight_grad_product(features, q.reshape(features.shape[0], f * k))
         ddense = ddense.reshape(c, f, k).permute(0, 2, 1)            # [C, K, F]
         if l == 1:
@@ -537,8 +540,7 @@ class _PointConvLayer(torch.autograd.Function):
         feats = _gather_rows(features, view.point_rows)
         proj = _mc_project(weights, biases, feats, view.points_in, view.points_out, view.table,
                            view.ranges, ones, y, act, view.centre_rows)
-        with _lib.region("gemm_out"):
-            out = proj.reshape(proj.shape[0], -1) @ final_weights[0]
+        out = _final_product(proj.reshape(proj.shape[0], -1), final_weights[0])
         ctx.save_for_backward(weights, biases, final_weights, feats, features, per_point, max_pdf,
                               y, y_t, ones, *mlp)
         ctx.neighborhood, ctx.act = neighborhood, act
@@ -586,8 +588,7 @@ class _PointConvLayer(torch.autograd.Function):
         dfeat = None
         if ctx.needs_input_grad[7]:
             w_t = dense.reshape(c, k, f).permute(2, 1, 0).reshape(f * k, c)
-            with _lib.region("gemm_dfeat"):
-                dfeat = q @ w_t
+            dfeat = _final_product(q, w_t)
         ddense = _weight_grad_product(features, q).reshape(c, f, k).permute(0, 2, 1)
         dfinal = ddense.reshape(1, c * k, f)
         return (dw, db, dfinal, dmlp[0:16].reshape(1, 16), dmlp[16:32].reshape(1, 16),
@@ -834,8 +835,7 @@ class _KPConvRigidLayer(torch.autograd.Function):
         # rows of the projection go straight to the centres' original positions
         proj = _kp_project(feats, view.points_in, view.points_out, view.table, view.ranges,
                            inv_radii, kernel_points, k, kind, sigma, view.centre_rows)
-        with _lib.region("gemm_out"):
-            out = proj.reshape(proj.shape[0], -1) @ dense_weights
+        out = _final_product(proj.reshape(proj.shape[0], -1), dense_weights)
         ctx.save_for_backward(dense_weights, feats, features, inv_radii, kernel_points)
         ctx.neighborhood, ctx.k, ctx.kind, ctx.sigma = neighborhood, k, kind, sigma
         return out
@@ -856,8 +856,7 @@ class _KPConvRigidLayer(torch.autograd.Function):
         dfeat = ddense = None
         if ctx.needs_input_grad[1]:
             w2 = dense.reshape(c, k, f).permute(2, 1, 0).reshape(f * k, c)
-            with _lib.region("gemm_dfeat"):
-                dfeat = q @ w2
+            dfeat = _final_product(q, w2)
         if ctx.needs_input_grad[0]:
             ddense = _weight_grad_product(features, q).reshape(c, f, k).permute(0, 2, 1)
             ddense = ddense.reshape(c * k, f)

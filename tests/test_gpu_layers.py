@@ -384,6 +384,38 @@ def test_projection_grad_product_matches_float64(n, f, r):
         assert np.abs(got - expect).max() <= 1e-5 * np.abs(expect).max()
 
 
+@pytest.mark.parametrize("n,r,f", [(1, 256, 16), (15, 256, 128), (4099, 1024, 64), (20000, 512, 128),
+                                   (333, 1024, 32), (5000, 512, 32), (0, 1024, 64), (70001, 1024, 16)])
+def test_final_product_matches_float64(n, r, f):
+    """x w with all of w in the registers of each block, elementwise against float64
+    with the magnitude sum |x| |w| (1e-5), row permutation included; a second call must
+    return the same bits."""
+    from tensorflow_graphics_point_clouds_amd import _lib
+    from tensorflow_graphics_point_clouds_amd._lib import cint, i64, ptr, stream
+    assert _lib.lib().mccnn_final_product_supported(r, f) == 1
+    assert _lib.lib().mccnn_final_product_supported(2048, 64) == 0
+    assert _lib.lib().mccnn_final_product_supported(1024, 128) == 0
+    gen = torch.Generator(device="cuda").manual_seed(n + f)
+    x = torch.randn((n, r), device="cuda", generator=gen)
+    w = torch.randn((r, f), device="cuda", generator=gen)
+    rows = torch.randperm(n, device="cuda", generator=gen).int()
+    outs = []
+    for perm in (None, rows, rows):
+        out = torch.full((n, f), float("nan"), device="cuda")
+        _lib.call("final_product", stream(), i64(n), cint(r), ptr(x), cint(f), ptr(w), ptr(perm),
+                  ptr(out))
+        outs.append(out)
+    expect = x.double() @ w.double()
+    mag = x.double().abs() @ w.double().abs()
+    assert bool(((outs[0].double() - expect).abs() <= 1e-5 * mag).all())
+    assert torch.equal(outs[1], outs[2])
+    if n:
+        assert torch.equal(outs[1][rows.long()], outs[0])
+    with pytest.raises(ValueError):
+        _lib.call("final_product", stream(), i64(n), cint(2048), ptr(x), cint(64), ptr(w),
+                  ptr(None), ptr(outs[0]))
+
+
 def test_layers_accept_padded_input_and_return_padded_output():
     """Padded point clouds / features ([A, V, D], [A, V, C], sizes) give the same
     result as the segmented form, re-padded on request (layers/utils.py:22-49,
