@@ -31,7 +31,10 @@ def log(*a):
 
 
 def op_bytes(name, M, N_in, N_out, C, K, D):
-    """Algorithmic bytes of one launch of each op (fp32, int32 pair table)."""
+    """Operand bytes of one launch of each op (fp32, int32 pair table): every per-pair
+    gather counted at full width, as the survey's formulas do.  On grid-ordered inputs
+    most of the gathers are served by L2, so this figure can exceed what HBM moves; it is
+    reported as `operand_GBps`, never as a roofline fraction."""
     if name == "basis_proj":
         return 4 * (M * K + M * C + N_out * C * K) + 8 * M + 4 * N_out
     if name == "basis_proj_grads":
@@ -47,9 +50,59 @@ def op_bytes(name, M, N_in, N_out, C, K, D):
     return None
 
 
+def compulsory_bytes(name, M, N_in, N_out, C, K, D):
+    """HBM bytes one launch cannot avoid: every tensor counted once, whatever the number
+    of times its rows are gathered.  The roofline fraction of an op is this figure over
+    its launch time and the HBM peak, so it cannot exceed 1.
+
+      pair stream   8 M (table) [+ 4 M densities] [+ 4 M K basis rows]
+      coordinates   4 D (N_in + N_out)
+      features      4 N_in C        read once (not 4 M C)
+      projection    4 N_out C K     written (or read, for the gradient ops)
+      ranges        4 N_out
+    """
+    pairs = 8 * M
+    coords = 4 * D * (N_in + N_out)
+    feats = 4 * N_in * C
+    proj = 4 * N_out * C * K
+    if name == "basis_proj":
+        return pairs + 4 * M * K + feats + proj + 4 * N_out
+    if name == "basis_proj_grads":       # + basis gradient written, feature gradient written
+        return pairs + 2 * 4 * M * K + feats + proj + 4 * N_in * C + 4 * N_out
+    if name in ("mc_conv_project", "kp_conv_project"):
+        return pairs + (4 * M if name == "mc_conv_project" else 0) + coords + feats + proj + \
+            4 * N_out
+    if name == "mc_conv_project_grads":
+        return pairs + 4 * M + coords + feats + proj + 4 * N_out
+    if name in ("mc_basis", "mc_basis_grads"):
+        return pairs + 4 * M + coords + 4 * M * K
+    if name == "compute_pdf":
+        return pairs + 4 * D * N_in + 4 * N_out + 4 * N_out
+    if name == "compute_pdf_pt_grads":
+        return pairs + 4 * D * N_in + 8 * N_out + 4 * D * N_in
+    if name == "local_pool":
+        return pairs + feats + 4 * N_out * C + 4 * N_out
+    return None
+
+
+def roofline_entry(by, operand_by, ms, calls=1.0):
+    """GB/s and fraction of the HBM peak from compulsory bytes; `operand_GBps` beside it."""
+    gbps = by * calls / ms / 1e6
+    entry = {"GBps": round(gbps, 1), "frac_hbm_peak": round(gbps / HBM_PEAK_GBS, 4),
+             "compulsory_bytes": by}
+    if operand_by:
+        entry["operand_GBps"] = round(operand_by * calls / ms / 1e6, 1)
+        entry["operand_bytes"] = operand_by
+    if entry["frac_hbm_peak"] > 1.0:
+        entry["flag"] = "fraction above 1: the byte model counts more than HBM can have moved"
+    return entry
+
+
 def product_figures(name, N, C, K, CO):
     """(bytes, flops) of the dense products of the layer, one launch each."""
     flops = 2 * N * C * K * CO
+    if name == "final_product":               # [N, C*K] x [C*K, CO] and [N, CO*K] x [CO*K, C]
+        return 4 * (N * C * K + N * CO + C * K * CO), flops
     if name == "gemm_out":                    # [N, C*K] x [C*K, CO]
         return 4 * (N * C * K + N * CO + C * K * CO), flops
     if name == "gemm_dfeat":                  # [N, CO*K] x [CO*K, C]
@@ -61,20 +114,47 @@ def product_figures(name, N, C, K, CO):
     return None
 
 
+def _source_digest(files):
+    import hashlib
+    h = hashlib.sha256()
+    for f in files:
+        with open(os.path.join(ROOT, "tensorflow_graphics_point_clouds_amd", "csrc", f), "rb") as fh:
+            h.update(fh.read())
+    return h.hexdigest()[:16]
+
+
 def measured_traffic(op, workload):
-    """HBM-side bytes per launch from the committed counter summary (scaled
-    FETCH_SIZE + WRITE_SIZE), or None when the summary has no line for it."""
+    """HBM-side bytes per launch from the committed counter summary (scaled FETCH_SIZE +
+    WRITE_SIZE) -> (bytes, file) or (None, reason).  A summary names the kernel sources
+    it was taken from and their digest (`sources <digest> <file> ...`); when the sources
+    in the tree differ, the number belongs to another build and is not reported."""
     for fname in ("mcconv_layer_config3_hbm_traffic.txt",
                   "basis_proj_dense_case_hbm_traffic.txt"):
+        path = os.path.join(ROOT, "profiles", fname)
         try:
-            for line in open(os.path.join(ROOT, "profiles", fname)):
-                parts = line.split()
-                if len(parts) == 4 and parts[0] == "traffic_bytes" and parts[1] == op \
-                        and parts[2] == workload:
-                    return int(parts[3])
+            lines = open(path).read().splitlines()
         except OSError:
-            pass
-    return None
+            continue
+        digest = files = None
+        for line in lines:
+            parts = line.split()
+            if len(parts) >= 3 and parts[0] == "sources":
+                digest, files = parts[1], parts[2:]
+        for line in lines:
+            parts = line.split()
+            if len(parts) == 4 and parts[0] == "traffic_bytes" and parts[1] == op \
+                    and parts[2] == workload:
+                if digest is None:
+                    return None, "profiles/%s names no kernel sources" % fname
+                try:
+                    current = _source_digest(files)
+                except OSError:
+                    return None, "kernel sources of profiles/%s are missing" % fname
+                if current != digest:
+                    return None, ("profiles/%s was taken from other kernel sources (digest %s, "
+                                  "tree has %s)" % (fname, digest, current))
+                return int(parts[3]), "profiles/" + fname
+    return None, "no counter summary for %s on %s" % (op, workload)
 
 
 def build_scene(torch, pc, synthetic, scale):
@@ -121,50 +201,90 @@ def time_build(torch, pc, cloud, radius, reps=3):
     return grid, nbh, out
 
 
-def cpu_baseline(synthetic, sample_points=60000):
-    """MCConv fwd+bwd of the oracle (C with OpenMP, numpy GEMMs) on one cloud of
-    the same generator, cut to `sample_points` points."""
+def _set_cpu_threads(orc, n):
+    """Threads of the oracle's OpenMP loops and of numpy's BLAS."""
+    try:
+        orc.lib().omp_set_num_threads(int(n))
+    except AttributeError:
+        os.environ["OMP_NUM_THREADS"] = str(n)
+    try:
+        from threadpoolctl import threadpool_limits
+        return threadpool_limits(limits=int(n))
+    except Exception:
+        return None
+
+
+def cpu_baseline(synthetic):
+    """MCConv fwd+bwd of the oracle (C with OpenMP, numpy GEMMs) on the host cores:
+    the whole configuration-3 workload with all cores, and one of its clouds with a
+    single thread (bounded so that the default run stays within minutes)."""
     import numpy as np
     from oracle import mccnn_oracle as orc
-    cfg = synthetic.config3(scale=1.0, batch=1)
-    pts = cfg["points"][:sample_points]
-    n = len(pts)
-    bids = np.zeros(n, np.int32)
-    r = np.float32(cfg["radius"])
-    g = orc.Grid(pts, bids, 1, r)
-    nbh = orc.Neighborhood(g, r, pts, bids)
-    pdf = nbh.pdf_per_pair(0.2).astype(np.float32)
-    ids = nbh.original_neigh_ids
-    rng = np.random.default_rng(0)
-    C, K, CO = cfg["c_in"], cfg["hidden"], cfg["c_out"]
-    w, b, wo = synthetic.mcconv_weights(rng, 3, C, CO, K, 1)
-    feat = rng.standard_normal((n, C)).astype(np.float32)
-    up = rng.standard_normal((n, CO)).astype(np.float32)
-    inv_r = np.float32(1.0) / r
 
-    def step():
-        diff = (pts[ids[:, 0]] - pts[ids[:, 1]]) * inv_r
-        z = diff @ w[0] + b[0]
-        basis = (np.maximum(z, 0) / pdf[:, None]).astype(np.float32)
-        proj = orc.basis_proj_f32(basis, feat, ids, nbh.ranges)
-        out = proj.reshape(n, C * K) @ wo[0]
-        dproj = (up @ wo[0].T).reshape(n, C, K)
-        dwo = proj.reshape(n, C * K).T @ up
-        dbasis, dfeat = orc.basis_proj_grads_f32(basis, feat, ids, nbh.ranges, dproj)
-        dz = dbasis * (z > 0) / pdf[:, None]
-        dw = diff.T @ dz
-        db = dz.sum(axis=0)
-        return out, dwo, dfeat, dw, db
+    def prepare(cfg):
+        pts, bids = cfg["points"], cfg["batch_ids"]
+        n = len(pts)
+        r = np.float32(cfg["radius"])
+        t0 = time.perf_counter()
+        g = orc.Grid(pts, bids, cfg["batch_size"], r)
+        nbh = orc.Neighborhood(g, r, pts, bids)
+        pdf = nbh.pdf_per_pair(0.2).astype(np.float32)
+        build_s = time.perf_counter() - t0
+        ids = nbh.original_neigh_ids
+        rng = np.random.default_rng(0)
+        C, K, CO = cfg["c_in"], cfg["hidden"], cfg["c_out"]
+        w, b, wo = synthetic.mcconv_weights(rng, 3, C, CO, K, 1)
+        feat = rng.standard_normal((n, C)).astype(np.float32)
+        up = rng.standard_normal((n, CO)).astype(np.float32)
+        inv_r = np.float32(1.0) / r
 
-    step()
-    reps, t0 = 0, time.perf_counter()
-    while reps < 3 or time.perf_counter() - t0 < 10.0:
+        def step():
+            diff = (pts[ids[:, 0]] - pts[ids[:, 1]]) * inv_r
+            z = diff @ w[0] + b[0]
+            basis = (np.maximum(z, 0) / pdf[:, None]).astype(np.float32)
+            proj = orc.basis_proj_f32(basis, feat, ids, nbh.ranges)
+            out = proj.reshape(n, C * K) @ wo[0]
+            dproj = (up @ wo[0].T).reshape(n, C, K)
+            dwo = proj.reshape(n, C * K).T @ up
+            dbasis, dfeat = orc.basis_proj_grads_f32(basis, feat, ids, nbh.ranges, dproj)
+            dz = dbasis * (z > 0) / pdf[:, None]
+            dw = diff.T @ dz
+            db = dz.sum(axis=0)
+            return out, dwo, dfeat, dw, db
+
+        return n, len(ids), build_s, step
+
+    def timed(step, budget_s, min_reps):
         step()
-        reps += 1
-        if time.perf_counter() - t0 > 25.0:
-            break
-    dt = (time.perf_counter() - t0) / reps
+        times = []
+        t_start = time.perf_counter()
+        while len(times) < min_reps or time.perf_counter() - t_start < budget_s:
+            t0 = time.perf_counter()
+            step()
+            times.append(time.perf_counter() - t0)
+            if time.perf_counter() - t_start > 2.5 * budget_s:
+                break
+        return times
+
     cores = int(os.environ.get("OMP_NUM_THREADS", "0")) or len(os.sched_getaffinity(0))
+    limit = _set_cpu_threads(orc, cores)
+    n, m, build_s, step = prepare(synthetic.config3(scale=1.0))
+    times = timed(step, 10.0, 2)
+    all_cores = {"points_per_s": n / (sum(times) / len(times)), "cores": cores,
+                 "ms_per_step_mean": 1e3 * sum(times) / len(times),
+                 "ms_per_step_min": 1e3 * min(times), "passes": len(times),
+                 "build_s": round(build_s, 2), "points": n, "pairs": m}
+    del step
+    limit = _set_cpu_threads(orc, 1)
+    n1, m1, build1_s, step1 = prepare(synthetic.config3(scale=1.0, batch=1))
+    times1 = timed(step1, 8.0, 1)
+    one_thread = {"points_per_s": n1 / (sum(times1) / len(times1)), "cores": 1,
+                  "ms_per_step_mean": 1e3 * sum(times1) / len(times1),
+                  "ms_per_step_min": 1e3 * min(times1), "passes": len(times1),
+                  "points": n1, "pairs": m1,
+                  "sample": "the first cloud of the configuration-3 generator"}
+    del step1
+    limit = _set_cpu_threads(orc, cores)
 
     # configuration 1, the case the reference's own CPU path is quoted on: 2 x 1024
     # points, grid + neighbours + densities + one MCConv 8 -> 16 forward
@@ -173,9 +293,9 @@ def cpu_baseline(synthetic, sample_points=60000):
 
     def c1_step():
         g1 = orc.Grid(c1["points"], c1["batch_ids"], c1["batch_size"], r1)
-        n1 = orc.Neighborhood(g1, r1, c1["points"], c1["batch_ids"])
-        return orc.mc_conv_forward(c1["features"], c1["points"], c1["points"], n1,
-                                   n1.pdf_per_pair(c1["bandwidth"]), c1["weights"], c1["biases"],
+        n1_ = orc.Neighborhood(g1, r1, c1["points"], c1["batch_ids"])
+        return orc.mc_conv_forward(c1["features"], c1["points"], c1["points"], n1_,
+                                   n1_.pdf_per_pair(c1["bandwidth"]), c1["weights"], c1["biases"],
                                    c1["final_weights"], r1)
 
     c1_step()
@@ -183,9 +303,13 @@ def cpu_baseline(synthetic, sample_points=60000):
     for _ in range(10):
         c1_step()
     c1_ms = (time.perf_counter() - t0) * 100.0
-    return {"value": n / dt, "unit": "points/s", "cores": cores, "kind": "port",
-            "sample": "one config-3 cloud cut to %d points (%d pairs), %d fwd+bwd passes of "
-                      "the C/OpenMP oracle with numpy GEMMs" % (n, len(ids), reps),
+    return {"value": all_cores["points_per_s"], "unit": "points/s", "cores": cores,
+            "kind": "port",
+            "sample": "the whole configuration-3 workload (%d points, %d pairs), %d fwd+bwd "
+                      "passes of the C/OpenMP oracle with numpy GEMMs on %d threads; "
+                      "`one_thread` is the same on one cloud with a single thread"
+                      % (n, m, len(times), cores),
+            "all_cores": all_cores, "one_thread": one_thread,
             "config1_forward_with_build_ms": c1_ms,
             "config1_points_per_s": len(c1["points"]) / (c1_ms * 1e-3)}
 
@@ -414,12 +538,18 @@ def per_op_times(torch, pc, layers, synthetic, _lib, radius=0.04, reps=5):
     }
     out = {"workload": "4x200k uniform, r=%.2f, self neighbourhood, %d pairs; pooling C=64"
                        % (radius, M)}
+    # ops whose operand count includes per-pair gathers: the roofline uses the compulsory bytes
+    compulsory = {name: compulsory_bytes(name, M, N, N, 64, 1, D)
+                  for name in ("compute_pdf", "compute_pdf_pt_grads", "local_pool")}
+    compulsory["compute_pdf_pt_grads_symmetric"] = compulsory["compute_pdf_pt_grads"]
     for name, vals in sorted(t.items()):
         ms = sum(vals) / reps
-        entry = {"ms": round(ms, 4), "calls_per_pass": len(vals) // reps}
-        if name in by:
-            entry["GBps"] = round(by[name] * (len(vals) // reps) / ms / 1e6, 1)
-            entry["frac_hbm_peak"] = round(entry["GBps"] / HBM_PEAK_GBS, 4)
+        calls = len(vals) // reps
+        entry = {"ms": round(ms, 4), "calls_per_pass": calls}
+        if name in compulsory:
+            entry.update(roofline_entry(compulsory[name], by[name], ms, calls))
+        elif name in by:
+            entry.update(roofline_entry(by[name], None, ms, calls))
         out[name] = entry
     return out
 
@@ -454,9 +584,18 @@ def isolated_basis_proj(torch, pc, synthetic, tfg, _lib, radius=0.04, steps=5):
         for name in ("basis_proj", "basis_proj_grads"):
             ms = sum(t[name]) / len(t[name])
             by = op_bytes(name, M, N, N, C, K, 3)
-            res[name + tag] = {"ms": ms, "GBps": by / ms / 1e6,
-                               "frac_hbm_peak": by / ms / 1e6 / HBM_PEAK_GBS,
-                               "algorithmic_bytes": by}
+            entry = {"ms": ms}
+            entry.update(roofline_entry(compulsory_bytes(name, M, N, N, C, K, 3), by, ms))
+            # the metric's own definition: operand bytes (4*C per pair for the feature rows)
+            # over kernel time; with the pairs in the caller's order those rows do come from
+            # HBM (counter traffic 0.99x this figure), in grid order L2 serves most of them
+            entry["operand_frac_hbm_peak"] = round(by / ms / 1e6 / HBM_PEAK_GBS, 4)
+            traffic, source = measured_traffic(name, "dense_C%d_K%d%s" % (C, K, tag)) \
+                if radius == 0.04 else (None, "no counter run at this radius")
+            entry["traffic"], entry["traffic_source"] = traffic, source
+            if traffic:
+                entry["traffic_frac"] = round(traffic / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
+            res[name + tag] = entry
 
     # the reference's call pattern: pairs address the features by original point id
     # (custom_ops_wrapper.py:185-189), points and centres in the caller's (random) order
@@ -476,8 +615,8 @@ def isolated_basis_proj(torch, pc, synthetic, tfg, _lib, radius=0.04, steps=5):
     t = _lib.collect_timing()
     ms = sum(t["compute_pdf"]) / steps
     by = N * 4 * 3 + 8 * M + 4 * N + M * 4 * 3 + 4 * N
-    res["compute_pdf"] = {"ms": ms, "GBps": by / ms / 1e6, "frac_hbm_peak": by / ms / 1e6 / HBM_PEAK_GBS,
-                          "algorithmic_bytes": by}
+    res["compute_pdf"] = {"ms": ms}
+    res["compute_pdf"].update(roofline_entry(compulsory_bytes("compute_pdf", M, N, N, 1, 1, 3), by, ms))
     res["poisson_disk_sampling"] = {"ms": (sum(t["sampling_count"]) + sum(t["sampling_fill"])) / steps,
                                     "selected": int(sampled._points.shape[0])}
     return res
@@ -486,8 +625,8 @@ def isolated_basis_proj(torch, pc, synthetic, tfg, _lib, radius=0.04, steps=5):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=10)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--scale", type=float, default=1.0, help="shrink the point counts (tests)")
     ap.add_argument("--fuse-final", action="store_true",
                     help="run the product with the final weights inside the projection kernel")
@@ -549,31 +688,33 @@ def main():
         step()
     torch.cuda.synchronize()
     _lib.start_timing()
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    marks[0].record()
+    for i in range(args.steps):
         step()
+        marks[i + 1].record()
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     per_op = {k.replace("_ordered", ""): v for k, v in _lib.collect_timing().items()}
     ms_per_step = dt * 1e3 / args.steps
+    step_ms = sorted(marks[i].elapsed_time(marks[i + 1]) for i in range(args.steps))
 
     ops = {}
     for name, vals in per_op.items():
         ms = sum(vals) / args.steps            # per step, over all calls of the op
         calls = len(vals) / args.steps
-        by = op_bytes(name, M, N, N, C, K, D)
+        by = compulsory_bytes(name, M, N, N, C, K, D)
         ops[name] = {"ms": round(ms, 4), "calls_per_step": calls}
         if by:
-            ops[name].update(GBps=round(by * calls / ms / 1e6, 1),
-                             frac_hbm_peak=round(by * calls / ms / 1e6 / HBM_PEAK_GBS, 4),
-                             algorithmic_bytes=by)
+            ops[name].update(roofline_entry(by, op_bytes(name, M, N, N, C, K, D), ms, calls))
         fig = product_figures(name, N, C, K, CO)
         if fig:                           # dense products: matrix-core and HBM figures
             pby, flops = fig
             ops[name].update(flops=flops, TFLOPs=round(flops * calls / ms / 1e9, 1),
                              frac_fp32_matrix_peak=round(flops * calls / ms / 1e9 /
                                                          FP32_MATRIX_PEAK_TFLOPS, 4),
-                             algorithmic_bytes=pby, GBps_dense=round(pby * calls / ms / 1e6, 1),
+                             compulsory_bytes=pby, GBps_dense=round(pby * calls / ms / 1e6, 1),
                              library="hipBLASLt via torch.matmul" if name.startswith("gemm_")
                              else "hand-written")
         if name in ("permute_rows", "gather_rows"):
@@ -581,25 +722,34 @@ def main():
     kernel_ms = sum(v["ms"] for v in ops.values())
     ops["host_gaps_and_small_kernels"] = {"ms": round(ms_per_step - kernel_ms, 4)}
     dominant = max((n for n in ops if "GBps" in ops[n]), key=lambda n: ops[n]["ms"])
+    launch_ms = ops[dominant]["ms"] / ops[dominant]["calls_per_step"]
+    traffic, traffic_source = (measured_traffic(dominant, "config3_C%d_K%d" % (C, K))
+                               if args.scale == 1.0 else (None, "reduced scale"))
     roof = {"kernel": dominant, "bound": "hbm", "achieved": ops[dominant]["GBps"],
             "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": ops[dominant]["frac_hbm_peak"],
-            "traffic": measured_traffic(dominant, "config3_C%d_K%d" % (C, K))
-            if args.scale == 1.0 else None,
-            "launch_ms": round(ops[dominant]["ms"] / ops[dominant]["calls_per_step"], 4),
+            "traffic": traffic, "traffic_source": traffic_source,
+            "launch_ms": round(launch_ms, 4),
             "launches_per_step": ops[dominant]["calls_per_step"],
-            "algorithmic_bytes": ops[dominant]["algorithmic_bytes"],
-            "note": "algorithmic bytes count every per-pair feature row read (4*C per pair); "
-                    "on the grid-ordered view most of those reads are served by L2, so "
-                    "`traffic` (HBM bytes measured by counters) is below them and `frac` can "
-                    "exceed 1; `traffic_frac` is the measured traffic over launch time and peak"}
-    if roof["traffic"]:
-        roof["traffic_frac"] = round(roof["traffic"] / (roof["launch_ms"] * 1e-3) / 1e9 /
-                                     HBM_PEAK_GBS, 4)
+            "compulsory_bytes": ops[dominant]["compulsory_bytes"],
+            "operand_GBps": ops[dominant].get("operand_GBps"),
+            "matrix_TFLOPs": round(2.0 * M * C * K / launch_ms / 1e9, 1),
+            "matrix_frac_fp32_peak": round(2.0 * M * C * K / launch_ms / 1e9 /
+                                           FP32_MATRIX_PEAK_TFLOPS, 4),
+            "note": "achieved = compulsory HBM bytes of one launch (pair table and densities, "
+                    "coordinates, the feature table once, the [N, C, K] output) over the launch "
+                    "time from HIP events; `operand_GBps` counts every per-pair feature-row read "
+                    "(4*C per pair, served mostly by L2 on the grid-ordered view); `traffic` is "
+                    "what the HBM counters saw per launch, `traffic_frac` that over launch time "
+                    "and peak; `matrix_*` is the segmented C x K contraction against the fp32 "
+                    "matrix peak"}
+    if traffic:
+        roof["traffic_frac"] = round(traffic / (launch_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
 
     result = {
         "metric": "MCConv layer fwd+bwd points/sec", "value": N / (ms_per_step * 1e-3),
         "unit": "points/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
+        "ms_per_step": ms_per_step, "ms_per_step_median": step_ms[len(step_ms) // 2],
+        "ms_per_step_min": step_ms[0], "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "config 3: 8 clustered clouds of 50k-150k points (seed 1003), "
                                "MCConv 64->64, 16-unit kernel MLP, radius 0.15, fp32, fwd+bwd, "
