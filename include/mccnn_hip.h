@@ -525,6 +525,40 @@ int mccnn_kp_conv_project(mccnn_stream_t stream, int num_dims, int64_t num_pts,
                           const float *kernel_points, int kind, float sigma,
                           const int32_t *out_rows, float *out);
 
+/* Projection of the deformable kernel-point convolution (KPConv.py:317-392):
+ * mccnn_kp_conv_project with the kernel points of every centre shifted by its row
+ * of offsets [N_centres, num_kernel_points, D] (at most 16 kernel points).  With
+ * offsets_follow_points != 0 the pair table is the transposed one (rows grouped
+ * by point) and the shifts are those of the gathered side of each pair, which is
+ * how the layer backward obtains its feature gradient.  No counterpart among the
+ * reference's ops (kp_basis in TensorFlow + BasisProj). */
+int mccnn_kp_deform_project(mccnn_stream_t stream, int num_dims, int64_t num_pts,
+                            const float *points_in, int num_features,
+                            const float *features, int64_t num_samples,
+                            const float *points_out, int64_t num_neighbors,
+                            const int32_t *neighbors, const int32_t *ranges,
+                            const float *inv_radii, int num_kernel_points,
+                            const float *kernel_points, int kind, float sigma,
+                            const float *offsets, int offsets_follow_points,
+                            const int32_t *out_rows, float *out);
+
+/* Gradient of that projection with respect to the offsets for an upstream
+ * gradient in_grads [N_out, C, 16]: offset_grads_out [N_out, num_kernel_points, D]
+ * (overwritten).  The [M, 16] basis gradient is formed tile by tile on the matrix
+ * cores and folded in registers; no atomics, fixed summation order.  D in {2,3},
+ * C in {16,32,64,128}.  No counterpart among the reference's ops (TensorFlow
+ * autodiff of KPConv.py:193-224 + BasisProjGrads). */
+int mccnn_kp_deform_offset_grads_supported(int num_dims, int num_features);
+int mccnn_kp_deform_offset_grads(mccnn_stream_t stream, int num_dims, int64_t num_pts,
+                                 const float *points_in, int num_features,
+                                 const float *features, int64_t num_samples,
+                                 const float *points_out, int64_t num_neighbors,
+                                 const int32_t *neighbors, const int32_t *ranges,
+                                 const float *inv_radii, int num_kernel_points,
+                                 const float *kernel_points, int kind, float sigma,
+                                 const float *offsets, const float *in_grads,
+                                 float *offset_grads_out);
+
 /* The whole Monte-Carlo convolution (MCConv.py:137-194) in one kernel:
  *   out[i, f] = sum_{c,k} proj[i, c, k] * final_weights[c*K + k, f]
  * with proj as produced by mccnn_mc_conv_project; the projection is handed from

@@ -37,6 +37,7 @@ __device__ __forceinline__ void load_weight_column(const McParams<D> &p, int j, 
 struct PairStage {
   float4 geo[kWave];      // delta * inv_radii in x, y, z (z = 0 for D = 2), 1 / pdf in w
   unsigned row[kWave];    // byte offset of the neighbour's feature row
+  int aux[kWave];         // row of a per-centre side table (deformable kernel points)
 };
 
 // The activation is a template parameter of the fused kernels: with a run-time
@@ -62,7 +63,8 @@ struct MlpBasis {                  // act(delta . W[:, col] + b[col]) / pdf   (M
       load_weight_column<D>(p, 16 * kt + (lane_id() & 15), w[kt], &b[kt]);
     }
   }
-  __device__ __forceinline__ float operator()(const float4 &g, int kt = 0) const {
+  static constexpr bool kUsesAux = false;
+  __device__ __forceinline__ float operator()(const float4 &g, int kt = 0, int = 0) const {
     const float z = b[kt] + g.x * w[kt][0] + g.y * w[kt][1] + g.z * w[kt][2];
     return act_fwd(kAct, z) * g.w;
   }
@@ -83,7 +85,8 @@ struct KpBasis {                   // kernel-point correlation (KPConv.py:29-57,
       for (int d = 0; d < D; ++d) k[kt][d] = live[kt] ? kernel_points[col * D + d] : 0.0f;
     }
   }
-  __device__ __forceinline__ float operator()(const float4 &g, int kt = 0) const {
+  static constexpr bool kUsesAux = false;
+  __device__ __forceinline__ float operator()(const float4 &g, int kt = 0, int = 0) const {
     const float dx = g.x - k[kt][0], dy = g.y - k[kt][1], dz = g.z - k[kt][2];
     const float dist = sqrtf(dx * dx + dy * dy + dz * dz);
     float wgt;
@@ -95,6 +98,50 @@ struct KpBasis {                   // kernel-point correlation (KPConv.py:29-57,
       wgt = expf(-(q * q));
     }
     return live[kt] ? wgt * g.w : 0.0f;
+  }
+};
+
+// Correlation weight of the kernel-point convolution for a distance.
+template <int kKind>
+__device__ __forceinline__ float kp_weight(float dist, float sigma) {
+  if (kKind == 0) {
+    const float v = 1.0f - dist / sigma;
+    return v > 0.0f ? v : 0.0f;
+  }
+  const float q = dist / (sigma / 3.0f);
+  return expf(-(q * q));
+}
+
+// Deformable kernel points (KPConv.py:317-392): kernel point `col` of the centre of a
+// pair is shifted by offsets[row, col, :], where `row` (the staged aux value) is the
+// centre's row in the [N_centres, num_kp, D] offset table.  Up to 16 kernel points.
+template <int D, int kKind>
+struct KpDeformBasis {
+  float k[3], sigma;
+  const float *off;                // offsets + col * D, or null for a padding column
+  int stride;                      // num_kp * D
+  __device__ __forceinline__ KpDeformBasis(const float *__restrict__ kernel_points, int num_kp,
+                                           float sigma_, const float *__restrict__ offsets)
+      : sigma(sigma_), stride(num_kp * D) {
+    const int col = lane_id() & 15;
+    const bool live = col < num_kp;
+    k[0] = k[1] = k[2] = 0.0f;
+#pragma unroll
+    for (int d = 0; d < D; ++d) k[d] = live ? kernel_points[col * D + d] : 0.0f;
+    off = live ? offsets + col * D : nullptr;
+  }
+  static constexpr bool kUsesAux = true;
+  __device__ __forceinline__ float operator()(const float4 &g, int, int aux) const {
+    if (off == nullptr) return 0.0f;
+    const float *o = off + (int64_t)aux * stride;
+    float diff[3] = {g.x - k[0], g.y - k[1], g.z - k[2]};
+    float sq = 0.0f;
+#pragma unroll
+    for (int d = 0; d < D; ++d) {
+      diff[d] -= o[d];
+      sq += diff[d] * diff[d];
+    }
+    return kp_weight<kKind>(sqrtf(sq), sigma) * g.w;
   }
 };
 

@@ -17,6 +17,7 @@
 namespace mccnn {
 
 constexpr int kProjRun = 8;        // consecutive centres per wavefront
+constexpr int kGradRun = 8;        // the same in the gradient kernels
 
 // One wavefront per (run of kProjRun consecutive centres, chunk of 16*kCPL channels):
 // projection of the centres' pairs with the basis evaluated in registers, rows
@@ -40,7 +41,7 @@ __device__ __forceinline__ void project_run_body(
     int64_t n_out, int C, int chunks, const float *__restrict__ feat,
     const int2 *__restrict__ nbrs, const int *__restrict__ ranges, const McParams<D> &p,
     const Basis &basis, const int *__restrict__ out_rows, float *__restrict__ out,
-    PairStage *stage) {
+    PairStage *stage, bool aux_is_point = false) {
   constexpr int K = kFusedK * KT;          // basis columns, KT tiles of 16
   constexpr int kCW = 16 * kCPL;
   const int lane = lane_id();
@@ -72,13 +73,14 @@ __device__ __forceinline__ void project_run_body(
 
   // in flight for one chunk: the pair, its centre's and its neighbour's coordinates, its density
   struct Pending {
-    int idx;
+    int idx, aux;
     float ctr[D], pt[D], pdf;
   };
   auto fetch_index = [&](int m0) { return m0 + lane < total_end ? nbrs[m0 + lane].x : 0; };
   auto fetch_rest = [&](int m0, int idx) {
     Pending q;
     q.idx = idx;
+    q.aux = 0;
     q.pdf = 1.0f;
 #pragma unroll
     for (int d = 0; d < D; ++d) q.ctr[d] = q.pt[d] = 0.0f;
@@ -93,6 +95,9 @@ __device__ __forceinline__ void project_run_body(
         q.pt[d] = p.pin[(int64_t)idx * D + d];
       }
       if (p.pdf) q.pdf = p.pdf[m];
+      // row of the per-centre side table: the pair's centre, or (transposed table) the
+      // gathered point, which is the centre of the original direction
+      if constexpr (Basis::kUsesAux) q.aux = aux_is_point ? idx : (int)(c0 + ci);
     }
     return q;
   };
@@ -134,6 +139,7 @@ __device__ __forceinline__ void project_run_body(
     wave_lds_sync();                    // the previous chunk has been read
     stage->geo[lane] = g;
     stage->row[lane] = live ? row : row0;
+    if constexpr (Basis::kUsesAux) stage->aux[lane] = pend.aux;
     wave_lds_sync();
     pend = fetch_rest(m0 + kWave, next_idx);
     next_idx = fetch_index(m0 + 2 * kWave);
@@ -149,8 +155,10 @@ __device__ __forceinline__ void project_run_body(
 #pragma unroll
         for (int j = 0; j < kCPL; ++j)
           f[u].v[j] = *reinterpret_cast<const float *>(feat_base + rn + lane_off + j * 64);
+        int aux = 0;
+        if constexpr (Basis::kUsesAux) aux = stage->aux[n];
 #pragma unroll
-        for (int kt = 0; kt < KT; ++kt) w[u][kt] = basis(gn, kt);
+        for (int kt = 0; kt < KT; ++kt) w[u][kt] = basis(gn, kt, aux);
       }
 #pragma unroll
       for (int u = 0; u < kFusedUnroll; ++u) {
@@ -209,6 +217,149 @@ __global__ void __launch_bounds__(256) kp_conv_project16_kernel(
   const KpBasis<D, kKind, KT> basis(kernel_points, num_kp, sigma);
   project_run_body<kCPL, D, KT>(n_out, C, chunks, feat, nbrs, ranges, p, basis, out_rows, out,
                                 &stages[threadIdx.x / kWave]);
+}
+
+// The projection of the deformable kernel-point convolution (KPConv.py:317-392): as
+// above with every centre's kernel points shifted by its row of `offsets`
+// [N_centres, num_kp, D].  Over the transposed pair table (`offsets_follow_points`)
+// the shifts belong to the gathered side of a pair.
+template <int kCPL, int D, int kKind>
+__global__ void __launch_bounds__(256) kp_deform_project16_kernel(
+    int64_t n_out, int C, int chunks, const float *__restrict__ feat,
+    const int2 *__restrict__ nbrs, const int *__restrict__ ranges, McParams<D> p,
+    const float *__restrict__ kernel_points, int num_kp, float sigma,
+    const float *__restrict__ offsets, int offsets_follow_points,
+    const int *__restrict__ out_rows, float *__restrict__ out) {
+  __shared__ PairStage stages[kWavesPerBlock];
+  const KpDeformBasis<D, kKind> basis(kernel_points, num_kp, sigma, offsets);
+  project_run_body<kCPL, D, 1>(n_out, C, chunks, feat, nbrs, ranges, p, basis, out_rows, out,
+                               &stages[threadIdx.x / kWave], offsets_follow_points != 0);
+}
+
+// Gradient of the deformable convolution with respect to the kernel-point offsets,
+//   doff[i, k, :] = sum_{pairs m of centre i} dbasis[m, k] * w'(dist) * (-diff / dist),
+//   dbasis[m, k] = sum_c G[i, c, k] * feat[nbr_m, c],   diff = delta_m - kp_k - off[i, k],
+// without the [M, 16] basis gradient in memory: per centre the upstream tile G [C x 16]
+// sits in registers as the A operand, a chunk of 64 pairs is parked in LDS, every tile
+// of 16 pairs takes C/4 matrix steps for dbasis^T [k x pair], and each lane folds its
+// four (pair, k) entries into running sums that are added over the 16 lanes of a
+// quarter at the end of the centre: fixed order, no atomics.
+template <int C, int D, int kKind>
+__global__ void __launch_bounds__(256) kp_deform_offset_grads16_kernel(
+    int64_t n_out, const float *__restrict__ feat, const int2 *__restrict__ nbrs,
+    const int *__restrict__ ranges, McParams<D> p, const float *__restrict__ kernel_points,
+    int num_kp, float sigma, const float *__restrict__ offsets,
+    const float *__restrict__ in_grad, float *__restrict__ doffsets) {
+  constexpr int K = kFusedK;
+  constexpr int kQuarterC = C / 4;
+  __shared__ PairStage stages[kWavesPerBlock];
+  const int lane = lane_id(), wave = threadIdx.x / kWave;
+  const int quarter = lane >> 4, col = lane & 15;
+  PairStage *stage = &stages[wave];
+  float ir[D];
+#pragma unroll
+  for (int d = 0; d < D; ++d) ir[d] = p.inv_radii[d];
+  float kp[4][3];                     // kernel points 4 quarter + r of this lane's rows
+#pragma unroll
+  for (int r = 0; r < 4; ++r)
+#pragma unroll
+    for (int d = 0; d < 3; ++d)
+      kp[r][d] = (d < D && 4 * quarter + r < num_kp) ? kernel_points[(4 * quarter + r) * D + d]
+                                                     : 0.0f;
+  const char *feat_lane = reinterpret_cast<const char *>(feat + quarter * kQuarterC);
+  const int64_t first = wave_slot() * kGradRun;
+  const int64_t last = first + kGradRun < n_out ? first + kGradRun : n_out;
+  for (int64_t centre = first; centre < last; ++centre) {
+    const int a = centre > 0 ? ranges[centre - 1] : 0, b = ranges[centre];
+    float sum[4][3];
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+#pragma unroll
+      for (int d = 0; d < 3; ++d) sum[r][d] = 0.0f;
+    if (b > a) {
+      const float *gi = in_grad + centre * (int64_t)C * K;
+      float gk[kQuarterC];
+#pragma unroll
+      for (int s = 0; s < kQuarterC; ++s) gk[s] = gi[(quarter * kQuarterC + s) * K + col];
+      float ctr[D];
+#pragma unroll
+      for (int d = 0; d < D; ++d) ctr[d] = p.pout[centre * D + d];
+      // this centre's shifted kernel points 4 quarter + r
+      float kpo[4][3];
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+#pragma unroll
+        for (int d = 0; d < 3; ++d)
+          kpo[r][d] = kp[r][d] + ((d < D && 4 * quarter + r < num_kp)
+                                      ? offsets[(centre * num_kp + 4 * quarter + r) * D + d]
+                                      : 0.0f);
+      for (int m0 = a; m0 < b; m0 += kWave) {
+        const int cnt = b - m0 < kWave ? b - m0 : kWave;
+        float4 g = {0.0f, 0.0f, 0.0f, 0.0f};
+        unsigned row = 0;
+        if (lane < cnt) {
+          const int idx = nbrs[m0 + lane].x;
+          float dl[3] = {0.0f, 0.0f, 0.0f};
+#pragma unroll
+          for (int d = 0; d < D; ++d) dl[d] = (p.pin[(int64_t)idx * D + d] - ctr[d]) * ir[d];
+          g = make_float4(dl[0], dl[1], dl[2], 1.0f);
+          row = (unsigned)idx * (unsigned)(C * 4);
+        }
+        const unsigned row0 = __builtin_amdgcn_readfirstlane(row);
+        stage->geo[lane] = g;
+        stage->row[lane] = lane < cnt ? row : row0;
+        wave_lds_sync();
+        const int tiles = (cnt + 15) >> 4;
+        FVec<kQuarterC> f = load_vec<kQuarterC>(
+            reinterpret_cast<const float *>(feat_lane + stage->row[col]), true);
+        for (int t = 0; t < tiles; ++t) {
+          FVec<kQuarterC> fn = f;
+          if (t + 1 < tiles)
+            fn = load_vec<kQuarterC>(
+                reinterpret_cast<const float *>(feat_lane + stage->row[16 * (t + 1) + col]), true);
+          const float4 geo = stage->geo[16 * t + col];
+          v4f acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+          for (int s = 0; s < kQuarterC; ++s)
+            acc = __builtin_amdgcn_mfma_f32_16x16x4f32(gk[s], f.v[s], acc, 0, 0, 0);
+          // acc[r] = dbasis[pair col][k = 4*quarter + r]; geo.w = 1 for a live pair, else 0
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const float dx = geo.x - kpo[r][0], dy = geo.y - kpo[r][1], dz = geo.z - kpo[r][2];
+            const float dist = sqrtf(dx * dx + dy * dy + dz * dz);
+            float slope;
+            if (kKind == 0) {
+              slope = dist < sigma ? -1.0f / sigma : 0.0f;
+            } else {
+              const float sg = sigma / 3.0f, q = dist / sg;
+              slope = -2.0f * q / sg * expf(-(q * q));
+            }
+            const float coef = dist > 0.0f ? -acc[r] * geo.w * slope / dist : 0.0f;
+            sum[r][0] += coef * dx;
+            sum[r][1] += coef * dy;
+            if (D > 2) sum[r][2] += coef * dz;
+          }
+          f = fn;
+        }
+        wave_lds_sync();                      // the stage is free for the next chunk
+      }
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+#pragma unroll
+        for (int d = 0; d < D; ++d)
+#pragma unroll
+          for (int off = 8; off > 0; off >>= 1) sum[r][d] += __shfl_xor(sum[r][d], off, kWave);
+    }
+    if (col == 0) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        if (4 * quarter + r < num_kp) {
+#pragma unroll
+          for (int d = 0; d < D; ++d)
+            doffsets[(centre * num_kp + 4 * quarter + r) * D + d] = sum[r][d];
+        }
+    }
+  }
 }
 
 // Feature gradient by scatter, for callers that do not use the transposed
@@ -304,7 +455,6 @@ __global__ void __launch_bounds__(256) mc_conv_feature_grads16_kernel(
 // steps for dbasis^T [k x pair] while the feature rows of the next tile are
 // already in flight, and the result is folded in registers into
 //   dW[d][k] += delta_d * dz,  db[k] += dz,  dz = dbasis * act'(z) / pdf.
-constexpr int kGradRun = 8;
 
 static int64_t grad_blocks(int64_t num_samples) {
   const int64_t per_block = (int64_t)kWavesPerBlock * kGradRun;
@@ -777,6 +927,125 @@ extern "C" int mccnn_kp_conv_project(mccnn_stream_t stream, int num_dims, int64_
   }
 #undef MCCNN_KP_FWD_D
 #undef MCCNN_KP_FWD
+  MCCNN_LAUNCH_CHECK();
+  return MCCNN_OK;
+}
+
+static int check_deform_args(const char *op, int num_dims, int num_features, int num_kernel_points,
+                             int kind, float sigma, int64_t num_pts, int64_t num_neighbors,
+                             int64_t num_samples) {
+  MCCNN_REQUIRE(num_kernel_points > 0 && num_kernel_points <= kFusedK,
+                "%s supports 1 to 16 kernel points (got %d)", op, num_kernel_points);
+  MCCNN_REQUIRE(kind == 0 || kind == 1, "%s expects kind 0 (linear) or 1 (gaussian)", op);
+  MCCNN_REQUIRE(sigma > 0.0f, "%s expects a positive sigma", op);
+  MCCNN_REQUIRE(num_neighbors >= 0 && num_neighbors < ((int64_t)1 << 31) && num_samples >= 0 &&
+                    num_samples < ((int64_t)1 << 31),
+                "%s expects sizes in [0, 2^31)", op);
+  MCCNN_REQUIRE(num_pts >= 0 && num_pts * num_features < ((int64_t)1 << 30),
+                "%s expects a feature table of fewer than 2^30 elements", op);
+  return MCCNN_OK;
+}
+
+extern "C" int mccnn_kp_deform_project(mccnn_stream_t stream, int num_dims, int64_t num_pts,
+                                       const float *points_in, int num_features,
+                                       const float *features, int64_t num_samples,
+                                       const float *points_out, int64_t num_neighbors,
+                                       const int32_t *neighbors, const int32_t *ranges,
+                                       const float *inv_radii, int num_kernel_points,
+                                       const float *kernel_points, int kind, float sigma,
+                                       const float *offsets, int offsets_follow_points,
+                                       const int32_t *out_rows, float *out) {
+  MCCNN_REQUIRE(project_supported(num_dims, num_features, kFusedK),
+                "kp_deform_project supports D in {2,3} and C in {16, 32, ..., 512} (got D=%d, "
+                "C=%d)", num_dims, num_features);
+  int rc = check_deform_args("kp_deform_project", num_dims, num_features, num_kernel_points,
+                             kind, sigma, num_pts, num_neighbors, num_samples);
+  if (rc != MCCNN_OK) return rc;
+  if (num_samples == 0) return MCCNN_OK;
+  MCCNN_REQUIRE(ranges && out && points_out && inv_radii && kernel_points &&
+                    (num_neighbors == 0 || (points_in && features && neighbors && offsets)),
+                "kp_deform_project received a null tensor");
+  hipStream_t s = as_stream(stream);
+  int cpl = 1;
+  for (int c = 8; c >= 1; c >>= 1)
+    if (num_features % (16 * c) == 0) { cpl = c; break; }
+  const int chunks = num_features / (16 * cpl);
+  const dim3 grid(wave_grid((num_samples + kProjRun - 1) / kProjRun * chunks)), block(256);
+  const int2 *nb = (const int2 *)neighbors;
+#define MCCNN_KPD(CPL_, D_, KIND_)                                                             \
+  {                                                                                            \
+    McParams<D_> prm{points_in, points_out, inv_radii, nullptr, nullptr, nullptr, 1, 0};       \
+    hipLaunchKernelGGL((kp_deform_project16_kernel<CPL_, D_, KIND_>), grid, block, 0, s,       \
+                       num_samples, num_features, chunks, features, nb, ranges, prm,           \
+                       kernel_points, num_kernel_points, sigma, offsets, offsets_follow_points, \
+                       out_rows, out);                                                         \
+  }
+#define MCCNN_KPD_D(CPL_)                                                  \
+  if (num_dims == 3) {                                                     \
+    if (kind == 0) MCCNN_KPD(CPL_, 3, 0) else MCCNN_KPD(CPL_, 3, 1)        \
+  } else {                                                                 \
+    if (kind == 0) MCCNN_KPD(CPL_, 2, 0) else MCCNN_KPD(CPL_, 2, 1)        \
+  }
+  switch (cpl) {
+    case 8: MCCNN_KPD_D(8); break;
+    case 4: MCCNN_KPD_D(4); break;
+    case 2: MCCNN_KPD_D(2); break;
+    default: MCCNN_KPD_D(1); break;
+  }
+#undef MCCNN_KPD_D
+#undef MCCNN_KPD
+  MCCNN_LAUNCH_CHECK();
+  return MCCNN_OK;
+}
+
+extern "C" int mccnn_kp_deform_offset_grads_supported(int num_dims, int num_features) {
+  return fused_supported(num_dims, num_features, kFusedK, true) ? 1 : 0;
+}
+
+extern "C" int mccnn_kp_deform_offset_grads(mccnn_stream_t stream, int num_dims, int64_t num_pts,
+                                            const float *points_in, int num_features,
+                                            const float *features, int64_t num_samples,
+                                            const float *points_out, int64_t num_neighbors,
+                                            const int32_t *neighbors, const int32_t *ranges,
+                                            const float *inv_radii, int num_kernel_points,
+                                            const float *kernel_points, int kind, float sigma,
+                                            const float *offsets, const float *in_grads,
+                                            float *offset_grads_out) {
+  MCCNN_REQUIRE(fused_supported(num_dims, num_features, kFusedK, true),
+                "kp_deform_offset_grads supports D in {2,3} and C in {16,32,64,128} (got D=%d, "
+                "C=%d)", num_dims, num_features);
+  int rc = check_deform_args("kp_deform_offset_grads", num_dims, num_features,
+                             num_kernel_points, kind, sigma, num_pts, num_neighbors, num_samples);
+  if (rc != MCCNN_OK) return rc;
+  if (num_samples == 0) return MCCNN_OK;
+  MCCNN_REQUIRE(ranges && offset_grads_out && points_out && inv_radii && kernel_points &&
+                    offsets && in_grads && (num_neighbors == 0 || (points_in && features &&
+                                                                   neighbors)),
+                "kp_deform_offset_grads received a null tensor");
+  hipStream_t s = as_stream(stream);
+  const dim3 grid((unsigned)grad_blocks(num_samples)), block(256);
+  const int2 *nb = (const int2 *)neighbors;
+#define MCCNN_KPG(C_, D_, KIND_)                                                               \
+  {                                                                                            \
+    McParams<D_> prm{points_in, points_out, inv_radii, nullptr, nullptr, nullptr, 1, 0};       \
+    hipLaunchKernelGGL((kp_deform_offset_grads16_kernel<C_, D_, KIND_>), grid, block, 0, s,    \
+                       num_samples, features, nb, ranges, prm, kernel_points,                  \
+                       num_kernel_points, sigma, offsets, in_grads, offset_grads_out);         \
+  }
+#define MCCNN_KPG_D(C_)                                                  \
+  if (num_dims == 3) {                                                   \
+    if (kind == 0) MCCNN_KPG(C_, 3, 0) else MCCNN_KPG(C_, 3, 1)          \
+  } else {                                                               \
+    if (kind == 0) MCCNN_KPG(C_, 2, 0) else MCCNN_KPG(C_, 2, 1)          \
+  }
+  switch (num_features) {
+    case 16: MCCNN_KPG_D(16); break;
+    case 32: MCCNN_KPG_D(32); break;
+    case 64: MCCNN_KPG_D(64); break;
+    default: MCCNN_KPG_D(128); break;
+  }
+#undef MCCNN_KPG_D
+#undef MCCNN_KPG
   MCCNN_LAUNCH_CHECK();
   return MCCNN_OK;
 }

@@ -829,15 +829,18 @@ class _KPConvRigidLayer(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, dense_weights, features, neighborhood, inv_radii, kernel_points, k, kind,
-                sigma):
+                sigma, rows_in_view_order):
         view = neighborhood.sorted_view()
         feats = _gather_rows(features, view.point_rows)
-        # rows of the projection go straight to the centres' original positions
+        # rows of the projection go straight to the centres' original positions (or stay
+        # in the view's order, for a consumer that works on the view itself)
         proj = _kp_project(feats, view.points_in, view.points_out, view.table, view.ranges,
-                           inv_radii, kernel_points, k, kind, sigma, view.centre_rows)
+                           inv_radii, kernel_points, k, kind, sigma,
+                           None if rows_in_view_order else view.centre_rows)
         out = _final_product(proj.reshape(proj.shape[0], -1), dense_weights)
         ctx.save_for_backward(dense_weights, feats, features, inv_radii, kernel_points)
         ctx.neighborhood, ctx.k, ctx.kind, ctx.sigma = neighborhood, k, kind, sigma
+        ctx.rows_in_view_order = rows_in_view_order
         return out
 
     @staticmethod
@@ -845,7 +848,7 @@ class _KPConvRigidLayer(torch.autograd.Function):
         dense, feats, features, inv_radii, kernel_points = ctx.saved_tensors
         view = ctx.neighborhood.sorted_view()
         k, c, f = ctx.k, feats.shape[1], dense.shape[1]
-        if view.centre_order is not None:
+        if view.centre_order is not None and not ctx.rows_in_view_order:
             dout = _gather_rows(dout, view.centre_rows)
         else:
             dout = dout.contiguous()
@@ -860,7 +863,80 @@ class _KPConvRigidLayer(torch.autograd.Function):
         if ctx.needs_input_grad[0]:
             ddense = _weight_grad_product(features, q).reshape(c, f, k).permute(0, 2, 1)
             ddense = ddense.reshape(c * k, f)
-        return ddense, dfeat, None, None, None, None, None, None
+        return ddense, dfeat, None, None, None, None, None, None, None
+
+
+def _kp_deform_project(features, points_in, points_out, neighbors, ranges, inv_radii,
+                       kernel_points, kind, sigma, offsets, offsets_follow_points, out_rows=None):
+    """Projection with per-centre kernel-point offsets -> [N_out, C, 16]."""
+    kp, dims = kernel_points.shape
+    c = features.shape[1]
+    out = torch.empty((ranges.shape[0], c, 16), dtype=_F32, device=features.device)
+    _lib.call("kp_deform_project", stream(), cint(dims), i64(features.shape[0]),
+              ptr(points_in, _F32), cint(c), ptr(features, _F32), i64(ranges.shape[0]),
+              ptr(points_out, _F32), i64(neighbors.shape[0]), ptr(neighbors, _I32),
+              ptr(ranges, _I32), ptr(inv_radii, _F32), cint(kp), ptr(kernel_points, _F32),
+              cint(kind), cfloat(sigma), ptr(offsets, _F32), cint(1 if offsets_follow_points else 0),
+              ptr(out_rows), ptr(out))
+    return out
+
+
+class _KPConvDeformLayer(torch.autograd.Function):
+    """Deformable kernel-point convolution (KPConv.py:317-392) on the neighbourhood's
+    grid-ordered view, given the per-centre offsets in the view's centre order.  The
+    kernel-point weights are evaluated in registers in the forward projection, in the
+    transposed projection that yields the feature and weight gradients (there the
+    offsets belong to the gathered side of a pair), and in the offset-gradient kernel,
+    which forms the basis gradient tile by tile from dproj = dout W^T; the [M, K] basis
+    and its gradient never reach memory and nothing is scattered."""
+
+    @staticmethod
+    def forward(ctx, dense_weights, offsets, features, neighborhood, inv_radii, kernel_points,
+                kind, sigma):
+        view = neighborhood.sorted_view()
+        feats = _gather_rows(features, view.point_rows)
+        offsets = offsets.contiguous()
+        proj = _kp_deform_project(feats, view.points_in, view.points_out, view.table,
+                                  view.ranges, inv_radii, kernel_points, kind, sigma, offsets,
+                                  False, view.centre_rows)
+        out = _final_product(proj.reshape(proj.shape[0], -1), dense_weights)
+        ctx.save_for_backward(dense_weights, offsets, feats, features, inv_radii, kernel_points)
+        ctx.neighborhood, ctx.kind, ctx.sigma = neighborhood, kind, sigma
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        dense, offsets, feats, features, inv_radii, kernel_points = ctx.saved_tensors
+        view = ctx.neighborhood.sorted_view()
+        kp, dims = kernel_points.shape
+        k, c, f = 16, feats.shape[1], dense.shape[1]
+        n_out = view.ranges.shape[0]
+        if view.centre_order is not None:
+            dout = _gather_rows(dout, view.centre_rows)
+        else:
+            dout = dout.contiguous()
+        dfeat = ddense = doff = None
+        if ctx.needs_input_grad[0] or ctx.needs_input_grad[2]:
+            q = _kp_deform_project(dout, view.points_out, view.points_in, view.table_t,
+                                   view.ranges_t, -inv_radii, kernel_points, ctx.kind, ctx.sigma,
+                                   offsets, True, view.point_rows)
+            q = q.reshape(feats.shape[0], f * k)
+            if ctx.needs_input_grad[2]:
+                w2 = dense.reshape(c, k, f).permute(2, 1, 0).reshape(f * k, c)
+                dfeat = _final_product(q, w2)
+            if ctx.needs_input_grad[0]:
+                ddense = _weight_grad_product(features, q).reshape(c, f, k).permute(0, 2, 1)
+                ddense = ddense.reshape(c * k, f)
+        if ctx.needs_input_grad[1]:
+            dproj = _projection_grad_product(dout, dense)            # [N_out, C*16]
+            doff = torch.empty((n_out, kp, dims), dtype=_F32, device=dout.device)
+            _lib.call("kp_deform_offset_grads", stream(), cint(dims), i64(feats.shape[0]),
+                      ptr(view.points_in, _F32), cint(c), ptr(feats, _F32), i64(n_out),
+                      ptr(view.points_out, _F32), i64(view.table.shape[0]),
+                      ptr(view.table, _I32), ptr(view.ranges, _I32), ptr(inv_radii, _F32),
+                      cint(kp), ptr(kernel_points, _F32), cint(ctx.kind), cfloat(ctx.sigma),
+                      ptr(offsets, _F32), ptr(dproj, _F32), ptr(doff))
+        return ddense, doff, dfeat, None, None, None, None, None
 
 
 class KPConv(torch.nn.Module):
@@ -909,6 +985,7 @@ class KPConv(torch.nn.Module):
             self.offset_weights = torch.nn.Parameter(offset_weights.to(_F32).contiguous())
         self.last_neighborhood = None
         self._last = None
+        self.last_offsets = None      # [N_out, K, D] offsets of the last deformable call
 
     def _padded(self, w):
         """[C*KP, F] -> [C*K, F] with zero rows for the padded basis columns."""
@@ -942,7 +1019,10 @@ class KPConv(torch.nn.Module):
         if not self.deformable and self.transposed_grads:
             return _KPConvRigidLayer.apply(self._padded(self.weights), features, neighborhood,
                                            torch.reciprocal(radii), self._kernel_points, k,
-                                           self._kind, sigma)
+                                           self._kind, sigma, False)
+        if self.deformable and self.transposed_grads and k == 16 and d in (2, 3) and \
+                _lib.lib().mccnn_kp_deform_offset_grads_supported(cint(d), cint(c)):
+            return self._convolve_deformed_on_view(features, neighborhood, radii, sigma)
         ids, ranges = neighborhood._original_neigh_ids, neighborhood._samples_neigh_ranges
         transposed = None
         if features.requires_grad and tfg_custom_ops.gathered_grads_supported(c, k):
@@ -963,14 +1043,43 @@ class KPConv(torch.nn.Module):
                 w_off = torch.nn.functional.pad(w_off, (0, -cols % 16))
                 offsets = _KPConvRigidLayer.apply(w_off, features, neighborhood,
                                                   torch.reciprocal(radii), self._kernel_points, k,
-                                                  self._kind, sigma)[:, :cols]
+                                                  self._kind, sigma, False)[:, :cols]
             else:
                 rigid = _KPBasis.apply(None, *geometry, k, self._kind, sigma)
                 offsets = project(rigid).reshape(-1, c * k) @ w_off
             offsets = offsets.reshape(-1, kp, d).contiguous()
         self._last = (offsets, geometry, sigma)
+        self.last_offsets = offsets
         basis = _KPBasis.apply(offsets, *geometry, k, self._kind, sigma)
         return project(basis).reshape(-1, c * k) @ self._padded(self.weights)
+
+    def _convolve_deformed_on_view(self, features, neighborhood, radii, sigma):
+        """KPConv.py:317-392 on the grid-ordered view: a rigid convolution predicts the
+        offsets (rows in the caller's centre order, `last_offsets`), which are brought
+        into the view's centre order for the deformed convolution and for the
+        regularisation loss."""
+        kp, k, d = self._num_kernel_points, self._num_basis, self._num_dims
+        view = neighborhood.sorted_view()
+        inv_radii = torch.reciprocal(radii)
+        cols = kp * d
+        w_off = torch.nn.functional.pad(self._padded(self.offset_weights), (0, -cols % 16))
+        offsets = _KPConvRigidLayer.apply(w_off, features, neighborhood, inv_radii,
+                                          self._kernel_points, k, self._kind, sigma,
+                                          False)[:, :cols]
+        offsets = offsets.reshape(-1, kp, d)
+        self.last_offsets = offsets
+        on_view = offsets if view.centre_order is None else \
+            offsets.index_select(0, view.centre_order)
+        on_view = on_view.contiguous()
+        geometry = (view.points_in, view.points_out, view.table, view.ranges, inv_radii,
+                    self._kernel_points)
+        self._last = (on_view, geometry, sigma)
+        # output columns padded to a multiple of 16 (the transposed projection runs on them)
+        f = self._num_features_out
+        dense = torch.nn.functional.pad(self._padded(self.weights), (0, -f % 16))
+        out = _KPConvDeformLayer.apply(dense, on_view, features, neighborhood, inv_radii,
+                                       self._kernel_points, self._kind, sigma)
+        return out[:, :f] if f % 16 else out
 
     def _convolve_moving(self, features, point_cloud_in, point_cloud_out, radii, neighborhood,
                          sigma):
@@ -1003,6 +1112,7 @@ class KPConv(torch.nn.Module):
             offsets = (project(correlation(None)) @ self._padded(self.offset_weights))
             offsets = offsets.reshape(-1, kp, d)
         self._last = None
+        self.last_offsets = offsets
         if self.deformable:
             geometry = (point_cloud_in._points.detach(), point_cloud_out._points.detach(), ids,
                         ranges, torch.reciprocal(radii), self._kernel_points)

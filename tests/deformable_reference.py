@@ -1,0 +1,131 @@
+"""Float64 reference of the deformable kernel-point convolution, shared by the GPU tests
+(not a test module itself)."""
+import numpy as np
+import torch
+
+REL = 1e-5
+
+
+def dev(a):
+    return torch.as_tensor(np.ascontiguousarray(a)).cuda().contiguous()
+
+
+def assert_rel_t(got, expect, mag, tol=REL):
+    """|got - expect| <= tol * mag elementwise on device tensors (float64 expect / mag)."""
+    err = (got.double() - expect).abs()
+    bad = err > tol * mag + 1e-30
+    assert not bool(bad.any()), "max err/mag = %g at %d of %d entries" % (
+        float((err / mag.clamp(min=1e-300)).max()), int(bad.sum()), err.numel())
+
+
+def check_deformable_kpconv(pts, bids, ctr, cb, batch, ids_np, radius, feat, kp, wts, woff,
+                            influence, kind, tol=2e-5):
+    """Deformable kernel-point convolution (KPConv.py:317-429) and its regularisation
+    loss against float64 autograd (run on the device) on the given pair table.
+
+    The output and the loss are continuous in the inputs; their gradients are not: the
+    linear correlation relu(1 - d / sigma) has a kink at d = sigma, and the fitting loss
+    follows the pair that attains a minimum.  Where float32 and float64 may decide
+    differently (|1 - d / sigma| < 1e-5; two smallest squared distances within 1e-5 of
+    each other; two deformed kernel points within 0.004 of each other, whose linear
+    repulsion has an ill-conditioned direction) the offset gradient of that (centre, kernel point) is left out of the
+    comparison: the reference is cut at the offsets, its offset gradient is compared with
+    the layer's entry by entry outside that set (which must stay below 2 % of the
+    entries), takes the layer's values inside it, and is then carried on to the
+    features and the offset weights, so that every parameter gradient is compared in
+    full."""
+    from tensorflow_graphics_point_clouds_amd import layers, pc
+    n, c = len(ctr), feat.shape[1]
+    kpn = kp.shape[0]
+    f_out = wts.shape[1]
+    sigma = influence / radius
+    f64 = dict(dtype=torch.float64, device="cuda")
+    ids = torch.as_tensor(ids_np).long().cuda()
+    radii = np.full(3, np.float32(radius), np.float32)
+    delta = torch.tensor(((pts[ids_np[:, 0]] - ctr[ids_np[:, 1]]) / radii).astype(np.float64)).cuda()
+    tkp = torch.tensor(kp.astype(np.float64) * 0.75).cuda()
+    centre = ids[:, 1]
+
+    def weight(dist):
+        if kind == "linear":
+            return torch.relu(1 - dist / sigma)
+        return torch.exp(-(dist / (sigma / 3)) ** 2)
+
+    tf = torch.tensor(feat.astype(np.float64), device="cuda", requires_grad=True)
+    tw = torch.tensor(wts.astype(np.float64), device="cuda", requires_grad=True)
+    two = torch.tensor(woff.astype(np.float64), device="cuda", requires_grad=True)
+
+    def project(basis, f):
+        return torch.zeros(n, c, kpn, **f64).index_add(
+            0, centre, f[ids[:, 0]][:, :, None] * basis[:, None, :])
+
+    rigid = weight((delta[:, None, :] - tkp[None]).norm(dim=2))
+    off = (project(rigid, tf).reshape(n, -1) @ two).reshape(n, kpn, 3)
+    cut = off.detach().clone().requires_grad_(True)          # the reference, cut at the offsets
+    dist = (delta[:, None, :] - (tkp[None] + cut[centre])).norm(dim=2)
+    deformed = weight(dist)
+    ref_out = project(deformed, tf).reshape(n, -1) @ tw
+    with torch.no_grad():
+        out_mag = project(deformed, tf.abs()).reshape(n, -1) @ tw.abs()
+    sq = (dist / sigma) ** 2
+    expand = centre[:, None].expand(-1, kpn)
+    fit = torch.full((n, kpn), float("inf"), **f64).scatter_reduce(0, expand, sq, "amin")
+    kpd = tkp[None] + cut
+    kd = (kpd[:, None] - kpd[:, :, None] + 1e-300).norm(dim=3)
+    rep = weight(kd) * (1 - torch.eye(kpn, **f64))[None]
+    ref_loss = fit.sum() + rep.sum()
+
+    with torch.no_grad():       # (centre, kernel point) entries whose gradient may flip
+        unsure_out = torch.zeros((n, kpn), dtype=torch.bool, device="cuda")
+        unsure_loss = torch.zeros((n, kpn), dtype=torch.bool, device="cuda")
+        if kind == "linear":
+            near = ((1 - dist / sigma).abs() < 1e-5).to(torch.float64)
+            unsure_out = torch.zeros((n, kpn), **f64).index_add(0, centre, near) > 0
+            # (two kernel points closer than 0.004 -- the 15-point layout of the reference
+            # holds two coincident pairs, which only the offsets separate -- make the
+            # direction of their repulsion ill-conditioned in float32)
+            kink = (((1 - kd / sigma).abs() < 1e-5) | (kd < 4e-3)) & \
+                ~torch.eye(kpn, dtype=torch.bool, device="cuda")
+            unsure_loss = kink.any(dim=1) | kink.any(dim=2)
+        runner_up = torch.full((n, kpn), float("inf"), **f64).scatter_reduce(
+            0, expand, torch.where(sq > fit[centre], sq, torch.full_like(sq, float("inf"))), "amin")
+        unsure_loss |= (runner_up - fit) < 1e-5 * fit.clamp(min=1e-30)
+
+    cloud = pc.PointCloud(dev(pts), dev(bids), batch)
+    centres = cloud if ctr is pts else pc.PointCloud(dev(ctr), dev(cb), batch)
+    conv = layers.KPConv(c, f_out, custom_kernel_points=kp, kp_interpolation=kind,
+                         weights=dev(wts), deformable=True, offset_weights=dev(woff))
+    tfeat = dev(feat).requires_grad_(True)
+    out = conv(tfeat, cloud, centres, radius, kernel_influence_dist=influence)
+    loss = conv.regularization_loss()
+    offsets = conv.last_offsets
+    assert float((offsets.double() - off.detach()).abs().max()) <= tol * float(off.detach().abs().max())
+    assert_rel_t(out.detach(), ref_out.detach(), out_mag, tol=tol)
+    np.testing.assert_allclose(float(loss.detach()), float(ref_loss.detach()), rtol=REL)
+
+    def normwise(got, expect, what):
+        diff = (got.double() - expect).abs()
+        err, scale = float(diff.max()), float(expect.abs().max())
+        where = int(diff.argmax())
+        assert err <= tol * scale, "%s: %g at flat index %d (got %r, expected %r)" % (
+            what, err / scale, where, float(got.reshape(-1)[where]),
+            float(expect.reshape(-1)[where]))
+
+    up = torch.tensor(np.random.default_rng(7).standard_normal((n, f_out)).astype(np.float32)).cuda()
+    for name, scalar, ref_scalar, unsure in (("output", (out * up).sum(), (ref_out * up.double()).sum(), unsure_out),
+                                             ("loss", loss, ref_loss, unsure_loss)):
+        assert float(unsure.double().mean()) < 2e-2, name
+        got = torch.autograd.grad(scalar, [offsets, tfeat, conv.weights, conv.offset_weights],
+                                  retain_graph=True, allow_unused=True)
+        d_cut, d_tf, d_tw = torch.autograd.grad(ref_scalar, [cut, tf, tw], retain_graph=True,
+                                                allow_unused=True)
+        keep = (~unsure)[:, :, None].to(torch.float64)
+        normwise(got[0].double() * keep, d_cut * keep, name + " / offsets")
+        d_cut = torch.where(unsure[:, :, None], got[0].double(), d_cut)
+        c_tf, c_two = torch.autograd.grad(off, [tf, two], grad_outputs=d_cut, retain_graph=True)
+        normwise(got[1], c_tf if d_tf is None else d_tf + c_tf, name + " / features")
+        normwise(got[3], c_two, name + " / offset weights")
+        if d_tw is not None:
+            normwise(got[2], d_tw, name + " / weights")
+        else:
+            assert got[2] is None or float(got[2].abs().max()) == 0.0

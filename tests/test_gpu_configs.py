@@ -220,110 +220,6 @@ def test_config5_kpconv_matches_oracle_at_reduced_size(oracle, kind, influence_f
     assert_rel(conv.weights.grad.cpu().numpy(), proj.T @ up64, pmag.T @ np.abs(up64))
 
 
-def check_deformable_kpconv(pts, bids, batch, ids_np, radius, feat, kp, wts, woff, influence,
-                            kind, tol=2e-5):
-    """Deformable kernel-point convolution (KPConv.py:317-429) and its regularisation
-    loss against float64 autograd (run on the device) on the given pair table.
-
-    The output and the loss are continuous in the inputs; their gradients are not: the
-    linear correlation relu(1 - d / sigma) has a kink at d = sigma, and the fitting loss
-    follows the pair that attains a minimum.  Where float32 and float64 may decide
-    differently (|1 - d / sigma| < 1e-5; two smallest squared distances within 1e-5 of
-    each other) the offset gradient of that (centre, kernel point) is left out of the
-    comparison: the reference is cut at the offsets, its offset gradient is compared with
-    the layer's entry by entry outside that set (which must stay below 0.2 % of the
-    entries), takes the layer's values inside it, and is then carried on to the
-    features and the offset weights, so that every parameter gradient is compared in
-    full."""
-    from tensorflow_graphics_point_clouds_amd import layers, pc
-    n, c = feat.shape
-    kpn = kp.shape[0]
-    f_out = wts.shape[1]
-    sigma = influence / radius
-    f64 = dict(dtype=torch.float64, device="cuda")
-    ids = torch.as_tensor(ids_np).long().cuda()
-    radii = np.full(3, np.float32(radius), np.float32)
-    delta = torch.tensor(((pts[ids_np[:, 0]] - pts[ids_np[:, 1]]) / radii).astype(np.float64)).cuda()
-    tkp = torch.tensor(kp.astype(np.float64) * 0.75).cuda()
-    centre = ids[:, 1]
-
-    def weight(dist):
-        if kind == "linear":
-            return torch.relu(1 - dist / sigma)
-        return torch.exp(-(dist / (sigma / 3)) ** 2)
-
-    tf = torch.tensor(feat.astype(np.float64), device="cuda", requires_grad=True)
-    tw = torch.tensor(wts.astype(np.float64), device="cuda", requires_grad=True)
-    two = torch.tensor(woff.astype(np.float64), device="cuda", requires_grad=True)
-
-    def project(basis, f):
-        return torch.zeros(n, c, kpn, **f64).index_add(
-            0, centre, f[ids[:, 0]][:, :, None] * basis[:, None, :])
-
-    rigid = weight((delta[:, None, :] - tkp[None]).norm(dim=2))
-    off = (project(rigid, tf).reshape(n, -1) @ two).reshape(n, kpn, 3)
-    cut = off.detach().clone().requires_grad_(True)          # the reference, cut at the offsets
-    dist = (delta[:, None, :] - (tkp[None] + cut[centre])).norm(dim=2)
-    deformed = weight(dist)
-    ref_out = project(deformed, tf).reshape(n, -1) @ tw
-    with torch.no_grad():
-        out_mag = project(deformed, tf.abs()).reshape(n, -1) @ tw.abs()
-    sq = (dist / sigma) ** 2
-    expand = centre[:, None].expand(-1, kpn)
-    fit = torch.full((n, kpn), float("inf"), **f64).scatter_reduce(0, expand, sq, "amin")
-    kpd = tkp[None] + cut
-    kd = (kpd[:, None] - kpd[:, :, None] + 1e-300).norm(dim=3)
-    rep = weight(kd) * (1 - torch.eye(kpn, **f64))[None]
-    ref_loss = fit.sum() + rep.sum()
-
-    with torch.no_grad():       # (centre, kernel point) entries whose gradient may flip
-        unsure_out = torch.zeros((n, kpn), dtype=torch.bool, device="cuda")
-        unsure_loss = torch.zeros((n, kpn), dtype=torch.bool, device="cuda")
-        if kind == "linear":
-            near = ((1 - dist / sigma).abs() < 1e-5).to(torch.float64)
-            unsure_out = torch.zeros((n, kpn), **f64).index_add(0, centre, near) > 0
-            kink = ((1 - kd / sigma).abs() < 1e-5) & ~torch.eye(kpn, dtype=torch.bool, device="cuda")
-            unsure_loss = kink.any(dim=1) | kink.any(dim=2)
-        runner_up = torch.full((n, kpn), float("inf"), **f64).scatter_reduce(
-            0, expand, torch.where(sq > fit[centre], sq, torch.full_like(sq, float("inf"))), "amin")
-        unsure_loss |= (runner_up - fit) < 1e-5 * fit.clamp(min=1e-30)
-
-    cloud = pc.PointCloud(dev(pts), dev(bids), batch)
-    conv = layers.KPConv(c, f_out, custom_kernel_points=kp, kp_interpolation=kind,
-                         weights=dev(wts), deformable=True, offset_weights=dev(woff))
-    tfeat = dev(feat).requires_grad_(True)
-    out = conv(tfeat, cloud, cloud, radius, kernel_influence_dist=influence)
-    loss = conv.regularization_loss()
-    offsets = conv._last[0]
-    assert float((offsets.double() - off.detach()).abs().max()) <= tol * float(off.detach().abs().max())
-    assert_rel_t(out.detach(), ref_out.detach(), out_mag, tol=tol)
-    np.testing.assert_allclose(float(loss.detach()), float(ref_loss.detach()), rtol=REL)
-
-    def normwise(got, expect, what):
-        err = float((got.double() - expect).abs().max())
-        scale = float(expect.abs().max())
-        assert err <= tol * scale, "%s: %g" % (what, err / scale)
-
-    up = torch.tensor(np.random.default_rng(7).standard_normal((n, f_out)).astype(np.float32)).cuda()
-    for name, scalar, ref_scalar, unsure in (("output", (out * up).sum(), (ref_out * up.double()).sum(), unsure_out),
-                                             ("loss", loss, ref_loss, unsure_loss)):
-        assert float(unsure.double().mean()) < 2e-3, name
-        got = torch.autograd.grad(scalar, [offsets, tfeat, conv.weights, conv.offset_weights],
-                                  retain_graph=True, allow_unused=True)
-        d_cut, d_tf, d_tw = torch.autograd.grad(ref_scalar, [cut, tf, tw], retain_graph=True,
-                                                allow_unused=True)
-        keep = (~unsure)[:, :, None].to(torch.float64)
-        normwise(got[0].double() * keep, d_cut * keep, name + " / offsets")
-        d_cut = torch.where(unsure[:, :, None], got[0].double(), d_cut)
-        c_tf, c_two = torch.autograd.grad(off, [tf, two], grad_outputs=d_cut, retain_graph=True)
-        normwise(got[1], c_tf if d_tf is None else d_tf + c_tf, name + " / features")
-        normwise(got[3], c_two, name + " / offset weights")
-        if d_tw is not None:
-            normwise(got[2], d_tw, name + " / weights")
-        else:
-            assert got[2] is None or float(got[2].abs().max()) == 0.0
-
-
 @pytest.mark.parametrize("kind", ["linear", "gaussian"])
 def test_config5_deformable_kpconv_matches_float64_autograd(oracle, kind):
     """Deformable variant of configuration 5 at the reduced size (radius 0.4, 13
@@ -338,8 +234,9 @@ def test_config5_deformable_kpconv_matches_float64_autograd(oracle, kind):
     kp = synthetic.spherical_kernel_points(15, rotate=False) * 0.8
     wts = (rng.standard_normal((kpn * c, c)) * np.sqrt(2.0 / (kpn * c + c))).astype(np.float32)
     woff = (rng.standard_normal((kpn * c, kpn * 3)) * 5e-4).astype(np.float32)
-    check_deformable_kpconv(pts, bids, batch, nbh.original_neigh_ids, radius, feat, kp, wts, woff,
-                            0.5 * radius, kind)
+    from tests.deformable_reference import check_deformable_kpconv
+    check_deformable_kpconv(pts, bids, pts, bids, batch, nbh.original_neigh_ids, radius, feat, kp,
+                            wts, woff, 0.5 * radius, kind)
 
 
 def test_config5_kpconv_at_full_scene_size():

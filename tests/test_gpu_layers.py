@@ -240,73 +240,27 @@ def test_kpconv_forward_backward(oracle, kind, influence, c_in, c_out, transpose
              tol=2e-5)
 
 
+@pytest.mark.parametrize("c_in,c_out", [(16, 8), (8, 16), (32, 32)])
 @pytest.mark.parametrize("kind", ["linear", "gaussian"])
-def test_deformable_kpconv_and_regularization(oracle, kind):
+def test_deformable_kpconv_and_regularization(oracle, kind, c_in, c_out):
     """Deformable kernel points (offsets predicted by a rigid convolution) and the
     regularisation loss, forward and backward, against float64 autograd of the
-    expressions of KPConv.py:165-232, 317-429 on the oracle's neighbour pairs."""
-    from tensorflow_graphics_point_clouds_amd import layers, pc, synthetic
+    expressions of KPConv.py:165-232, 317-429 on the oracle's neighbour pairs; foreign
+    centres; 16 and 32 input channels take the kernels with the weights in registers, 8
+    the materialising ops.  Normwise 2e-5 for the gradients (non-smooth points of the
+    correlation and of the fitting minimum are handled as the helper describes)."""
+    from tensorflow_graphics_point_clouds_amd import synthetic
+    from tests.deformable_reference import check_deformable_kpconv
     rng = np.random.default_rng(17)
-    batch, radius, c_in, c_out, kpn = 2, 0.2, 16, 8, 15
+    batch, radius, kpn = 2, 0.2, 15
     pts, bids, ctr, cb, nbh = _setup(oracle, rng, n=1500, n_out=400, batch=batch, radius=radius)
     feat = rng.standard_normal((len(pts), c_in)).astype(np.float32)
     kp = synthetic.spherical_kernel_points(15, rotate=False) * 0.8
     wts = (rng.standard_normal((kpn * c_in, c_out)) * 0.1).astype(np.float32)
-    woff = (rng.standard_normal((kpn * c_in, kpn * 3)) * 0.002).astype(np.float32)
-    influence = 0.5 * radius
-    sigma = influence / radius
-    ids = torch.tensor(nbh.original_neigh_ids).long()
-    radii = np.full(3, np.float32(radius), np.float32)
-    delta = torch.tensor(((pts[ids[:, 0]] - ctr[ids[:, 1]]) / radii).astype(np.float64))
-    tkp = torch.tensor(kp.astype(np.float64) * 0.75)
-
-    def weight(dist):
-        if kind == "linear":
-            return torch.relu(1 - dist / sigma)
-        return torch.exp(-(dist / (sigma / 3)) ** 2)
-
-    tf = torch.tensor(feat.astype(np.float64), requires_grad=True)
-    tw = torch.tensor(wts.astype(np.float64), requires_grad=True)
-    two = torch.tensor(woff.astype(np.float64), requires_grad=True)
-
-    def project(basis):
-        per_pair = tf[ids[:, 0]][:, :, None] * basis[:, None, :]
-        return torch.zeros(len(ctr), c_in, kpn, dtype=torch.float64).index_add(
-            0, ids[:, 1], per_pair)
-
-    rigid = weight((delta[:, None, :] - tkp[None]).norm(dim=2))
-    off = (project(rigid).reshape(len(ctr), -1) @ two).reshape(len(ctr), kpn, 3)
-    dist = (delta[:, None, :] - (tkp[None] + off[ids[:, 1]])).norm(dim=2)
-    ref_out = project(weight(dist)).reshape(len(ctr), -1) @ tw
-    fit = torch.full((len(ctr), kpn), float("inf"), dtype=torch.float64).scatter_reduce(
-        0, ids[:, 1][:, None].expand(-1, kpn), (dist / sigma) ** 2, "amin")
-    kpd = tkp[None] + off
-    kd = (kpd[:, None] - kpd[:, :, None] + 1e-300).norm(dim=3)
-    rep = weight(kd) * (1 - torch.eye(kpn, dtype=torch.float64))[None]
-    ref_loss = fit.sum() + rep.sum()
-
-    conv = layers.KPConv(c_in, c_out, custom_kernel_points=kp, kp_interpolation=kind,
-                         weights=dev(wts),
-                         deformable=True, offset_weights=dev(woff))
-    tfeat = dev(feat).requires_grad_(True)
-    out = conv(tfeat, pc.PointCloud(dev(pts), dev(bids), batch),
-               pc.PointCloud(dev(ctr), dev(cb), batch), radius, kernel_influence_dist=influence)
-    loss = conv.regularization_loss()
-    normwise(out.detach().cpu().numpy(), ref_out.detach().numpy(), tol=2e-5)
-    np.testing.assert_allclose(float(loss.detach()), float(ref_loss.detach()), rtol=2e-5)
-
-    up = rng.standard_normal(ref_out.shape).astype(np.float32)
-    (out * dev(up)).sum().backward(retain_graph=True)
-    (ref_out * torch.tensor(up.astype(np.float64))).sum().backward(retain_graph=True)
-    normwise(tfeat.grad.cpu().numpy(), tf.grad.numpy(), tol=5e-5)
-    normwise(conv.weights.grad.cpu().numpy(), tw.grad.numpy(), tol=5e-5)
-    normwise(conv.offset_weights.grad.cpu().numpy(), two.grad.numpy(), tol=1e-4)
-    for t in (tfeat, conv.weights, conv.offset_weights, tf, tw, two):
-        t.grad = None
-    loss.backward()
-    ref_loss.backward()
-    normwise(conv.offset_weights.grad.cpu().numpy(), two.grad.numpy(), tol=1e-4)
-    normwise(tfeat.grad.cpu().numpy(), tf.grad.numpy(), tol=1e-4)
+    # offsets of about N(0, 0.02): enough to separate the layout's two coincident pairs
+    woff = (rng.standard_normal((kpn * c_in, kpn * 3)) * 2.0 / c_in).astype(np.float32)
+    check_deformable_kpconv(pts, bids, ctr, cb, batch, nbh.original_neigh_ids, radius, feat, kp,
+                            wts, woff, 0.5 * radius, kind)
 
 
 @pytest.mark.parametrize("c", [1, 4, 5, 16, 64, 100, 128, 256])
