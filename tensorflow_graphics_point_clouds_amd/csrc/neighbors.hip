@@ -6,11 +6,11 @@
 //           a binary search over the descending keys give the contiguous slice
 //           of sorted points that lies in the offset cell row
 //           (find_ranges_grid_ds_kernels.cu.cc:48-235);
-//   count   16 lanes per centre stride over the slices and test
+//   count   8 lanes per centre stride over the slices and test
 //           |(s - p) * inv_radii| < 1 (count_neighbors_kernels.cu.cc:83-86; as the
 //           squared length against 1, which decides identically);
 //   fill    same traversal; the slot of a hit is the centre's start offset plus
-//           a ballot prefix inside the 16-lane group, so the pairs of a centre
+//           a ballot prefix inside the 8-lane group, so the pairs of a centre
 //           come out in ascending sorted-point index without atomics or a sort.
 // Offsets are enumerated so that the slices of a centre ascend in index.
 // (Keeping the count pass's hit masks for the fill pass, so that it need not load
@@ -25,7 +25,11 @@
 
 namespace mccnn {
 
-constexpr int kGroup = 16;                 // lanes per centre
+// 8 lanes per centre: with the unreachable cells left out a slice holds one or two cells,
+// and a wavefront steps through the union of what its centres need, so narrow groups
+// waste fewer lanes (16 lanes: 7 % slower on the dense case, 10 % on clustered clouds;
+// 32 lanes: 25 % slower).
+constexpr int kGroup = 8;                  // lanes per centre
 constexpr int kNbrThreads = 256;
 constexpr int kCentresPerBlock = kNbrThreads / kGroup;
 
@@ -45,13 +49,17 @@ __global__ void __launch_bounds__(256) nbr_ranges_kernel(
     int64_t ns, const float *__restrict__ samples, const int *__restrict__ sbids,
     const int64_t *__restrict__ keys, const int2 *__restrict__ ds,
     const int *__restrict__ num_cells, const float *__restrict__ smin,
-    const float *__restrict__ inv_cell, int2 *__restrict__ ranges) {
+    const float *__restrict__ inv_cell, const float *__restrict__ inv_radii,
+    int2 *__restrict__ ranges) {
   constexpr int R = OffsetInfo<D>::count();
   constexpr int OD = OffsetInfo<D>::kDims;
   const GridShape<D> g = load_shape<D>(num_cells);
-  float ic[D];
+  float ic[D], rho[D];                 // rho: one cell in units of the radius
 #pragma unroll
-  for (int d = 0; d < D; ++d) ic[d] = inv_cell[d];
+  for (int d = 0; d < D; ++d) {
+    ic[d] = inv_cell[d];
+    rho[d] = inv_radii[d] / ic[d];
+  }
   const int64_t total = ns * R;
   for (int64_t t = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; t < total;
        t += (int64_t)gridDim.x * blockDim.x) {
@@ -66,14 +74,37 @@ __global__ void __launch_bounds__(256) nbr_ranges_kernel(
     }
     int cell[D];
     cell_of_point<D>(p, m, ic, g, cell);
-    // offset digits, most significant = dim 0, value 1 - digit (descending)
+    // The centre in cell units, as the keys were computed, and what rounding can have
+    // moved a point across a cell face: a point filed under cell x has a true
+    // coordinate within `slack` of [x, x + 1) (outermost cells: unbounded outwards).
+    float rel[D], slack[D];
+#pragma unroll
+    for (int d = 0; d < D; ++d) {
+      const float prod = p[d] * ic[d];
+      rel[d] = prod - m[d];
+      slack[d] = 9.6e-7f * (fabsf(prod) + fabsf(m[d]) + 1.0f);       // 8 float epsilons
+    }
+    // offset digits, most significant = dim 0, value 1 - digit (descending); g2 = lower
+    // bound of the squared scaled distance to any point of the offset cell row, taken
+    // over the offset dimensions
     bool inside = true;
+    float g2 = 0.0f;
 #pragma unroll
     for (int d = OD - 1; d >= 0; --d) {
-      cell[d] += 1 - (r % 3);
+      const int off = 1 - (r % 3);
       r /= 3;
+      float gap = off < 0 ? rel[d] - (float)cell[d]
+                          : (off > 0 ? (float)(cell[d] + 1) - rel[d] : 0.0f);
+      gap = fmaxf(gap - slack[d], 0.0f) * rho[d];
+      g2 += gap * gap;
+      cell[d] += off;
       inside = inside && cell[d] >= 0 && cell[d] < g.n[d];
     }
+    // Cells that no pair of the exact test can come from are left out: every candidate
+    // dropped here has a scaled distance of at least sqrt(1 + 1e-5) > 1, whatever the
+    // rounding of the test itself (a few 1e-7), so the pairs found do not change.
+    g2 *= 0.99999f;
+    inside = inside && g2 < 1.0f;
     int2 out = make_int2(0, 0);
     if (inside) {
       const int64_t col = ((int64_t)b * g.n[0] + cell[0]) * g.n[1] + cell[1];
@@ -83,9 +114,19 @@ __global__ void __launch_bounds__(256) nbr_ranges_kernel(
           out = span;
         } else {
           const int64_t aux = key_of_cell<D>(cell, g, b);
-          const int w = cell[D - 1];
-          const int64_t maxk = aux + (w < g.n[D - 1] - 1 ? 1 : 0);
-          const int64_t mink = aux - (w > 0 ? 1 : 0);
+          const int w = cell[D - 1], nw = g.n[D - 1];
+          // last dimension: the cells w - 1 .. w + 1 of the reference, cut to those the
+          // sphere can reach given the offset in the other dimensions (out-of-range
+          // coordinates belong to the outermost cells)
+          const float reach = sqrtf(1.0f - g2) / rho[D - 1] * 1.00001f + slack[D - 1];
+          int wlo = (int)floorf(fmaxf(rel[D - 1] - reach, -1.0f));
+          int whi = (int)floorf(fminf(rel[D - 1] + reach, (float)nw));
+          wlo = wlo < 0 ? 0 : (wlo > nw - 1 ? nw - 1 : wlo);
+          whi = whi < 0 ? 0 : (whi > nw - 1 ? nw - 1 : whi);
+          wlo = wlo > w - 1 ? wlo : (w > 0 ? w - 1 : 0);
+          whi = whi < w + 1 ? whi : (w < nw - 1 ? w + 1 : nw - 1);
+          const int64_t maxk = aux + (whi - w);
+          const int64_t mink = aux + (wlo - w);
           int lo = span.x, hi = span.y;
           while (lo < hi) {                       // first index with key <= maxk
             const int mid = lo + ((hi - lo) >> 1);
@@ -97,7 +138,7 @@ __global__ void __launch_bounds__(256) nbr_ranges_kernel(
             const int mid = lo + ((hi - lo) >> 1);
             if (keys[mid] >= mink) lo = mid + 1; else hi = mid;
           }
-          if (lo > first) out = make_int2(first, lo);
+          if (lo > first && whi >= wlo) out = make_int2(first, lo);
         }
       }
     }
@@ -291,7 +332,8 @@ extern "C" int mccnn_find_neighbors_count(
                    hipLaunchKernelGGL(nbr_ranges_kernel<D>, dim3(blocks_for(work, 256)), dim3(256),
                                       0, s, num_samples, samples, sample_batch_ids,
                                       (const int64_t *)point_keys, (const int2 *)grid_ds,
-                                      num_cells, scaled_aabb_min, inv_cell_sizes, w.ranges));
+                                      num_cells, scaled_aabb_min, inv_cell_sizes, inv_radii,
+                                      w.ranges));
   MCCNN_LAUNCH_CHECK();
   const unsigned grid = blocks_for(num_samples, kCentresPerBlock);
   MCCNN_DIM_SWITCH(num_dims, hipLaunchKernelGGL((nbr_visit_kernel<D, false>), dim3(grid),
