@@ -50,16 +50,26 @@ __global__ void __launch_bounds__(kPdfThreads) compute_pdf_kernel(
 #pragma unroll
   for (int d = 0; d < D; ++d) p[d] = pts[c * D + d];
   const int64_t a = c > 0 ? ranges[c - 1] : 0, b = ranges[c];
+  // four pairs per lane and trip: their index loads, then their coordinate gathers, are
+  // in flight together (the sums keep the order of a one-pair-per-trip loop)
   float acc = 0.0f;
-  for (int64_t m = a + sub; m < b; m += kPdfGroup) {
-    const int64_t j = nbrs[m].x;
-    float e = 0.0f;
+  for (int64_t m = a + sub; m < b; m += 4 * kPdfGroup) {
+    int64_t j[4];
 #pragma unroll
-    for (int d = 0; d < D; ++d) {
-      const float u = (pts[j * D + d] - p[d]) * sc.s[d];
-      e += u * u;
+    for (int q = 0; q < 4; ++q) j[q] = m + q * kPdfGroup < b ? nbrs[m + q * kPdfGroup].x : -1;
+    float e[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      e[q] = 0.0f;
+      const int64_t jj = j[q] < 0 ? c : j[q];
+#pragma unroll
+      for (int d = 0; d < D; ++d) {
+        const float u = (pts[jj * D + d] - p[d]) * sc.s[d];
+        e[q] += u * u;
+      }
     }
-    acc += expf(-0.5f * e);
+#pragma unroll
+    for (int q = 0; q < 4; ++q) acc += j[q] < 0 ? 0.0f : expf(-0.5f * e[q]);
   }
 #pragma unroll
   for (int off = kPdfGroup / 2; off > 0; off >>= 1) acc += __shfl_xor(acc, off, kWave);
