@@ -192,9 +192,9 @@ __device__ __forceinline__ void project_pairs(const char *__restrict__ feat_base
         if constexpr (kStrided) {
 #pragma unroll
           for (int j = 0; j < kCPL; ++j)
-            f[u].v[j] = *reinterpret_cast<const float *>(feat_base + rn + lane_off + j * 64);
+            f[u].v[j] = *reinterpret_cast<const float *>(feat_base + (size_t)(rn + lane_off) + j * 64);
         } else {
-          f[u] = load_vec<kCPL>(reinterpret_cast<const float *>(feat_base + rn + lane_off), true);
+          f[u] = load_vec<kCPL>(reinterpret_cast<const float *>(feat_base + (size_t)(rn + lane_off)), true);
         }
         w[u] = basis(gn);
       }

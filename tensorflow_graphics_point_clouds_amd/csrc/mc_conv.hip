@@ -151,10 +151,11 @@ __device__ __forceinline__ void project_run_body(
       for (int u = 0; u < kFusedUnroll; ++u) {
         const int n = 4 * (t + u) + quarter;
         const float4 gn = stage->geo[n];
+        // one 32-bit lane offset on the wavefront's (scalar) base address
         const unsigned rn = stage->row[n];
 #pragma unroll
         for (int j = 0; j < kCPL; ++j)
-          f[u].v[j] = *reinterpret_cast<const float *>(feat_base + rn + lane_off + j * 64);
+          f[u].v[j] = *reinterpret_cast<const float *>(feat_base + (size_t)(rn + lane_off) + j * 64);
         int aux = 0;
         if constexpr (Basis::kUsesAux) aux = stage->aux[n];
 #pragma unroll
