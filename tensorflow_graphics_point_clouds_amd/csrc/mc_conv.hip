@@ -45,7 +45,7 @@ __device__ __forceinline__ void project_run_body(
   constexpr int K = kFusedK * KT;          // basis columns, KT tiles of 16
   constexpr int kCW = 16 * kCPL;
   const int lane = lane_id();
-  const int64_t wid = wave_slot();
+  const int64_t wid = wave_slot_xcd();
   const int64_t run = wid / chunks;
   const int64_t c0 = run * kProjRun;
   if (c0 >= n_out) return;
@@ -501,8 +501,9 @@ __global__ void __launch_bounds__(256) mc_conv_weight_grads16_kernel(
   // (grid-ordered) centres and the feature rows of that window stay in L2.
   // (Giving each XCD its own contiguous eighth of the centres instead was measured
   // on the scene-scale case, for this kernel and the projection: 12 % slower; dealing
-  // groups of 4 to 64 consecutive blocks to the XCDs in turn: no different.)
-  const int64_t first = wave_slot() * kGradRun;
+  // windows of consecutive blocks to the XCDs in turn leaves the time as it is and
+  // cuts the re-fetched feature rows.)
+  const int64_t first = wave_slot_xcd() * kGradRun;
   const int64_t last = first + kGradRun < n_out ? first + kGradRun : n_out;
   for (int64_t centre = first; centre < last; ++centre) {
     const int a = centre > 0 ? ranges[centre - 1] : 0, b = ranges[centre];

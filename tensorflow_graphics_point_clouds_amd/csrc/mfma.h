@@ -18,6 +18,24 @@ __device__ __forceinline__ int64_t wave_slot() {
       (int)(blockIdx.x * kWavesPerBlock + threadIdx.x / kWave));
 }
 
+// The same with the blocks renumbered for the eight XCDs, each of which has its own L2:
+// the hardware deals consecutive blocks to the XCDs in turn (block b runs on XCD b % 8),
+// so plain numbering sends neighbouring centres -- which share most of their feature
+// rows on a grid-ordered table -- to eight different caches, and each row is fetched from
+// HBM up to eight times.  Here XCD x works through windows of kXcdWindow consecutive
+// virtual blocks (x, x + 8, x + 16, ... in units of windows), so its resident blocks are
+// neighbours.  Measured on the 763 k-point scene batch (projection kernel): read requests
+// to the fabric 28.9 M -> 6.3 M per launch at equal run time (windows of 8 / 32 / 128 /
+// 512 blocks: 14.3 / 10.1 / 6.3 / 6.6 M; one contiguous eighth per XCD is 10 % slower,
+// the XCDs then finish at different times on clustered clouds).
+constexpr unsigned kXcdWindow = 128;
+__device__ __forceinline__ int64_t wave_slot_xcd() {
+  const unsigned b = blockIdx.x;
+  const unsigned full = gridDim.x / (8 * kXcdWindow) * (8 * kXcdWindow);   // the rest keeps its number
+  const unsigned v = b < full ? ((b / (8 * kXcdWindow)) * 8 + b % 8) * kXcdWindow + (b / 8) % kXcdWindow : b;
+  return __builtin_amdgcn_readfirstlane((int)(v * kWavesPerBlock + threadIdx.x / kWave));
+}
+
 __device__ __forceinline__ int64_t centre_of(int64_t slot_centre, const int *__restrict__ order) {
   return order ? (int64_t)__builtin_amdgcn_readfirstlane(order[slot_centre]) : slot_centre;
 }
