@@ -134,15 +134,26 @@ __global__ void __launch_bounds__(256) nt_product_kernel(int64_t n, int R,
 #pragma unroll
       for (int j = 0; j < 4; ++j)
         acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.v[s], b[j][s], acc[j], 0, 0, 0);
-    // acc[j][r]: point 16 t + 4*kk + r, column col0 + 4*c16 + j
+    // acc[j][r]: point 16 t + 4*kk + r, column col0 + 4*c16 + j.  The four rows leave from
+    // four register tuples of their own: a store fetches its data only when the memory
+    // pipeline gets to it, and whatever overwrites a register with a store pending on it
+    // (the next row's copy, the next tile's matrix instructions) waits for that fetch.
+    v4f rows[4];
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-      const int64_t pt = 16 * t + 4 * kk + r;
-      if (pt < n) {
-        const v4f v = {acc[0][r], acc[1][r], acc[2][r], acc[3][r]};
-        // streamed: the product is read once, by a later kernel
-        __builtin_nontemporal_store(v, reinterpret_cast<v4f *>(out + pt * R + col0 + 4 * c16));
-      }
+      rows[r] = v4f{acc[0][r], acc[1][r], acc[2][r], acc[3][r]};
+      asm volatile("" : "+v"(rows[r]));
+    }
+    float *o = out + (16 * t + 4 * kk) * R + col0 + 4 * c16;
+    if (16 * t + 16 <= n) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r)   // streamed: the product is read once, by a later kernel
+        __builtin_nontemporal_store(rows[r], reinterpret_cast<v4f *>(o + (int64_t)r * R));
+    } else {
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        if (16 * t + 4 * kk + r < n)
+          __builtin_nontemporal_store(rows[r], reinterpret_cast<v4f *>(o + (int64_t)r * R));
     }
     a = an;
   }
@@ -221,7 +232,14 @@ extern "C" int mccnn_projection_grad_product(mccnn_stream_t stream, int64_t num_
   MCCNN_REQUIRE(x && w && out, "projection_grad_product received a null tensor");
   hipStream_t s = as_stream(stream);
   const int F = num_cols_in, R = num_cols_out, groups = R / 256;
-  int slices = 2048 / groups;
+  // one round of blocks: the kernel keeps 3 blocks of 4 wavefronts resident per compute unit
+  // (136 registers), and a grid of exactly that many leaves no partly filled last round
+  // (2048 blocks on 256 units: 2.7 rounds, 8 % slower)
+  int device = 0, cus = 0;
+  MCCNN_HIP_CHECK(hipGetDevice(&device));
+  MCCNN_HIP_CHECK(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device));
+  int slices = 3 * cus / groups;
+  if (slices < 1) slices = 1;
   const int64_t tiles = (num_pts + 15) / 16;
   if (slices > tiles) slices = (int)tiles;
   const dim3 grid(groups * slices), block(256);

@@ -111,14 +111,26 @@ __device__ __forceinline__ void project_run_body(
   auto finish_centre = [&]() {          // store and clear the accumulators, move to the next centre
     const int64_t row = __builtin_amdgcn_readlane(my_row, cur);
     float *o = out_base + row * (int64_t)C * K;
+    // The tile leaves from copies of the accumulators: a store fetches its data from the
+    // register file only when the memory pipeline gets to it, and a matrix instruction
+    // that overwrites a register with a store pending on it waits for that fetch (in a
+    // micro-benchmark of 80 MFMAs + a 4 KB tile per round, storing the accumulators
+    // themselves takes 1.19 ms, storing copies 0.92 ms, the MFMAs alone 0.84 ms).
+    v4f tile[kCPL][KT];
 #pragma unroll
     for (int j = 0; j < kCPL; ++j)
 #pragma unroll
       for (int kt = 0; kt < KT; ++kt) {
-        __builtin_nontemporal_store(acc[j][kt],
-                                    reinterpret_cast<v4f *>(o + (j * 16 + col) * K + 16 * kt));
+        tile[j][kt] = acc[j][kt];
+        asm volatile("" : "+v"(tile[j][kt]));
         acc[j][kt] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
       }
+#pragma unroll
+    for (int j = 0; j < kCPL; ++j)
+#pragma unroll
+      for (int kt = 0; kt < KT; ++kt)
+        __builtin_nontemporal_store(tile[j][kt],
+                                    reinterpret_cast<v4f *>(o + (j * 16 + col) * K + 16 * kt));
     ++cur;
     cur_start = cur_end;
     cur_end = __builtin_amdgcn_readlane(my_end, cur < nc ? cur : nc - 1);
