@@ -317,6 +317,67 @@ def test_config5_kpconv_at_full_scene_size():
                          torch.einsum("mck,mk->c", dmag, bt))
 
 
+def test_config5_deformable_kpconv_at_full_scene_size():
+    """The deformable layer at configuration 5's real size (128 -> 128, 15 kernel points):
+    with the offset layer's weights at zero it reproduces the rigid layer (both fp32 paths,
+    so 2e-5 between them); with learned offsets, sampled output rows equal the float64
+    sum over the layer's own pairs with each centre's kernel points shifted by the offsets
+    the layer reports (`last_offsets`), and the output is linear in the convolution
+    weights: <up, conv(x)> == <dW, W>."""
+    from tensorflow_graphics_point_clouds_amd import layers, pc, synthetic
+    cfg = synthetic.config5()
+    cloud = pc.PointCloud(dev(cfg["points"]), dev(cfg["batch_ids"]), cfg["batch_size"])
+    radius, c, kpn = cfg["radius"], 128, 15
+    n = cloud._points.shape[0]
+    kp = synthetic.spherical_kernel_points(15, rotate=False) * 0.8
+    gen = torch.Generator(device="cuda").manual_seed(8)
+    x = torch.randn((n, c), device="cuda", generator=gen)
+    up = torch.randn((n, c), device="cuda", generator=gen)
+    rigid = layers.KPConv(c, c, custom_kernel_points=kp, seed=2)
+    with torch.no_grad():
+        ref = rigid(x, cloud, cloud, radius)
+    nbh = rigid.last_neighborhood
+    conv = layers.KPConv(c, c, custom_kernel_points=kp, deformable=True, seed=2,
+                         weights=rigid.weights.detach().clone(),
+                         offset_weights=torch.zeros((c * kpn, kpn * 3), device="cuda"))
+    with torch.no_grad():
+        out0 = conv(x, cloud, cloud, radius, neighborhood=nbh)
+    assert float(conv.last_offsets.abs().max()) == 0.0
+    assert float((out0 - ref).abs().max()) <= 2e-5 * float(ref.abs().max())
+
+    woff = 2e-4 * torch.randn((c * kpn, kpn * 3), device="cuda", generator=gen)
+    with torch.no_grad():
+        conv.offset_weights.copy_(woff)
+    out = conv(x, cloud, cloud, radius, neighborhood=nbh)
+    out.backward(up)
+    off = conv.last_offsets.detach().double()                      # [N, 15, 3]
+    assert 1e-3 < float(off.abs().max()) < 0.5
+    terms = up.double() * out.detach().double()
+    lhs, scale = float(terms.sum()), float(terms.abs().sum())
+    assert abs(lhs - float((conv.weights.grad.double() * conv.weights.detach().double()).sum())) \
+        <= REL * scale
+
+    pts = cloud._points.double()
+    tkp = torch.as_tensor(kp.astype(np.float64) * 0.75).cuda()
+    ids = nbh._original_neigh_ids.long()
+    ranges = nbh._samples_neigh_ranges.long()
+    w3 = conv.weights.detach().double().reshape(c, kpn, c)
+    rng = np.random.default_rng(1)
+    picks = torch.as_tensor(rng.choice(n, 100, replace=False), device="cuda")
+    starts = torch.where(picks > 0, ranges[(picks - 1).clamp(min=0)], torch.zeros_like(picks))
+    xs = x.double()
+    for centre, a, e in zip(picks.tolist(), starts.tolist(), ranges[picks].tolist()):
+        seg = torch.arange(a, e, device="cuda")
+        diff = (pts[ids[seg, 0]] - pts[centre]) / radius
+        dist = (diff[:, None, :] - tkp[None] - off[centre][None]).norm(dim=2)
+        bas = torch.relu(1 - dist)
+        proj = torch.einsum("mc,mk->ck", xs[ids[seg, 0]], bas)
+        pmag = torch.einsum("mc,mk->ck", xs[ids[seg, 0]].abs(), bas)
+        # 2e-5: the offsets enter in float32 on the GPU and in float64 here
+        assert_rel_t(out[centre].detach(), torch.einsum("ck,ckf->f", proj, w3),
+                     torch.einsum("ck,ckf->f", pmag, w3.abs()), tol=2e-5)
+
+
 # ------------------------------------------------------------ configuration 4 ----
 
 def _chunked_dot(a, b, chunk=1 << 27):
