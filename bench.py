@@ -627,6 +627,23 @@ def isolated_basis_proj(torch, pc, synthetic, tfg, _lib, radius=0.04, steps=5):
             if traffic:
                 entry["traffic_frac"] = round(traffic / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
             res[name + tag] = entry
+        # the atomic-free variant: per-pair rows of the feature gradient written to a
+        # [M, C] workspace and summed per point over the transposed pair lists (built once
+        # per neighbourhood, timed separately)
+        if tfg.gathered_grads_supported(C, K):
+            tr = tfg.transpose_neighbors(ids, N)
+            tfg.basis_proj_grads(basis, feat, ids, ranges, up, None, transposed=tr)
+            _lib.start_timing()
+            for _ in range(steps):
+                tr = tfg.transpose_neighbors(ids, N)
+                tfg.basis_proj_grads(basis, feat, ids, ranges, up, None, transposed=tr)
+            t = _lib.collect_timing()
+            ms = sum(t["basis_proj_grads_gathered"]) / steps
+            by = op_bytes("basis_proj_grads", M, N, N, C, K, 3)
+            entry = {"ms": ms, "transpose_neighbors_ms": sum(t["transpose_neighbors"]) / steps,
+                     "workspace_bytes": 4 * M * C}
+            entry.update(roofline_entry(compulsory_bytes("basis_proj_grads", M, N, N, C, K, 3), by, ms))
+            res["basis_proj_grads_gathered" + tag] = entry
 
     # the reference's call pattern: pairs address the features by original point id
     # (custom_ops_wrapper.py:185-189), points and centres in the caller's (random) order

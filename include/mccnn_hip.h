@@ -602,9 +602,12 @@ int mccnn_kp_conv_layer(mccnn_stream_t stream, int num_dims, int64_t num_pts,
  * weights (the tf.matmul of MCConv.py:187 / KPConv.py:226-230) for x [N, R] in
  * HBM and w [R, F].  One block per compute unit keeps all of w in registers and
  * streams x through LDS tiles of 16 rows, reading it exactly once; sums in a
- * fixed order (bit-reproducible).  Supported: R in {256, 512, 1024}, F in {16,
- * 32, 64, 128}, R*F <= 65536.  No counterpart among the reference's ops
- * (TensorFlow's matmul). */
+ * fixed order (bit-reproducible).  One launch covers a block of up to 1024 rows
+ * and up to 128 columns of w with at most 65536 weights; larger w (R a multiple
+ * of 256 up to 8192, F a multiple of 16 up to 1024) take one launch per block,
+ * x being read once per column block and the later row blocks adding to what
+ * the earlier ones wrote, in launch order.  No counterpart among the
+ * reference's ops (TensorFlow's matmul). */
 int mccnn_final_product_supported(int num_cols_in, int num_cols_out);
 int mccnn_final_product(mccnn_stream_t stream, int64_t num_rows, int num_cols_in,
                         const float *x, int num_cols_out, const float *w,
@@ -627,8 +630,9 @@ int mccnn_weight_grad_product(mccnn_stream_t stream, int64_t num_pts,
 /* out[n, r] = sum_f x[n, f] * w[r, f]: the gradient of the projection entering a
  * layer's final product (x = output gradient [N, F], w = final weights [R, F],
  * out [N, R]); write-bound, each wavefront keeps its slice of w in registers.
- * Supported: F in {16,32,64}, R a multiple of 256.  No counterpart among the
- * reference's ops (TensorFlow's matmul gradient). */
+ * Supported: F in {16,32,64} with R a multiple of 256, F = 128 with R a multiple
+ * of 128, F = 256 with R a multiple of 64.  No counterpart among the reference's
+ * ops (TensorFlow's matmul gradient). */
 int mccnn_projection_grad_product_supported(int num_cols_in, int num_cols_out);
 int mccnn_projection_grad_product(mccnn_stream_t stream, int64_t num_pts,
                                   int num_cols_in, const float *x,

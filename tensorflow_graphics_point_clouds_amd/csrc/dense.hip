@@ -92,26 +92,34 @@ __global__ void __launch_bounds__(256) tn_reduce_kernel(int64_t elems, int slice
 // out[n, r] = sum_f x[n, f] * w[r, f]: the gradient of the projection that enters
 // a layer's final product (x = output gradient [N, F], w = dense final weights
 // [R, F], R = C * K).  Write-bound: 4 R bytes per point leave, 4 F arrive.  A
-// wavefront keeps its 64 x F slice of w in registers for its whole life and
-// streams tiles of 16 points through the matrix cores; a lane owns 4 consecutive
-// output columns so that every row of a tile leaves as 256 contiguous bytes.
-template <int F>
+// wavefront keeps its (16 kCols) x F slice of w in registers for its whole life (64
+// registers: kCols = 4 columns per lane up to F = 64, 2 for F = 128, 1 for F = 256) and
+// streams tiles of 16 points through the matrix cores; a lane owns kCols consecutive
+// output columns so that every row of a tile leaves as 64 kCols contiguous bytes.
+template <int kCols> struct ColVec;
+template <> struct ColVec<4> { using type = v4f; };
+template <> struct ColVec<2> { using type = v2f; };
+template <> struct ColVec<1> { using type = float; };
+
+template <int F, int kCols>
 __global__ void __launch_bounds__(256) nt_product_kernel(int64_t n, int R,
                                                          const float *__restrict__ x,
                                                          const float *__restrict__ w,
                                                          int slices, float *__restrict__ out) {
+  using Row = typename ColVec<kCols>::type;
   constexpr int kSteps = F / 4;            // reduction steps; lane (kk, row) owns f = kk*kSteps + s
+  constexpr int kWaveCols = 16 * kCols;    // output columns of a wavefront
   const int lane = lane_id(), wave = threadIdx.x / kWave;
   const int kk = lane >> 4, c16 = lane & 15;
-  const int groups = R >> 8;
+  const int groups = R / (4 * kWaveCols);
   const int grp = blockIdx.x % groups, slice = blockIdx.x / groups;
-  const int col0 = grp * 256 + wave * 64;
-  // B operand of step s, column tile j: w[col0 + 4*c16 + j][kk*kSteps + s]
-  float b[4][kSteps];
+  const int col0 = (grp * 4 + wave) * kWaveCols;
+  // B operand of step s, column tile j: w[col0 + kCols*c16 + j][kk*kSteps + s]
+  float b[kCols][kSteps];
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const FVec<kSteps> t = load_vec<kSteps>(w + (int64_t)(col0 + 4 * c16 + j) * F + kk * kSteps,
-                                            true);
+  for (int j = 0; j < kCols; ++j) {
+    const FVec<kSteps> t = load_vec<kSteps>(
+        w + (int64_t)(col0 + kCols * c16 + j) * F + kk * kSteps, true);
 #pragma unroll
     for (int s = 0; s < kSteps; ++s) b[j][s] = t.v[s];
   }
@@ -126,41 +134,168 @@ __global__ void __launch_bounds__(256) nt_product_kernel(int64_t n, int R,
   FVec<kSteps> a = load_a(t0);
   for (int64_t t = t0; t < t1; ++t) {
     const FVec<kSteps> an = load_a(t + 1);
-    v4f acc[4];
+    v4f acc[kCols];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) acc[j] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+    for (int j = 0; j < kCols; ++j) acc[j] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
     for (int s = 0; s < kSteps; ++s)
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
+      for (int j = 0; j < kCols; ++j)
         acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.v[s], b[j][s], acc[j], 0, 0, 0);
-    // acc[j][r]: point 16 t + 4*kk + r, column col0 + 4*c16 + j.  The four rows leave from
+    // acc[j][r]: point 16 t + 4*kk + r, column col0 + kCols*c16 + j.  The four rows leave from
     // four register tuples of their own: a store fetches its data only when the memory
     // pipeline gets to it, and whatever overwrites a register with a store pending on it
     // (the next row's copy, the next tile's matrix instructions) waits for that fetch.
-    v4f rows[4];
+    Row rows[4];
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-      rows[r] = v4f{acc[0][r], acc[1][r], acc[2][r], acc[3][r]};
+      if constexpr (kCols == 4) rows[r] = v4f{acc[0][r], acc[1][r], acc[2][r], acc[3][r]};
+      else if constexpr (kCols == 2) rows[r] = v2f{acc[0][r], acc[1][r]};
+      else rows[r] = acc[0][r];
       asm volatile("" : "+v"(rows[r]));
     }
-    float *o = out + (16 * t + 4 * kk) * R + col0 + 4 * c16;
-    if (16 * t + 16 <= n) {
+    float *o = out + (16 * t + 4 * kk) * R + col0 + kCols * c16;
 #pragma unroll
-      for (int r = 0; r < 4; ++r)   // streamed: the product is read once, by a later kernel
-        __builtin_nontemporal_store(rows[r], reinterpret_cast<v4f *>(o + (int64_t)r * R));
-    } else {
-#pragma unroll
-      for (int r = 0; r < 4; ++r)
-        if (16 * t + 4 * kk + r < n)
-          __builtin_nontemporal_store(rows[r], reinterpret_cast<v4f *>(o + (int64_t)r * R));
-    }
+    for (int r = 0; r < 4; ++r)     // streamed: the product is read once, by a later kernel
+      if (16 * t + 16 <= n || 16 * t + 4 * kk + r < n)
+        __builtin_nontemporal_store(rows[r], reinterpret_cast<Row *>(o + (int64_t)r * R));
     a = an;
   }
 }
 
+static int nt_cols(int F) { return F <= 64 ? 4 : F == 128 ? 2 : 1; }
+
 static bool nt_supported(int F, int R) {
-  return (F == 16 || F == 32 || F == 64) && R >= 256 && R % 256 == 0;
+  if (!(F == 16 || F == 32 || F == 64 || F == 128 || F == 256)) return false;
+  const int block_cols = 64 * nt_cols(F);
+  return R >= block_cols && R % block_cols == 0;
+}
+
+// out[out_rows[n] or n, :] = x[n, :] * w for x [N, R], w [R, F] when w is too large to sit in
+// the registers of one block (R * F > 65536: the 128 -> 128 kernel-point layers, R = 2048):
+// the classic tiled product.  A block of four wavefronts owns a 128 x BN tile of the output
+// (wavefront (wm, wn): 64 x BN/2, i.e. 4 x BN/32 accumulator tiles) and walks the reduction
+// in steps of 32: the 128 x 32 block of x and the 32 x BN block of w of the next step are
+// fetched into registers while the current one is multiplied out of LDS (x rows as they
+// are, w transposed, rows 36 floats apart), two barriers per step.  The reduction index of a
+// matrix step may be permuted as long as both operands agree: lane quarter q takes indices
+// 4q .. 4q+3 of each group of 16, so every operand fetch is one 16-byte LDS read.
+// x is read once per column block (F / BN times); w comes from L2.  The lanes of a
+// wavefront fetch their pieces of w with the reduction index running fastest (32 rows of
+// w, 16 bytes of each), so that the four transposing LDS writes of a lane land in 32
+// consecutive banks; with the columns running fastest the fetch is coalesced but the
+// writes hit two banks 16 ways (0.9 G conflict cycles per launch, 104 instead of 113
+// TFLOP/s on [825 274, 2048] x [2048, 128]).  A second LDS buffer (one barrier per step)
+// costs a resident block per compute unit and is slower (107 TFLOP/s).
+constexpr int kTileRows = 128, kTileK = 32, kTileLd = kTileK + 4;
+
+template <int BN>
+__global__ void __launch_bounds__(256) tile_product_kernel(int64_t n, int R, int F,
+                                                           const float *__restrict__ x,
+                                                           const float *__restrict__ w,
+                                                           const int *__restrict__ out_rows,
+                                                           float *__restrict__ out) {
+  constexpr int kCT = BN / 32;                    // accumulator tiles per wavefront along the columns
+  constexpr int kBLoads = kTileK * BN / 4 / 256;  // float4 loads of w per thread and step
+  __shared__ __align__(16) float a_lds[kTileRows * kTileLd];
+  __shared__ __align__(16) float b_lds[BN * kTileLd];
+  const int t = threadIdx.x, lane = lane_id(), wave = t / kWave;
+  const int q = lane >> 4, c16 = lane & 15;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int col_blocks = F / BN;
+  const int64_t row0 = (int64_t)(blockIdx.x / col_blocks) * kTileRows;
+  const int col0 = (blockIdx.x % col_blocks) * BN;
+
+  v4f acc[4][kCT];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < kCT; ++j) acc[i][j] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+
+  // this thread's pieces of a step: 4 x (row, 4 k) of x, kBLoads x (k, 4 columns) of w
+  v4f xa[4], wb[kBLoads];
+  auto fetch = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int idx = t + 256 * i, row = idx >> 3, c4 = idx & 7;
+      xa[i] = row0 + row < n
+                  ? *reinterpret_cast<const v4f *>(x + (row0 + row) * R + k0 + 4 * c4)
+                  : v4f{0.0f, 0.0f, 0.0f, 0.0f};
+    }
+#pragma unroll
+    for (int i = 0; i < kBLoads; ++i) {
+      const int idx = t + 256 * i, kk = idx % kTileK, c4 = idx / kTileK;
+      wb[i] = *reinterpret_cast<const v4f *>(w + (int64_t)(k0 + kk) * F + col0 + 4 * c4);
+    }
+  };
+  auto park = [&]() {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int idx = t + 256 * i, row = idx >> 3, c4 = idx & 7;
+      *reinterpret_cast<v4f *>(a_lds + row * kTileLd + 4 * c4) = xa[i];
+    }
+#pragma unroll
+    for (int i = 0; i < kBLoads; ++i) {
+      const int idx = t + 256 * i, kk = idx % kTileK, c4 = idx / kTileK;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) b_lds[(4 * c4 + j) * kTileLd + kk] = wb[i][j];
+    }
+  };
+
+  const float *a_rd = a_lds + (wm * 64 + c16) * kTileLd + 4 * q;
+  const float *b_rd = b_lds + (wn * (BN / 2) + c16) * kTileLd + 4 * q;
+  fetch(0);
+  for (int k0 = 0; k0 < R; k0 += kTileK) {
+    __syncthreads();                  // the previous step has been multiplied
+    park();
+    __syncthreads();
+    if (k0 + kTileK < R) fetch(k0 + kTileK);
+#pragma unroll
+    for (int ks = 0; ks < kTileK / 16; ++ks) {
+      v4f a[4], b[kCT];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        a[i] = *reinterpret_cast<const v4f *>(a_rd + 16 * i * kTileLd + 16 * ks);
+#pragma unroll
+      for (int j = 0; j < kCT; ++j)
+        b[j] = *reinterpret_cast<const v4f *>(b_rd + 16 * j * kTileLd + 16 * ks);
+#pragma unroll
+      for (int s = 0; s < 4; ++s)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+          for (int j = 0; j < kCT; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[i][s], b[j][s], acc[i][j], 0, 0, 0);
+    }
+  }
+  // acc[i][j][r]: row row0 + 64 wm + 16 i + 4 q + r, column col0 + (BN/2) wn + 16 j + c16
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int64_t row = row0 + wm * 64 + 16 * i + 4 * q + r;
+      if (row < n) {
+        const int64_t orow = out_rows ? out_rows[row] : row;
+        float *o = out + orow * F + col0 + wn * (BN / 2) + c16;
+#pragma unroll
+        for (int j = 0; j < kCT; ++j) o[16 * j] = acc[i][j][r];
+      }
+    }
+}
+
+bool tile_product_supported(int R, int F) { return R >= 32 && R % 32 == 0 && F >= 64 && F % 64 == 0; }
+
+int launch_tile_product(hipStream_t s, int64_t n, int R, const float *x, int F, const float *w,
+                        const int *out_rows, float *out) {
+  const int64_t row_blocks = (n + kTileRows - 1) / kTileRows;
+  if (F % 128 == 0)
+    hipLaunchKernelGGL(tile_product_kernel<128>, dim3((unsigned)(row_blocks * (F / 128))),
+                       dim3(256), 0, s, n, R, F, x, w, out_rows, out);
+  else
+    hipLaunchKernelGGL(tile_product_kernel<64>, dim3((unsigned)(row_blocks * (F / 64))), dim3(256),
+                       0, s, n, R, F, x, w, out_rows, out);
+  MCCNN_LAUNCH_CHECK();
+  return MCCNN_OK;
 }
 
 static bool tn_supported(int C, int R) {
@@ -224,14 +359,14 @@ extern "C" int mccnn_projection_grad_product(mccnn_stream_t stream, int64_t num_
                                              int num_cols_in, const float *x, int num_cols_out,
                                              const float *w, float *out) {
   MCCNN_REQUIRE(nt_supported(num_cols_in, num_cols_out),
-                "projection_grad_product supports 16/32/64 input columns and a multiple of 256 "
-                "output columns (got %d -> %d)", num_cols_in, num_cols_out);
+                "projection_grad_product supports 16/32/64/128/256 input columns and a multiple of "
+                "256/256/256/128/64 output columns (got %d -> %d)", num_cols_in, num_cols_out);
   MCCNN_REQUIRE(num_pts >= 0 && num_pts < ((int64_t)1 << 31),
                 "projection_grad_product expects a size in [0, 2^31)");
   if (num_pts == 0) return MCCNN_OK;
   MCCNN_REQUIRE(x && w && out, "projection_grad_product received a null tensor");
   hipStream_t s = as_stream(stream);
-  const int F = num_cols_in, R = num_cols_out, groups = R / 256;
+  const int F = num_cols_in, R = num_cols_out, groups = R / (64 * nt_cols(F));
   // one round of blocks: the kernel keeps 3 blocks of 4 wavefronts resident per compute unit
   // (136 registers), and a grid of exactly that many leaves no partly filled last round
   // (2048 blocks on 256 units: 2.7 rounds, 8 % slower)
@@ -244,9 +379,11 @@ extern "C" int mccnn_projection_grad_product(mccnn_stream_t stream, int64_t num_
   if (slices > tiles) slices = (int)tiles;
   const dim3 grid(groups * slices), block(256);
   switch (F) {
-    case 64: hipLaunchKernelGGL(nt_product_kernel<64>, grid, block, 0, s, num_pts, R, x, w, slices, out); break;
-    case 32: hipLaunchKernelGGL(nt_product_kernel<32>, grid, block, 0, s, num_pts, R, x, w, slices, out); break;
-    default: hipLaunchKernelGGL(nt_product_kernel<16>, grid, block, 0, s, num_pts, R, x, w, slices, out); break;
+    case 256: hipLaunchKernelGGL((nt_product_kernel<256, 1>), grid, block, 0, s, num_pts, R, x, w, slices, out); break;
+    case 128: hipLaunchKernelGGL((nt_product_kernel<128, 2>), grid, block, 0, s, num_pts, R, x, w, slices, out); break;
+    case 64: hipLaunchKernelGGL((nt_product_kernel<64, 4>), grid, block, 0, s, num_pts, R, x, w, slices, out); break;
+    case 32: hipLaunchKernelGGL((nt_product_kernel<32, 4>), grid, block, 0, s, num_pts, R, x, w, slices, out); break;
+    default: hipLaunchKernelGGL((nt_product_kernel<16, 4>), grid, block, 0, s, num_pts, R, x, w, slices, out); break;
   }
   MCCNN_LAUNCH_CHECK();
   return MCCNN_OK;

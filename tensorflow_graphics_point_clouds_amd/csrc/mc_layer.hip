@@ -53,6 +53,14 @@ struct LayerShape {
       sizeof(float) * (kTileFloats + kPartialFloats) + sizeof(PairStage) * kLayerWaves;
 };
 
+// Row strides (in floats) of the dense product's operands when they are blocks of larger
+// matrices: x [N, ldx], W [., ldw], out [N, ldo]; `accumulate` adds to what `out` holds.
+// Zero means "the block is the whole matrix" (R, F and F).
+struct DenseStrides {
+  int64_t ldx = 0, ldw = 0, ldo = 0;
+  int accumulate = 0;
+};
+
 template <int kCPL, int FT, int D, class Basis, bool kDense = false>
 __device__ __forceinline__ void layer_body(int64_t n_out, const float *__restrict__ feat,
                                            const int2 *__restrict__ nbrs,
@@ -60,7 +68,7 @@ __device__ __forceinline__ void layer_body(int64_t n_out, const float *__restric
                                            const Basis &basis, const float *__restrict__ w,
                                            const int *__restrict__ out_rows,
                                            float *__restrict__ proj_out, float *__restrict__ out,
-                                           float *lds) {
+                                           float *lds, const DenseStrides ld = DenseStrides{}) {
   using S = LayerShape<kCPL, FT>;
   constexpr int C = S::C, R = S::R, F = S::F, kSteps = S::kSteps;
   float *tile = lds;
@@ -73,11 +81,13 @@ __device__ __forceinline__ void layer_body(int64_t n_out, const float *__restric
 
   // B operands of this wavefront: step s of lane (quarter, col) multiplies tile column
   // slice*kSliceRows + quarter*kSteps + s with W[that row][16 ft + col]
+  const int64_t ldx = kDense && ld.ldx ? ld.ldx : R, ldw = kDense && ld.ldw ? ld.ldw : F;
+  const int64_t ldo = kDense && ld.ldo ? ld.ldo : F;
   float wreg[kSteps];
   {
-    const float *wl = w + (int64_t)(slice * S::kSliceRows + quarter * kSteps) * F + 16 * ft + col;
+    const float *wl = w + (int64_t)(slice * S::kSliceRows + quarter * kSteps) * ldw + 16 * ft + col;
 #pragma unroll
-    for (int s = 0; s < kSteps; ++s) wreg[s] = wl[(int64_t)s * F];
+    for (int s = 0; s < kSteps; ++s) wreg[s] = wl[(int64_t)s * ldw];
   }
   const float *arow = tile + col * S::kTileStride + slice * S::kSliceRows + quarter * kSteps;
 
@@ -93,7 +103,7 @@ __device__ __forceinline__ void layer_body(int64_t n_out, const float *__restric
 #pragma unroll
       for (int i = 0; i < kRowLoads; ++i)
         xrow[i] = live ? __builtin_nontemporal_load(reinterpret_cast<const v4f *>(
-                             feat + row * R + 4 * (i * 64 + lane)))
+                             feat + row * ldx + 4 * (i * 64 + lane)))
                        : v4f{0.0f, 0.0f, 0.0f, 0.0f};
     }
   };
@@ -169,7 +179,9 @@ __device__ __forceinline__ void layer_body(int64_t n_out, const float *__restric
       for (int q = 0; q < S::kSlices; ++q) s += partial[q * 16 * F + e];
       if (centre0 + ce < n_out) {
         const int64_t orow = out_rows ? out_rows[centre0 + ce] : centre0 + ce;
-        out[orow * F + (e - ce * F)] = s;
+        float *dst = out + orow * ldo + (e - ce * F);
+        if (kDense && ld.accumulate) s += *dst;
+        *dst = s;
       }
     }
     // The next tile's rows are written after this barrier pair: every wavefront has
@@ -208,11 +220,11 @@ struct NoBasis {};
 template <int kCPL, int FT>
 __global__ void __launch_bounds__(kLayerThreads) final_product_kernel(
     int64_t n, const float *__restrict__ x, const float *__restrict__ w,
-    const int *__restrict__ out_rows, float *__restrict__ out) {
+    const int *__restrict__ out_rows, float *__restrict__ out, DenseStrides ld) {
   extern __shared__ __align__(16) float lds[];
   const McParams<3> none{};
   layer_body<kCPL, FT, 3, NoBasis, true>(n, x, nullptr, nullptr, none, NoBasis{}, w, out_rows,
-                                         nullptr, out, lds);
+                                         nullptr, out, lds, ld);
 }
 
 // One block per compute unit (the LDS tile and 1024 threads fill it), fewer if
@@ -375,9 +387,27 @@ extern "C" int mccnn_kp_conv_layer(mccnn_stream_t stream, int num_dims, int64_t 
   return MCCNN_OK;
 }
 
+// Blocks of the reduction and of the output columns that one launch covers: the
+// largest column block first (x is read once per column block), then the longest
+// reduction block whose weights still fit the registers of a block of wavefronts.
+static bool product_blocks(int R, int F, int *rb, int *fb) {
+  if (R < 256 || R % 256 != 0 || F < 16 || F % 16 != 0) return false;
+  for (int f = 128; f >= 16; f >>= 1) {
+    if (F % f != 0) continue;
+    for (int r = 1024; r >= 256; r >>= 1)
+      if (R % r == 0 && r * f <= 65536) {
+        *rb = r;
+        *fb = f;
+        return true;
+      }
+  }
+  return false;
+}
+
 extern "C" int mccnn_final_product_supported(int num_cols_in, int num_cols_out) {
-  return num_cols_in % kFusedK == 0 &&
-                 layer_supported(3, num_cols_in / kFusedK, kFusedK, num_cols_out)
+  int rb = 0, fb = 0;
+  return num_cols_in <= 8192 && num_cols_out <= 1024 &&
+                 product_blocks(num_cols_in, num_cols_out, &rb, &fb)
              ? 1 : 0;
 }
 
@@ -385,8 +415,8 @@ extern "C" int mccnn_final_product(mccnn_stream_t stream, int64_t num_rows, int 
                                    const float *x, int num_cols_out, const float *w,
                                    const int32_t *out_rows, float *out) {
   MCCNN_REQUIRE(mccnn_final_product_supported(num_cols_in, num_cols_out),
-                "final_product supports 256, 512 or 1024 input columns and 16, 32, 64 or 128 "
-                "output columns with at most 65536 weights (got %d x %d)", num_cols_in,
+                "final_product supports a multiple of 256 (at most 8192) input columns and a "
+                "multiple of 16 (at most 1024) output columns (got %d x %d)", num_cols_in,
                 num_cols_out);
   MCCNN_REQUIRE(num_rows >= 0 && num_rows < ((int64_t)1 << 31),
                 "final_product expects a size in [0, 2^31)");
@@ -396,11 +426,27 @@ extern "C" int mccnn_final_product(mccnn_stream_t stream, int64_t num_rows, int 
   unsigned blocks = 1;
   int rc = layer_grid(num_rows, &blocks);
   if (rc != MCCNN_OK) return rc;
-  MCCNN_LAYER_SHAPE_SWITCH(num_cols_in / kFusedK, num_cols_out,
-                           rc = launch_layer(final_product_kernel<CPL, FT>, s, blocks,
-                                             LayerShape<CPL, FT>::kLdsBytes, num_rows, x, w,
-                                             out_rows, out));
-  if (rc != MCCNN_OK) return rc;
-  MCCNN_LAUNCH_CHECK();
+  const int R = num_cols_in, F = num_cols_out;
+  if ((int64_t)R * F > 65536 && tile_product_supported(R, F))
+    return launch_tile_product(s, num_rows, R, x, F, w, out_rows, out);
+  int rb = 0, fb = 0;
+  product_blocks(R, F, &rb, &fb);
+  // out[:, f0:f0+fb] = sum over the reduction blocks r0 of x[:, r0:r0+rb] W[r0:r0+rb, f0:f0+fb]:
+  // one launch per (column block, reduction block), the later reduction blocks adding to
+  // what the earlier ones wrote (launches on one stream run in order: fixed summation order)
+  for (int f0 = 0; f0 < F; f0 += fb)
+    for (int r0 = 0; r0 < R; r0 += rb) {
+      DenseStrides ld;
+      ld.ldx = R;
+      ld.ldw = F;
+      ld.ldo = F;
+      ld.accumulate = r0 > 0;
+      MCCNN_LAYER_SHAPE_SWITCH(rb / kFusedK, fb,
+                               rc = launch_layer(final_product_kernel<CPL, FT>, s, blocks,
+                                                 LayerShape<CPL, FT>::kLdsBytes, num_rows, x + r0,
+                                                 w + (int64_t)r0 * F + f0, out_rows, out + f0, ld));
+      if (rc != MCCNN_OK) return rc;
+      MCCNN_LAUNCH_CHECK();
+    }
   return MCCNN_OK;
 }

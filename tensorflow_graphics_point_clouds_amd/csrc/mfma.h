@@ -51,8 +51,15 @@ static unsigned wave_grid(int64_t waves) {
 int launch_dfeat_gather(hipStream_t s, int64_t num_pts, int C, const int *point_ranges,
                         const int *pair_order, const float *pair_rows, float *dfeat);
 
+// out = x * w for x [N, R], w [R, F] as a tiled product (defined in dense.hip): for weight
+// matrices too large for the register-resident product of mc_layer.hip.
+bool tile_product_supported(int R, int F);
+int launch_tile_product(hipStream_t s, int64_t n, int R, const float *x, int F, const float *w,
+                        const int *out_rows, float *out);
+
 typedef float v16f __attribute__((ext_vector_type(16)));
 typedef float v4f __attribute__((ext_vector_type(4)));
+typedef float v2f __attribute__((ext_vector_type(2)));
 
 template <int N>
 struct FVec {

@@ -1,8 +1,9 @@
 """Convolution and pooling layers composed from the HIP ops, with the call
 signatures of the reference's layers (pylib/pc/layers/MCConv.py, KPConv.py,
 Pooling.py).  Per-pair basis evaluation, basis projection, pooling and all
-their gradients are kernels of libmccnn_hip.so; the dense
-[N, C*K] x [C*K, C_out] product is a plain library GEMM (torch.matmul)."""
+their gradients are kernels of libmccnn_hip.so, and so are the dense
+[N, C*K] x [C*K, C_out] product and its two gradient products for channel
+counts that are multiples of 16 (others fall back to torch.matmul)."""
 import math
 
 import numpy as np

@@ -86,7 +86,10 @@ def test_layer_entry_points_reject_uncovered_shapes(lib):
     assert lib.mccnn_weight_grad_product_supported(64, 1024) == 1
     assert lib.mccnn_weight_grad_product_supported(48, 1024) == 0
     assert lib.mccnn_projection_grad_product_supported(64, 1024) == 1
-    assert lib.mccnn_projection_grad_product_supported(128, 1024) == 0
+    assert lib.mccnn_projection_grad_product_supported(128, 1024) == 1
+    assert lib.mccnn_projection_grad_product_supported(96, 1024) == 0
+    assert lib.mccnn_final_product_supported(2048, 128) == 1
+    assert lib.mccnn_final_product_supported(1000, 128) == 0
     # K = 8 is not covered by the fused projection
     rc = lib.mccnn_mc_conv_project(None, 3, i64(10), None, 64, None, i64(10), None, i64(20), None,
                                    None, None, 8, 1, 0, None, None, None, None, None)
@@ -99,7 +102,7 @@ def test_layer_entry_points_reject_uncovered_shapes(lib):
     assert rc == 1 and b"kernel points" in lib.mccnn_last_error()
     rc = lib.mccnn_weight_grad_product(None, i64(10), 48, None, 1024, None, None, sz(0), None)
     assert rc == 1 and b"output rows" in lib.mccnn_last_error()
-    rc = lib.mccnn_projection_grad_product(None, i64(10), 128, None, 1024, None, None)
+    rc = lib.mccnn_projection_grad_product(None, i64(10), 96, None, 1024, None, None)
     assert rc == 1 and b"input columns" in lib.mccnn_last_error()
     # a feature table too large for 32-bit byte offsets is refused, not truncated
     rc = lib.mccnn_mc_conv_project(None, 3, i64(1 << 25), None, 64, None, i64(10), None, i64(20),

@@ -407,7 +407,9 @@ def test_weight_grad_product_matches_float64(n, c, r):
     assert np.abs(got - expect).max() <= 1e-5 * max(1.0, np.abs(expect).max())
 
 
-@pytest.mark.parametrize("n,f,r", [(1, 16, 256), (4099, 64, 1024), (20000, 32, 512), (0, 64, 256)])
+@pytest.mark.parametrize("n,f,r", [(1, 16, 256), (4099, 64, 1024), (20000, 32, 512), (0, 64, 256),
+                                   (4099, 128, 1024), (3001, 128, 2048), (1500, 256, 4096),
+                                   (17, 256, 64), (33, 128, 128)])
 def test_projection_grad_product_matches_float64(n, f, r):
     from tensorflow_graphics_point_clouds_amd import layers
     gen = torch.Generator(device="cuda").manual_seed(n + f)
@@ -421,16 +423,19 @@ def test_projection_grad_product_matches_float64(n, f, r):
 
 
 @pytest.mark.parametrize("n,r,f", [(1, 256, 16), (15, 256, 128), (4099, 1024, 64), (20000, 512, 128),
-                                   (333, 1024, 32), (5000, 512, 32), (0, 1024, 64), (70001, 1024, 16)])
+                                   (333, 1024, 32), (5000, 512, 32), (0, 1024, 64), (70001, 1024, 16),
+                                   (4099, 2048, 128), (3001, 1024, 128), (1500, 4096, 256),
+                                   (777, 2048, 48), (2000, 768, 192), (9000, 2048, 64)])
 def test_final_product_matches_float64(n, r, f):
-    """x w with all of w in the registers of each block, elementwise against float64
-    with the magnitude sum |x| |w| (1e-5), row permutation included; a second call must
-    return the same bits."""
+    """x w with a block of w in the registers of each block of wavefronts (one launch per
+    block of w for the larger shapes, later row blocks adding to the earlier ones),
+    elementwise against float64 with the magnitude sum |x| |w| (1e-5), row permutation
+    included; a second call must return the same bits."""
     from tensorflow_graphics_point_clouds_amd import _lib
     from tensorflow_graphics_point_clouds_amd._lib import cint, i64, ptr, stream
     assert _lib.lib().mccnn_final_product_supported(r, f) == 1
-    assert _lib.lib().mccnn_final_product_supported(2048, 64) == 0
-    assert _lib.lib().mccnn_final_product_supported(1024, 128) == 0
+    assert _lib.lib().mccnn_final_product_supported(2048 + 128, 64) == 0
+    assert _lib.lib().mccnn_final_product_supported(1024, 24) == 0
     gen = torch.Generator(device="cuda").manual_seed(n + f)
     x = torch.randn((n, r), device="cuda", generator=gen)
     w = torch.randn((r, f), device="cuda", generator=gen)
@@ -448,7 +453,7 @@ def test_final_product_matches_float64(n, r, f):
     if n:
         assert torch.equal(outs[1][rows.long()], outs[0])
     with pytest.raises(ValueError):
-        _lib.call("final_product", stream(), i64(n), cint(2048), ptr(x), cint(64), ptr(w),
+        _lib.call("final_product", stream(), i64(n), cint(2048 + 128), ptr(x), cint(64), ptr(w),
                   ptr(None), ptr(outs[0]))
 
 
