@@ -58,7 +58,8 @@ struct LayerShape {
 // Zero means "the block is the whole matrix" (R, F and F).
 struct DenseStrides {
   int64_t ldx = 0, ldw = 0, ldo = 0;
-  int accumulate = 0;
+  int r_total = 0;       // reduction length of the whole product, walked in blocks of R
+  int f_block = 0;       // columns per blockIdx.y
 };
 
 template <int kCPL, int FT, int D, class Basis, bool kDense = false>
@@ -83,15 +84,25 @@ __device__ __forceinline__ void layer_body(int64_t n_out, const float *__restric
   // slice*kSliceRows + quarter*kSteps + s with W[that row][16 ft + col]
   const int64_t ldx = kDense && ld.ldx ? ld.ldx : R, ldw = kDense && ld.ldw ? ld.ldw : F;
   const int64_t ldo = kDense && ld.ldo ? ld.ldo : F;
+  const int r_total = kDense && ld.r_total ? ld.r_total : R;
+  if constexpr (kDense) {           // this block's columns of a wider product
+    w += (int64_t)blockIdx.y * ld.f_block;
+    out += (int64_t)blockIdx.y * ld.f_block;
+  }
+  const float *arow = tile + col * S::kTileStride + slice * S::kSliceRows + quarter * kSteps;
+  const int64_t tiles = (n_out + kLayerWaves - 1) / kLayerWaves;
+  // A product whose weights exceed the block's registers walks the reduction in blocks of
+  // R rows of w: the block's tiles are visited once per block of rows, the later visits
+  // adding to what the earlier ones wrote (the same thread owns an output element in every
+  // visit, so the sum has a fixed order and needs no fence).
+  for (int r0 = 0; r0 < r_total; r0 += R, feat += kDense ? R : 0, w += (int64_t)R * ldw) {
   float wreg[kSteps];
   {
     const float *wl = w + (int64_t)(slice * S::kSliceRows + quarter * kSteps) * ldw + 16 * ft + col;
 #pragma unroll
     for (int s = 0; s < kSteps; ++s) wreg[s] = wl[(int64_t)s * ldw];
   }
-  const float *arow = tile + col * S::kTileStride + slice * S::kSliceRows + quarter * kSteps;
 
-  const int64_t tiles = (n_out + kLayerWaves - 1) / kLayerWaves;
   // dense producer: the wavefront's row of x, fetched one tile ahead (R / 256 loads of 16
   // bytes per lane, each covering one contiguous kilobyte of the row)
   constexpr int kRowLoads = R / 256;
@@ -180,7 +191,7 @@ __device__ __forceinline__ void layer_body(int64_t n_out, const float *__restric
       if (centre0 + ce < n_out) {
         const int64_t orow = out_rows ? out_rows[centre0 + ce] : centre0 + ce;
         float *dst = out + orow * ldo + (e - ce * F);
-        if (kDense && ld.accumulate) s += *dst;
+        if (kDense && r0 > 0) s += *dst;
         *dst = s;
       }
     }
@@ -188,6 +199,8 @@ __device__ __forceinline__ void layer_body(int64_t n_out, const float *__restric
     // left step 3 (second barrier) before any row of the tile changes, and every
     // thread has left step 4 before it reaches the next first barrier, after which
     // the partial sums change.
+  }
+  if (r0 + R < r_total) __syncthreads();   // step 4 of the last tile has read the partial sums
   }
 }
 
@@ -239,10 +252,10 @@ static int layer_grid(int64_t num_samples, unsigned *blocks) {
 }
 
 template <class Kernel, class... Args>
-static int launch_layer(Kernel kernel, hipStream_t s, unsigned blocks, size_t lds, Args... args) {
+static int launch_layer(Kernel kernel, hipStream_t s, dim3 blocks, size_t lds, Args... args) {
   MCCNN_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-  hipLaunchKernelGGL(kernel, dim3(blocks), dim3(kLayerThreads), lds, s, args...);
+  hipLaunchKernelGGL(kernel, blocks, dim3(kLayerThreads), lds, s, args...);
   return MCCNN_OK;
 }
 
@@ -427,26 +440,42 @@ extern "C" int mccnn_final_product(mccnn_stream_t stream, int64_t num_rows, int 
   int rc = layer_grid(num_rows, &blocks);
   if (rc != MCCNN_OK) return rc;
   const int R = num_cols_in, F = num_cols_out;
-  if ((int64_t)R * F > 65536 && tile_product_supported(R, F))
+  // weights beyond a block's registers: the tiled product, once its 128-row tiles give
+  // every compute unit a block (below that a launch is a few blocks walking the whole
+  // reduction alone: 170 us for 400 rows x 4096 x 256 against 20 us for the blocked
+  // register-resident product, whose tiles are 16 rows)
+  if ((int64_t)R * F > 65536 && tile_product_supported(R, F) &&
+      (num_rows + 127) / 128 * (F / (F % 128 == 0 ? 128 : 64)) >= (int64_t)blocks)
     return launch_tile_product(s, num_rows, R, x, F, w, out_rows, out);
   int rb = 0, fb = 0;
   product_blocks(R, F, &rb, &fb);
   // out[:, f0:f0+fb] = sum over the reduction blocks r0 of x[:, r0:r0+rb] W[r0:r0+rb, f0:f0+fb]:
-  // one launch per (column block, reduction block), the later reduction blocks adding to
-  // what the earlier ones wrote (launches on one stream run in order: fixed summation order)
-  for (int f0 = 0; f0 < F; f0 += fb)
-    for (int r0 = 0; r0 < R; r0 += rb) {
-      DenseStrides ld;
-      ld.ldx = R;
-      ld.ldw = F;
-      ld.ldo = F;
-      ld.accumulate = r0 > 0;
-      MCCNN_LAYER_SHAPE_SWITCH(rb / kFusedK, fb,
-                               rc = launch_layer(final_product_kernel<CPL, FT>, s, blocks,
-                                                 LayerShape<CPL, FT>::kLdsBytes, num_rows, x + r0,
-                                                 w + (int64_t)r0 * F + f0, out_rows, out + f0, ld));
-      if (rc != MCCNN_OK) return rc;
-      MCCNN_LAUNCH_CHECK();
-    }
+  // one launch, column block f0 = blockIdx.y * fb, every block walking the reduction blocks
+  // in order for its own tiles
+  DenseStrides ld;
+  ld.ldx = R;
+  ld.ldw = F;
+  ld.ldo = F;
+  ld.r_total = R;
+  ld.f_block = fb;
+  const int col_blocks = F / fb;
+  {
+    // one block per compute unit in all (the register-resident weights and the LDS tile
+    // fill it), shared among the column blocks; never more blocks than tiles
+    int device = 0, cus = 0;
+    MCCNN_HIP_CHECK(hipGetDevice(&device));
+    MCCNN_HIP_CHECK(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device));
+    const int64_t tiles = (num_rows + kLayerWaves - 1) / kLayerWaves;
+    int64_t per = cus / col_blocks < 1 ? 1 : cus / col_blocks;
+    if (per > tiles) per = tiles;
+    blocks = (unsigned)per;
+  }
+  MCCNN_LAYER_SHAPE_SWITCH(rb / kFusedK, fb,
+                           rc = launch_layer(final_product_kernel<CPL, FT>, s,
+                                             dim3(blocks, (unsigned)col_blocks),
+                                             LayerShape<CPL, FT>::kLdsBytes, num_rows, x, w,
+                                             out_rows, out, ld));
+  if (rc != MCCNN_OK) return rc;
+  MCCNN_LAUNCH_CHECK();
   return MCCNN_OK;
 }

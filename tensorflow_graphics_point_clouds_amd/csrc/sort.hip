@@ -106,6 +106,108 @@ __global__ void __launch_bounds__(kSortThreads) sort_scatter_kernel(
   }
 }
 
+// The whole sort in one launch for small inputs (a cloud of a few thousand points: the
+// multi-block passes above cost five launches each, 36 us for three passes of 16 k keys,
+// nearly all of it launch latency).  One block of 16 wavefronts runs every pass; wavefront
+// w owns the w-th sixteenth of the input, fetched into registers at the start of the pass.
+// Counting sweep: digit counts per wavefront with LDS atomics (counts do not depend on the
+// order).  Then 256 threads turn the [digit][wavefront] counts into start positions
+// (digits ascending, wavefronts ascending inside a digit).  Ranking sweep, without block
+// barriers: the wavefront walks its keys in rounds of 64 in input order, a lane's rank among
+// the lanes with its digit comes from ballots, the first such lane advances the
+// wavefront's start for the digit.  Same stable order as above.  The passes ping-pong
+// between two global buffers, which one block keeps coherent with its barriers.
+constexpr int kSmallSortThreads = 1024;
+constexpr int kSmallSortWaves = kSmallSortThreads / kWave;
+constexpr int kSmallSortRounds = 16;                 // keys per lane
+constexpr int64_t kSmallSortMax = (int64_t)kSmallSortThreads * kSmallSortRounds;
+
+__global__ void __launch_bounds__(kSmallSortThreads) sort_small_kernel(
+    int n, int passes, const int64_t *__restrict__ keys, int64_t *kbuf0, int *ibuf0,
+    int64_t *kbuf1, int *ibuf1) {
+  __shared__ int start[kSmallSortWaves][kRadix];     // counts, then next free positions
+  __shared__ int scan[kRadix];
+  const int t = threadIdx.x, lane = lane_id(), wave = t / kWave;
+  // the wavefront's chunk: a multiple of 64 keys, so that rounds are whole except the last
+  const int per_wave = ((n + kSmallSortWaves - 1) / kSmallSortWaves + kWave - 1) / kWave * kWave;
+  const int first = wave * per_wave;
+  const int last = first + per_wave < n ? first + per_wave : n;
+  const int64_t *kin = keys;
+  const int *iin = nullptr;
+  for (int p = 0; p < passes; ++p) {
+    const int shift = 8 * p;
+    int64_t *kout = (p & 1) ? kbuf1 : kbuf0;
+    int *iout = (p & 1) ? ibuf1 : ibuf0;
+    int64_t key[kSmallSortRounds];
+    int idx[kSmallSortRounds];
+#pragma unroll
+    for (int r = 0; r < kSmallSortRounds; ++r) {
+      const int i = first + r * kWave + lane;
+      key[r] = i < last ? kin[i] : 0;
+      idx[r] = i < last ? (p == 0 ? i : iin[i]) : 0;
+    }
+    if (t < kRadix) {
+#pragma unroll
+      for (int w = 0; w < kSmallSortWaves; ++w) start[w][t] = 0;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < kSmallSortRounds; ++r)
+      if (first + r * kWave + lane < last) atomicAdd(&start[wave][digit_of(key[r], shift)], 1);
+    __syncthreads();
+    // exclusive scan over (digit, wavefront): per-digit totals scanned over the digits
+    // (Hillis-Steele in LDS, every thread at every barrier), then spread over the wavefronts
+    int total = 0;
+    if (t < kRadix) {
+#pragma unroll
+      for (int w = 0; w < kSmallSortWaves; ++w) total += start[w][t];
+    }
+    int v = total;
+    for (int off = 1; off < kRadix; off <<= 1) {
+      if (t < kRadix) scan[t] = v;
+      __syncthreads();
+      if (t < kRadix && t >= off) v += scan[t - off];
+      __syncthreads();
+    }
+    if (t < kRadix) {
+      int run = v - total;
+#pragma unroll
+      for (int w = 0; w < kSmallSortWaves; ++w) {
+        const int c = start[w][t];
+        start[w][t] = run;
+        run += c;
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < kSmallSortRounds; ++r) {
+      if (first + r * kWave >= last) break;              // uniform in the wavefront
+      const bool live = first + r * kWave + lane < last;
+      const int d = digit_of(key[r], shift);
+      uint64_t same = __ballot(live);
+#pragma unroll
+      for (int bit = 0; bit < 8; ++bit) {
+        const uint64_t b = __ballot((d >> bit) & 1);
+        same &= ((d >> bit) & 1) ? b : ~b;
+      }
+      const int below = __popcll(same & ((1ull << lane) - 1ull));
+      int dst = 0;
+      if (live) dst = start[wave][d] + below;
+      wave_lds_sync();                                   // every lane has read its start
+      if (live && below == 0) start[wave][d] = dst + __popcll(same);
+      wave_lds_sync();
+      if (live) {
+        kout[dst] = key[r];
+        iout[dst] = idx[r];
+      }
+    }
+    __threadfence_block();
+    __syncthreads();               // the pass is in memory before the next one reads it
+    kin = kout;
+    iin = iout;
+  }
+}
+
 // keys[m] = num_pts - 1 - neighbour id (descending key order = ascending id), and
 // the number of pairs of each point.
 __global__ void __launch_bounds__(256) transpose_keys_kernel(int64_t m_total, int64_t num_pts,
@@ -184,6 +286,12 @@ extern "C" int mccnn_sort_keys_descending(mccnn_stream_t stream, int64_t num_pts
   } else {
     kbuf[0] = w.keys_tmp;                 ibuf[0] = w.idx_tmp;
     kbuf[1] = (int64_t *)sorted_keys_out; ibuf[1] = sorted_indices_out;
+  }
+  if (num_pts <= kSmallSortMax) {
+    hipLaunchKernelGGL(sort_small_kernel, dim3(1), dim3(kSmallSortThreads), 0, s, (int)num_pts,
+                       passes, (const int64_t *)keys, kbuf[0], ibuf[0], kbuf[1], ibuf[1]);
+    MCCNN_LAUNCH_CHECK();
+    return MCCNN_OK;
   }
   const int64_t *kin = (const int64_t *)keys;
   const int *iin = nullptr;

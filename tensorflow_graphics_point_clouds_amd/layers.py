@@ -263,7 +263,7 @@ class _MCConvLayer(torch.autograd.Function):
         del dproj
         # feature and final-weight gradients from the transposed convolution
         w2 = dense.reshape(c, k, f).permute(2, 1, 0).reshape(f * k, c)
-        neg = -inv_radii
+        neg = pc._negative(inv_radii)
         if ctx.fuse_final:
             # rows of Q and of dfeat go straight to the points' original positions
             dfeat, q = _mc_layer(weights, biases, dout, view.points_out, view.points_in,
@@ -396,7 +396,7 @@ class MCConv(torch.nn.Module):
                                             (0, g_pad - g, 0, 0, 0, c_pad - c))
             final = final.reshape(l, c_pad * h, g_pad)
             features = torch.nn.functional.pad(features, (0, c_pad - c))
-        inv_radii = torch.reciprocal(radii)
+        inv_radii = pc._reciprocal(radii)
         per = 16 // h if h <= 16 and 16 % h == 0 else 0       # kernel MLPs per 16 basis columns
         if k > 16 and per > 0 and l % per == 0 and (per * g_pad) % 16 == 0:
             # Kernel MLPs do not share final weights (MCConv.py:180-194), so the layer is
@@ -449,11 +449,11 @@ class MCConv(torch.nn.Module):
                                         point_cloud_in._points, point_cloud_out._points,
                                         neighborhood._original_neigh_ids,
                                         neighborhood._samples_neigh_ranges,
-                                        torch.reciprocal(radii), pdf, self._act, transposed)
+                                        pc._reciprocal(radii), pdf, self._act, transposed)
         else:
             basis = _MCBasis.apply(self.weights, biases, point_cloud_in._points,
                                    point_cloud_out._points, neighborhood._original_neigh_ids,
-                                   torch.reciprocal(radii), pdf, self._act)
+                                   pc._reciprocal(radii), pdf, self._act)
             proj = tfg_custom_ops.basis_proj(basis, features.contiguous(),
                                              neighborhood._original_neigh_ids,
                                              neighborhood._samples_neigh_ranges,
@@ -483,7 +483,7 @@ def _differentiable_pdf(neighborhood, bandwidth):
         grid.self_neighborhood(neighborhood._radii)
     per_point = tfg_custom_ops.compute_pdf_with_pt_grads(
         points[grid._sorted_indices.long()], own._neighbors, own._samples_neigh_ranges,
-        torch.reciprocal(pc._as_vector(bandwidth, d, dev)), own._inv_radii,
+        pc._reciprocal(pc._as_vector(bandwidth, d, dev)), own._inv_radii,
         mode.value, symmetric=own._equal_samples and own.max_neighbors == 0)
     pdf = per_point[nb[:, 0].long()]
     if neighborhood._pdf_normalize:              # Neighborhood.py:288-293
@@ -869,7 +869,8 @@ class _KPConvRigidLayer(torch.autograd.Function):
             dout = dout.contiguous()
         # rows of Q (and so of dfeat) go straight to the points' original positions
         q = _kp_project(dout, view.points_out, view.points_in, view.table_t, view.ranges_t,
-                        -inv_radii, kernel_points, k, ctx.kind, ctx.sigma, view.point_rows)
+                        pc._negative(inv_radii), kernel_points, k, ctx.kind, ctx.sigma,
+                        view.point_rows)
         q = q.reshape(feats.shape[0], f * k)
         dfeat = ddense = None
         if ctx.needs_input_grad[1]:
@@ -933,7 +934,7 @@ class _KPConvDeformLayer(torch.autograd.Function):
         dfeat = ddense = doff = None
         if ctx.needs_input_grad[0] or ctx.needs_input_grad[2]:
             q = _kp_deform_project(dout, view.points_out, view.points_in, view.table_t,
-                                   view.ranges_t, -inv_radii, kernel_points, ctx.kind, ctx.sigma,
+                                   view.ranges_t, pc._negative(inv_radii), kernel_points, ctx.kind, ctx.sigma,
                                    offsets, True, view.point_rows)
             q = q.reshape(feats.shape[0], f * k)
             if ctx.needs_input_grad[2]:
@@ -1033,7 +1034,7 @@ class KPConv(torch.nn.Module):
                                          neighborhood, sigma)
         if not self.deformable and self.transposed_grads:
             return _KPConvRigidLayer.apply(self._padded(self.weights), features, neighborhood,
-                                           torch.reciprocal(radii), self._kernel_points, k,
+                                           pc._reciprocal(radii), self._kernel_points, k,
                                            self._kind, sigma, False)
         if self.deformable and self.transposed_grads and k == 16 and d in (2, 3) and \
                 _lib.lib().mccnn_kp_deform_offset_grads_supported(cint(d), cint(c)):
@@ -1043,7 +1044,7 @@ class KPConv(torch.nn.Module):
         if features.requires_grad and tfg_custom_ops.gathered_grads_supported(c, k):
             transposed = neighborhood.transposed_pairs()
         geometry = (point_cloud_in._points, point_cloud_out._points, ids, ranges,
-                    torch.reciprocal(radii), self._kernel_points)
+                    pc._reciprocal(radii), self._kernel_points)
 
         def project(basis):
             return tfg_custom_ops.basis_proj(basis, features, ids, ranges,
@@ -1057,7 +1058,7 @@ class KPConv(torch.nn.Module):
                 cols = kp * d
                 w_off = torch.nn.functional.pad(w_off, (0, -cols % 16))
                 offsets = _KPConvRigidLayer.apply(w_off, features, neighborhood,
-                                                  torch.reciprocal(radii), self._kernel_points, k,
+                                                  pc._reciprocal(radii), self._kernel_points, k,
                                                   self._kind, sigma, False)[:, :cols]
             else:
                 rigid = _KPBasis.apply(None, *geometry, k, self._kind, sigma)
@@ -1075,7 +1076,7 @@ class KPConv(torch.nn.Module):
         regularisation loss."""
         kp, k, d = self._num_kernel_points, self._num_basis, self._num_dims
         view = neighborhood.sorted_view()
-        inv_radii = torch.reciprocal(radii)
+        inv_radii = pc._reciprocal(radii)
         cols = kp * d
         w_off = torch.nn.functional.pad(self._padded(self.offset_weights), (0, -cols % 16))
         offsets = _KPConvRigidLayer.apply(w_off, features, neighborhood, inv_radii,
@@ -1130,7 +1131,7 @@ class KPConv(torch.nn.Module):
         self.last_offsets = offsets
         if self.deformable:
             geometry = (point_cloud_in._points.detach(), point_cloud_out._points.detach(), ids,
-                        ranges, torch.reciprocal(radii), self._kernel_points)
+                        ranges, pc._reciprocal(radii), self._kernel_points)
             self._last = (offsets, geometry, sigma)
         return project(correlation(offsets)) @ self._padded(self.weights)
 

@@ -54,6 +54,32 @@ def _as_vector(value, dims, device):
     return t
 
 
+_derived_cache = {}      # (operation, address of a shared vector) -> shared result
+_shared_vectors = set()  # addresses of the derived vectors themselves
+
+
+def _derived(op, fn, t):
+    """fn(t) for a small device vector; the vectors `_as_vector` keeps (shared,
+    read-only) and what was derived from them get the result once instead of one
+    kernel launch per use."""
+    key = t.data_ptr()
+    if key not in _vector_values and key not in _shared_vectors:
+        return fn(t)
+    r = _derived_cache.get((op, key))
+    if r is None:
+        r = _derived_cache[(op, key)] = fn(t)
+        _shared_vectors.add(r.data_ptr())
+    return r
+
+
+def _reciprocal(t):
+    return _derived("reciprocal", torch.reciprocal, t)
+
+
+def _negative(t):
+    return _derived("negative", torch.neg, t)
+
+
 def _host_values(t):
     """The entries of a small device vector as a tuple of floats; no device round
     trip for the vectors `_as_vector` keeps."""
@@ -406,7 +432,7 @@ class Neighborhood:
             self._equal_samples = False
             self._point_cloud_sampled = point_cloud_sample
         self.max_neighbors = max_neighbors
-        self._inv_radii = torch.reciprocal(self._radii)
+        self._inv_radii = _reciprocal(self._radii)
         s = self._point_cloud_sampled
         self._self_neighborhood = None
         self._table = self._ranges = self._original = None
@@ -536,7 +562,7 @@ class Neighborhood:
         bw = _as_vector(bandwidth, d, dev)
         self._pdf_per_point = tfg_custom_ops.compute_pdf_with_pt_grads(
             self._grid._sorted_points, nbh._neighbors, nbh._samples_neigh_ranges,
-            torch.reciprocal(bw), nbh._inv_radii, mode.value,
+            _reciprocal(bw), nbh._inv_radii, mode.value,
             symmetric=nbh._equal_samples and nbh.max_neighbors == 0)
 
     def point_pdf(self, **kwargs):

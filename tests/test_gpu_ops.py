@@ -79,13 +79,14 @@ def test_keys_sort_table_bit_exact(ops, oracle, d, batch, n, cell):
     assert np.array_equal(grid.get_DS().cpu().numpy(), g.get_ds())
 
 
+@pytest.mark.parametrize("n", [70001, 16384, 16385, 1025, 1, 4097])
 @pytest.mark.parametrize("bits", [1, 7, 8, 9, 20, 33, 63])
-def test_sort_key_widths_and_ties(ops, bits):
-    """Stable descending order for every pass count, with many equal keys."""
+def test_sort_key_widths_and_ties(ops, bits, n):
+    """Stable descending order for every pass count, with many equal keys; sizes on both
+    sides of the single-block path (up to 16384 keys) and at its round boundaries."""
     from tensorflow_graphics_point_clouds_amd import _lib
     from tensorflow_graphics_point_clouds_amd._lib import cint, i64, ptr, stream
-    rng = np.random.default_rng(bits)
-    n = 70001
+    rng = np.random.default_rng(bits + n)
     hi = min(2 ** bits, 2 ** 62)
     keys = rng.integers(0, hi, n, dtype=np.int64)
     keys[::3] = keys[0]
