@@ -613,6 +613,18 @@ int mccnn_final_product(mccnn_stream_t stream, int64_t num_rows, int num_cols_in
                         const float *x, int num_cols_out, const float *w,
                         const int32_t *out_rows, float *out);
 
+/* The same product with the weights handed over transposed, wt [F, R] (the rows of
+ * wt run along the reduction, like the rows of x): the tiled product for weight
+ * matrices beyond a block's registers (the 128 -> 128 layers, R = 2048), 128 x 128
+ * or 256 x 64 output tiles per block of four wavefronts, reduction in steps of 32
+ * through LDS.  Supported: R a multiple of 32, F a multiple of 64.  mccnn_final_product
+ * itself switches to the same tiles (fetching w as it is, about a tenth slower) when
+ * R*F > 65536 and the tiles fill the device. */
+int mccnn_final_product_wt_supported(int num_cols_in, int num_cols_out);
+int mccnn_final_product_wt(mccnn_stream_t stream, int64_t num_rows, int num_cols_in,
+                           const float *x, int num_cols_out, const float *wt,
+                           const int32_t *out_rows, float *out);
+
 /* out[c, r] = sum_n x[n, c] * y[n, r]: the gradient of a layer's final weights
  * (the backward of the tf.matmul of MCConv.py:187 / KPConv.py:226-230), a product
  * with a reduction over all points and a small [C, R] output.  y is read from

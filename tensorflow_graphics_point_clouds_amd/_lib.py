@@ -151,9 +151,9 @@ def collect_timing():
     return out
 
 
-def call(name, *args):
+def call(name, *args, timed_as=None):
     """Invoke entry point mccnn_<name>, raise on a non-zero status, and time it
-    when timing is active."""
+    when timing is active (under `timed_as` if given)."""
     fn = getattr(lib(), "mccnn_" + name)
-    with region(name):
+    with region(timed_as or name):
         check(fn(*args))

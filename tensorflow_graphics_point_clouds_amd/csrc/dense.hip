@@ -173,77 +173,92 @@ static bool nt_supported(int F, int R) {
 
 // out[out_rows[n] or n, :] = x[n, :] * w for x [N, R], w [R, F] when w is too large to sit in
 // the registers of one block (R * F > 65536: the 128 -> 128 kernel-point layers, R = 2048):
-// the classic tiled product.  A block of four wavefronts owns a 128 x BN tile of the output
-// (wavefront (wm, wn): 64 x BN/2, i.e. 4 x BN/32 accumulator tiles) and walks the reduction
-// in steps of 32: the 128 x 32 block of x and the 32 x BN block of w of the next step are
-// fetched into registers while the current one is multiplied out of LDS (x rows as they
-// are, w transposed, rows 36 floats apart), two barriers per step.  The reduction index of a
-// matrix step may be permuted as long as both operands agree: lane quarter q takes indices
-// 4q .. 4q+3 of each group of 16, so every operand fetch is one 16-byte LDS read.
-// x is read once per column block (F / BN times); w comes from L2.  The lanes of a
-// wavefront fetch their pieces of w with the reduction index running fastest (32 rows of
-// w, 16 bytes of each), so that the four transposing LDS writes of a lane land in 32
-// consecutive banks; with the columns running fastest the fetch is coalesced but the
-// writes hit two banks 16 ways (0.9 G conflict cycles per launch, 104 instead of 113
-// TFLOP/s on [825 274, 2048] x [2048, 128]).  A second LDS buffer (one barrier per step)
-// costs a resident block per compute unit and is slower (107 TFLOP/s).
-constexpr int kTileRows = 128, kTileK = 32, kTileLd = kTileK + 4;
+// the classic tiled product.  A block of four wavefronts owns a BM x BN tile of the output,
+// 128 x 128 or 256 x 64, every wavefront 64 x 64 of it as 4 x 4 accumulator tiles, and walks
+// the reduction in steps of 32: the BM x 32 block of x and the 32 x BN block of w of the next
+// step are fetched into registers while the current one is multiplied out of LDS (both with
+// the reduction index running along a row, rows 36 floats apart), two barriers per step.
+// The reduction index of a matrix step may be permuted as long as both operands agree: lane
+// quarter q takes indices 4q .. 4q+3 of each group of 16, so every operand fetch is one
+// 16-byte LDS read.  x is read once per column block (F / BN times); w comes from L2.
+// w is taken as it is ([R, F]) or transposed (wt [F, R], kWT): transposed, its rows are
+// fetched and parked exactly like those of x (129 TFLOP/s on [825 274, 2048] x [2048, 128]).
+// As it is, the lanes of a wavefront fetch their pieces with the reduction index running
+// fastest (32 rows of w, 16 bytes of each), so that the four transposing LDS writes of a
+// lane land in 32 consecutive banks: 113 TFLOP/s; with the columns running fastest the
+// fetch is coalesced but the writes hit two banks 16 ways (0.9 G conflict cycles per
+// launch, 104 TFLOP/s).  A second LDS buffer (one barrier per step) costs a resident block
+// per compute unit and is slower (107 TFLOP/s); fetching the operands of the next half
+// group ahead of the matrix steps changes nothing.
+constexpr int kTileK = 32, kTileLd = kTileK + 4, kTileThreads = 256;
 
-template <int BN>
-__global__ void __launch_bounds__(256) tile_product_kernel(int64_t n, int R, int F,
-                                                           const float *__restrict__ x,
-                                                           const float *__restrict__ w,
-                                                           const int *__restrict__ out_rows,
-                                                           float *__restrict__ out) {
-  constexpr int kCT = BN / 32;                    // accumulator tiles per wavefront along the columns
-  constexpr int kBLoads = kTileK * BN / 4 / 256;  // float4 loads of w per thread and step
-  __shared__ __align__(16) float a_lds[kTileRows * kTileLd];
+template <int BN, bool kWT>
+__global__ void __launch_bounds__(kTileThreads) tile_product_kernel(
+    int64_t n, int R, int F, const float *__restrict__ x, const float *__restrict__ w,
+    const int *__restrict__ out_rows, float *__restrict__ out) {
+  constexpr int BM = 16384 / BN;                  // 4 wavefronts x (64 x 64)
+  constexpr int kWN = BN / 64;                    // wavefronts side by side
+  constexpr int kALoads = BM * kTileK / 4 / kTileThreads;   // 16-byte loads per thread and step
+  constexpr int kBLoads = BN * kTileK / 4 / kTileThreads;
+  __shared__ __align__(16) float a_lds[BM * kTileLd];
   __shared__ __align__(16) float b_lds[BN * kTileLd];
   const int t = threadIdx.x, lane = lane_id(), wave = t / kWave;
   const int q = lane >> 4, c16 = lane & 15;
-  const int wm = wave >> 1, wn = wave & 1;
+  const int wm = wave / kWN, wn = wave % kWN;
   const int col_blocks = F / BN;
-  const int64_t row0 = (int64_t)(blockIdx.x / col_blocks) * kTileRows;
+  const int64_t row0 = (int64_t)(blockIdx.x / col_blocks) * BM;
   const int col0 = (blockIdx.x % col_blocks) * BN;
 
-  v4f acc[4][kCT];
+  v4f acc[4][4];
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
-    for (int j = 0; j < kCT; ++j) acc[i][j] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+    for (int j = 0; j < 4; ++j) acc[i][j] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
 
-  // this thread's pieces of a step: 4 x (row, 4 k) of x, kBLoads x (k, 4 columns) of w
-  v4f xa[4], wb[kBLoads];
+  // this thread's pieces of a step: (row, 4 k) of x and of w^T, or (k, 4 columns) of w
+  v4f xa[kALoads], wb[kBLoads];
   auto fetch = [&](int k0) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int idx = t + 256 * i, row = idx >> 3, c4 = idx & 7;
-      xa[i] = row0 + row < n
-                  ? *reinterpret_cast<const v4f *>(x + (row0 + row) * R + k0 + 4 * c4)
-                  : v4f{0.0f, 0.0f, 0.0f, 0.0f};
+    for (int i = 0; i < kALoads; ++i) {
+      const int idx = t + kTileThreads * i, row = idx >> 3, c4 = idx & 7;
+      // rows past the end repeat the last row (their results are never stored): no branch
+      const int64_t r = row0 + row < n ? row0 + row : n - 1;
+      xa[i] = *reinterpret_cast<const v4f *>(x + r * R + k0 + 4 * c4);
     }
 #pragma unroll
     for (int i = 0; i < kBLoads; ++i) {
-      const int idx = t + 256 * i, kk = idx % kTileK, c4 = idx / kTileK;
-      wb[i] = *reinterpret_cast<const v4f *>(w + (int64_t)(k0 + kk) * F + col0 + 4 * c4);
+      const int idx = t + kTileThreads * i;
+      if constexpr (kWT) {
+        const int col = idx >> 3, c4 = idx & 7;
+        wb[i] = *reinterpret_cast<const v4f *>(w + (int64_t)(col0 + col) * R + k0 + 4 * c4);
+      } else {
+        const int kk = idx % kTileK, c4 = idx / kTileK;
+        wb[i] = *reinterpret_cast<const v4f *>(w + (int64_t)(k0 + kk) * F + col0 + 4 * c4);
+      }
     }
   };
   auto park = [&]() {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int idx = t + 256 * i, row = idx >> 3, c4 = idx & 7;
+    for (int i = 0; i < kALoads; ++i) {
+      const int idx = t + kTileThreads * i, row = idx >> 3, c4 = idx & 7;
       *reinterpret_cast<v4f *>(a_lds + row * kTileLd + 4 * c4) = xa[i];
     }
 #pragma unroll
     for (int i = 0; i < kBLoads; ++i) {
-      const int idx = t + 256 * i, kk = idx % kTileK, c4 = idx / kTileK;
+      const int idx = t + kTileThreads * i;
+      if constexpr (kWT) {
+        const int col = idx >> 3, c4 = idx & 7;
+        *reinterpret_cast<v4f *>(b_lds + col * kTileLd + 4 * c4) = wb[i];
+      } else {
+        const int kk = idx % kTileK, c4 = idx / kTileK;
 #pragma unroll
-      for (int j = 0; j < 4; ++j) b_lds[(4 * c4 + j) * kTileLd + kk] = wb[i][j];
+        for (int j = 0; j < 4; ++j) b_lds[(4 * c4 + j) * kTileLd + kk] = wb[i][j];
+      }
     }
   };
 
   const float *a_rd = a_lds + (wm * 64 + c16) * kTileLd + 4 * q;
-  const float *b_rd = b_lds + (wn * (BN / 2) + c16) * kTileLd + 4 * q;
+  const float *b_rd = b_lds + (wn * 64 + c16) * kTileLd + 4 * q;
   fetch(0);
   for (int k0 = 0; k0 < R; k0 += kTileK) {
     __syncthreads();                  // the previous step has been multiplied
@@ -252,23 +267,23 @@ __global__ void __launch_bounds__(256) tile_product_kernel(int64_t n, int R, int
     if (k0 + kTileK < R) fetch(k0 + kTileK);
 #pragma unroll
     for (int ks = 0; ks < kTileK / 16; ++ks) {
-      v4f a[4], b[kCT];
+      v4f a[4], b[4];
 #pragma unroll
       for (int i = 0; i < 4; ++i)
         a[i] = *reinterpret_cast<const v4f *>(a_rd + 16 * i * kTileLd + 16 * ks);
 #pragma unroll
-      for (int j = 0; j < kCT; ++j)
+      for (int j = 0; j < 4; ++j)
         b[j] = *reinterpret_cast<const v4f *>(b_rd + 16 * j * kTileLd + 16 * ks);
 #pragma unroll
       for (int s = 0; s < 4; ++s)
 #pragma unroll
         for (int i = 0; i < 4; ++i)
 #pragma unroll
-          for (int j = 0; j < kCT; ++j)
+          for (int j = 0; j < 4; ++j)
             acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[i][s], b[j][s], acc[i][j], 0, 0, 0);
     }
   }
-  // acc[i][j][r]: row row0 + 64 wm + 16 i + 4 q + r, column col0 + (BN/2) wn + 16 j + c16
+  // acc[i][j][r]: row row0 + 64 wm + 16 i + 4 q + r, column col0 + 64 wn + 16 j + c16
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
@@ -276,24 +291,33 @@ __global__ void __launch_bounds__(256) tile_product_kernel(int64_t n, int R, int
       const int64_t row = row0 + wm * 64 + 16 * i + 4 * q + r;
       if (row < n) {
         const int64_t orow = out_rows ? out_rows[row] : row;
-        float *o = out + orow * F + col0 + wn * (BN / 2) + c16;
+        float *o = out + orow * F + col0 + wn * 64 + c16;
 #pragma unroll
-        for (int j = 0; j < kCT; ++j) o[16 * j] = acc[i][j][r];
+        for (int j = 0; j < 4; ++j) o[16 * j] = acc[i][j][r];
       }
     }
 }
 
 bool tile_product_supported(int R, int F) { return R >= 32 && R % 32 == 0 && F >= 64 && F % 64 == 0; }
 
+// Output rows per block of the tiled product for F columns.
+int tile_product_rows(int F) { return F % 128 == 0 ? 128 : 256; }
+
 int launch_tile_product(hipStream_t s, int64_t n, int R, const float *x, int F, const float *w,
-                        const int *out_rows, float *out) {
-  const int64_t row_blocks = (n + kTileRows - 1) / kTileRows;
-  if (F % 128 == 0)
-    hipLaunchKernelGGL(tile_product_kernel<128>, dim3((unsigned)(row_blocks * (F / 128))),
-                       dim3(256), 0, s, n, R, F, x, w, out_rows, out);
-  else
-    hipLaunchKernelGGL(tile_product_kernel<64>, dim3((unsigned)(row_blocks * (F / 64))), dim3(256),
-                       0, s, n, R, F, x, w, out_rows, out);
+                        bool w_transposed, const int *out_rows, float *out) {
+  const int bn = F % 128 == 0 ? 128 : 64, bm = tile_product_rows(F);
+  const dim3 block(kTileThreads), grid((unsigned)((n + bm - 1) / bm * (F / bn)));
+  if (bn == 128) {
+    if (w_transposed)
+      hipLaunchKernelGGL((tile_product_kernel<128, true>), grid, block, 0, s, n, R, F, x, w, out_rows, out);
+    else
+      hipLaunchKernelGGL((tile_product_kernel<128, false>), grid, block, 0, s, n, R, F, x, w, out_rows, out);
+  } else {
+    if (w_transposed)
+      hipLaunchKernelGGL((tile_product_kernel<64, true>), grid, block, 0, s, n, R, F, x, w, out_rows, out);
+    else
+      hipLaunchKernelGGL((tile_product_kernel<64, false>), grid, block, 0, s, n, R, F, x, w, out_rows, out);
+  }
   MCCNN_LAUNCH_CHECK();
   return MCCNN_OK;
 }

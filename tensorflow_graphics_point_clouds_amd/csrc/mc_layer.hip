@@ -440,13 +440,14 @@ extern "C" int mccnn_final_product(mccnn_stream_t stream, int64_t num_rows, int 
   int rc = layer_grid(num_rows, &blocks);
   if (rc != MCCNN_OK) return rc;
   const int R = num_cols_in, F = num_cols_out;
-  // weights beyond a block's registers: the tiled product, once its 128-row tiles give
+  // weights beyond a block's registers: the tiled product, once its 128- or 256-row tiles give
   // every compute unit a block (below that a launch is a few blocks walking the whole
   // reduction alone: 170 us for 400 rows x 4096 x 256 against 20 us for the blocked
   // register-resident product, whose tiles are 16 rows)
   if ((int64_t)R * F > 65536 && tile_product_supported(R, F) &&
-      (num_rows + 127) / 128 * (F / (F % 128 == 0 ? 128 : 64)) >= (int64_t)blocks)
-    return launch_tile_product(s, num_rows, R, x, F, w, out_rows, out);
+      (num_rows + tile_product_rows(F) - 1) / tile_product_rows(F) *
+              (F / (F % 128 == 0 ? 128 : 64)) >= (int64_t)blocks)
+    return launch_tile_product(s, num_rows, R, x, F, w, false, out_rows, out);
   int rb = 0, fb = 0;
   product_blocks(R, F, &rb, &fb);
   // out[:, f0:f0+fb] = sum over the reduction blocks r0 of x[:, r0:r0+rb] W[r0:r0+rb, f0:f0+fb]:
@@ -478,4 +479,25 @@ extern "C" int mccnn_final_product(mccnn_stream_t stream, int64_t num_rows, int 
   if (rc != MCCNN_OK) return rc;
   MCCNN_LAUNCH_CHECK();
   return MCCNN_OK;
+}
+
+// The same product with the weights given transposed, wt [F, R] (rows of w^T are
+// contiguous along the reduction, like the rows of x): the layout the tiled product
+// fetches without a transposing pass through LDS.
+extern "C" int mccnn_final_product_wt_supported(int num_cols_in, int num_cols_out) {
+  return tile_product_supported(num_cols_in, num_cols_out) ? 1 : 0;
+}
+
+extern "C" int mccnn_final_product_wt(mccnn_stream_t stream, int64_t num_rows, int num_cols_in,
+                                      const float *x, int num_cols_out, const float *wt,
+                                      const int32_t *out_rows, float *out) {
+  MCCNN_REQUIRE(tile_product_supported(num_cols_in, num_cols_out),
+                "final_product_wt supports a multiple of 32 input columns and a multiple of 64 "
+                "output columns (got %d x %d)", num_cols_in, num_cols_out);
+  MCCNN_REQUIRE(num_rows >= 0 && num_rows < ((int64_t)1 << 31),
+                "final_product_wt expects a size in [0, 2^31)");
+  if (num_rows == 0) return MCCNN_OK;
+  MCCNN_REQUIRE(x && wt && out, "final_product_wt received a null tensor");
+  return launch_tile_product(as_stream(stream), num_rows, num_cols_in, x, num_cols_out, wt, true,
+                             out_rows, out);
 }

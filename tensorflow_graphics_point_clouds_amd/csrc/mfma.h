@@ -54,8 +54,9 @@ int launch_dfeat_gather(hipStream_t s, int64_t num_pts, int C, const int *point_
 // out = x * w for x [N, R], w [R, F] as a tiled product (defined in dense.hip): for weight
 // matrices too large for the register-resident product of mc_layer.hip.
 bool tile_product_supported(int R, int F);
+int tile_product_rows(int F);
 int launch_tile_product(hipStream_t s, int64_t n, int R, const float *x, int F, const float *w,
-                        const int *out_rows, float *out);
+                        bool w_transposed, const int *out_rows, float *out);
 
 typedef float v16f __attribute__((ext_vector_type(16)));
 typedef float v4f __attribute__((ext_vector_type(4)));

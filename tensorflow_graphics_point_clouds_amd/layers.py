@@ -172,16 +172,44 @@ def _projection_grad_product(x, w):
     return out
 
 
+_cu_count = {}
+
+
+def _compute_units(device):
+    idx = device.index if device.index is not None else torch.cuda.current_device()
+    if idx not in _cu_count:
+        _cu_count[idx] = torch.cuda.get_device_properties(idx).multi_processor_count
+    return _cu_count[idx]
+
+
+def _tiles(n, f):
+    """Blocks of the tiled product: 128 x 128 tiles, 256 x 64 for odd multiples of 64."""
+    return (n + 127) // 128 * (f // 128) if f % 128 == 0 else (n + 255) // 256 * (f // 64)
+
+
 def _final_product(x, w):
     """x w for x [N, R] and the final weights w [R, F]."""
     r, f = w.shape
-    if not _lib.lib().mccnn_final_product_supported(cint(r), cint(f)):
+    L = _lib.lib()
+    out = torch.empty((x.shape[0], f), dtype=_F32, device=x.device)
+    # Weights beyond the registers of a block of wavefronts (R * F > 65536) take the tiled
+    # product, which reads both operands along the reduction: w is handed over transposed
+    # (a copy of at most a few MB).  Only when its 128-row tiles give every compute unit
+    # one; smaller inputs take the register-resident product in blocks of w.
+    if r * f > _TILED_ABOVE and L.mccnn_final_product_wt_supported(cint(r), cint(f)) and \
+            _tiles(x.shape[0], f) >= _compute_units(x.device):
+        _lib.call("final_product_wt", stream(), i64(x.shape[0]), cint(r), ptr(x, _F32), cint(f),
+                  ptr(w.t().contiguous(), _F32), ptr(None), ptr(out), timed_as="final_product")
+        return out
+    if not L.mccnn_final_product_supported(cint(r), cint(f)):
         with _lib.region("gemm_final"):
             return x @ w
-    out = torch.empty((x.shape[0], f), dtype=_F32, device=x.device)
     _lib.call("final_product", stream(), i64(x.shape[0]), cint(r), ptr(x, _F32), cint(f),
               ptr(w.contiguous(), _F32), ptr(None), ptr(out))
     return out
+
+
+_TILED_ABOVE = 65536      # weights that fit the registers of a block of wavefronts
 
 
 def _dense_final_weights(final_weights, c):

@@ -457,6 +457,38 @@ def test_final_product_matches_float64(n, r, f):
                   ptr(None), ptr(outs[0]))
 
 
+@pytest.mark.parametrize("n,r,f", [(40001, 2048, 128), (70000, 1024, 64), (33000, 512, 192),
+                                   (129, 64, 64), (1, 32, 128), (0, 2048, 128)])
+def test_final_product_with_transposed_weights_matches_float64(n, r, f):
+    """The tiled product on wt [F, R] (128 x 128 and 256 x 64 tiles, partial last tiles, row
+    permutation), elementwise against float64 with the magnitude sum |x| |w| (1e-5); equal
+    bits on a second call; and the layer-level product, which picks the tiles for the large
+    shapes, against the same reference."""
+    from tensorflow_graphics_point_clouds_amd import _lib, layers
+    from tensorflow_graphics_point_clouds_amd._lib import cint, i64, ptr, stream
+    assert _lib.lib().mccnn_final_product_wt_supported(r, f) == 1
+    assert _lib.lib().mccnn_final_product_wt_supported(r, 48) == 0
+    gen = torch.Generator(device="cuda").manual_seed(n + f)
+    x = torch.randn((n, r), device="cuda", generator=gen)
+    w = torch.randn((r, f), device="cuda", generator=gen)
+    wt = w.t().contiguous()
+    rows = torch.randperm(n, device="cuda", generator=gen).int()
+    outs = []
+    for perm in (None, rows, rows):
+        out = torch.full((n, f), float("nan"), device="cuda")
+        _lib.call("final_product_wt", stream(), i64(n), cint(r), ptr(x), cint(f), ptr(wt),
+                  ptr(perm), ptr(out))
+        outs.append(out)
+    expect = x.double() @ w.double()
+    mag = x.double().abs() @ w.double().abs()
+    assert bool(((outs[0].double() - expect).abs() <= 1e-5 * mag).all())
+    assert torch.equal(outs[1], outs[2])
+    if n:
+        assert torch.equal(outs[1][rows.long()], outs[0])
+    got = layers._final_product(x, w)
+    assert bool(((got.double() - expect).abs() <= 1e-5 * mag).all())
+
+
 def test_layers_accept_padded_input_and_return_padded_output():
     """Padded point clouds / features ([A, V, D], [A, V, C], sizes) give the same
     result as the segmented form, re-padded on request (layers/utils.py:22-49,
