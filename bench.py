@@ -585,7 +585,7 @@ def per_op_times(torch, pc, layers, synthetic, _lib, radius=0.04, reps=5):
     return out
 
 
-def isolated_basis_proj(torch, pc, synthetic, tfg, _lib, radius=0.04, steps=5):
+def isolated_basis_proj(torch, pc, synthetic, tfg, _lib, radius=0.04, steps=5, gathered=False):
     """basis_proj forward and gradients alone on 4 x 200k uniform points,
     C=128, K=32 (the dense-neighbourhood case)."""
     import numpy as np
@@ -630,7 +630,7 @@ def isolated_basis_proj(torch, pc, synthetic, tfg, _lib, radius=0.04, steps=5):
         # the atomic-free variant: per-pair rows of the feature gradient written to a
         # [M, C] workspace and summed per point over the transposed pair lists (built once
         # per neighbourhood, timed separately)
-        if tfg.gathered_grads_supported(C, K):
+        if gathered and tfg.gathered_grads_supported(C, K):
             tr = tfg.transpose_neighbors(ids, N)
             tfg.basis_proj_grads(basis, feat, ids, ranges, up, None, transposed=tr)
             _lib.start_timing()
@@ -810,8 +810,10 @@ def main():
     if not args.no_isolated and args.scale == 1.0:
         del feats, up
         torch.cuda.empty_cache()
+        # (the atomic-free gradient variant is timed with --extra-configs only: it launches
+        # the same gradient kernel in another mode and would blur its average in a profile)
         result["basis_proj_isolated"] = isolated_basis_proj(torch, pc, synthetic, tfg_custom_ops,
-                                                            _lib)
+                                                            _lib, gathered=args.extra_configs)
         torch.cuda.empty_cache()
         # the other two radii of the dense case's sweep (about 7 and 180 pairs per point)
         result["dense_radius_sweep"] = {}
