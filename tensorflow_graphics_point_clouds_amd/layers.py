@@ -187,6 +187,14 @@ def _tiles(n, f):
     return (n + 127) // 128 * (f // 128) if f % 128 == 0 else (n + 255) // 256 * (f // 64)
 
 
+def _padded_columns(cols):
+    """Output columns of a layer whose count the kernels do not cover, with zero columns
+    added: a multiple of 16, and of 64 beyond 32 (the tiled product and the 64-channel
+    kernels of the backward take 64 columns in less time than the blocked product takes 48:
+    [825 274, 2048] x [2048, 48] 3.4 ms, x [2048, 64] 1.9 ms)."""
+    return -(-cols // 64) * 64 if cols > 32 else -(-cols // 16) * 16
+
+
 def _final_product(x, w):
     """x w for x [N, R] and the final weights w [R, F]."""
     r, f = w.shape
@@ -1082,9 +1090,9 @@ class KPConv(torch.nn.Module):
         if self.deformable:       # KPConv.py:317-392: offsets from a rigid convolution
             w_off = self._padded(self.offset_weights)
             if self.transposed_grads and k in (16, 32):
-                # the rigid layer's kernels, output columns padded to a multiple of 16
+                # the rigid layer's kernels, output columns padded (45 -> 64)
                 cols = kp * d
-                w_off = torch.nn.functional.pad(w_off, (0, -cols % 16))
+                w_off = torch.nn.functional.pad(w_off, (0, _padded_columns(cols) - cols))
                 offsets = _KPConvRigidLayer.apply(w_off, features, neighborhood,
                                                   pc._reciprocal(radii), self._kernel_points, k,
                                                   self._kind, sigma, False)[:, :cols]
@@ -1106,7 +1114,8 @@ class KPConv(torch.nn.Module):
         view = neighborhood.sorted_view()
         inv_radii = pc._reciprocal(radii)
         cols = kp * d
-        w_off = torch.nn.functional.pad(self._padded(self.offset_weights), (0, -cols % 16))
+        w_off = torch.nn.functional.pad(self._padded(self.offset_weights),
+                                        (0, _padded_columns(cols) - cols))
         offsets = _KPConvRigidLayer.apply(w_off, features, neighborhood, inv_radii,
                                           self._kernel_points, k, self._kind, sigma,
                                           False)[:, :cols]
