@@ -425,10 +425,12 @@ def test_projection_grad_product_matches_float64(n, f, r):
 @pytest.mark.parametrize("n,r,f", [(1, 256, 16), (15, 256, 128), (4099, 1024, 64), (20000, 512, 128),
                                    (333, 1024, 32), (5000, 512, 32), (0, 1024, 64), (70001, 1024, 16),
                                    (4099, 2048, 128), (3001, 1024, 128), (1500, 4096, 256),
-                                   (777, 2048, 48), (2000, 768, 192), (9000, 2048, 64)])
+                                   (777, 2048, 48), (2000, 768, 192), (9000, 2048, 64),
+                                   (33000, 1024, 128), (66100, 2048, 64)])
 def test_final_product_matches_float64(n, r, f):
-    """x w with a block of w in the registers of each block of wavefronts (one launch per
-    block of w for the larger shapes, later row blocks adding to the earlier ones),
+    """x w with a block of w in the registers of each block of wavefronts (the blocks of a
+    larger w walked inside one launch, later row blocks adding to the earlier ones; the last
+    two shapes are large enough for the tiled product on w as it is),
     elementwise against float64 with the magnitude sum |x| |w| (1e-5), row permutation
     included; a second call must return the same bits."""
     from tensorflow_graphics_point_clouds_amd import _lib
