@@ -178,7 +178,10 @@ int mccnn_compute_pdf(mccnn_stream_t stream, int64_t num_pts, int num_dims,
                       const float *inv_radii, int mode, float *pdf_out);
 
 /* ComputePdfPtGrads: compute_pdf/cc/ops/compute_pdf_ops.cpp:163-259.
- * pt_grads_out [num_pts, D] = d(sum_i pdf_grads_i * pdf_i) / d(points). */
+ * pt_grads_out [num_pts, D] = d(sum_i pdf_grads_i * pdf_i) / d(points).  Valid for any
+ * pair table; where the reverse of a pair is in the table too (always, in an
+ * untruncated self-neighbourhood) its term is gathered instead of scattered, so
+ * atomics are used only for pairs without a reverse. */
 int mccnn_compute_pdf_pt_grads(mccnn_stream_t stream, int64_t num_pts,
                                int num_dims, const float *points,
                                int64_t num_neighbors, int neighbors_rank,

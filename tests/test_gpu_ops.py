@@ -210,6 +210,35 @@ def test_pdf_and_point_grads(ops, oracle, d, mode):
     assert_normwise(sym.cpu().numpy(), gexp)
 
 
+@pytest.mark.parametrize("variant", ["truncated", "shuffled", "truncated+shuffled"])
+def test_pdf_point_grads_on_asymmetric_and_unordered_tables(ops, oracle, variant):
+    """compute_pdf_pt_grads looks the reverse of every pair up in the neighbour's list: lists
+    cut by max_neighbors (reverse pairs missing: their terms are scattered) and lists in
+    another order than find_neighbors writes (the binary search misses and the linear scan
+    decides) must give the oracle's gradient (normwise 1e-5)."""
+    rng = np.random.default_rng(77)
+    pts, bids = _cloud(rng, 2, 3000, 3)
+    g = oracle.Grid(pts, bids, 2, 0.15)
+    nbh = oracle.Neighborhood(g, 0.15, max_neighbors=6 if "truncated" in variant else 0)
+    pairs, ranges = nbh.neighbors.copy(), nbh.ranges
+    if "shuffled" in variant:              # every centre's list in random order
+        start = 0
+        for end in ranges:
+            pairs[start:end] = pairs[start:end][rng.permutation(end - start)]
+            start = end
+    if "truncated" in variant:             # the table really is asymmetric
+        have = set(map(tuple, pairs.tolist()))
+        assert any((c, j) not in have for j, c in have)
+    inv_bw = np.full(3, 1 / np.float32(0.2), np.float32)
+    up = rng.standard_normal(len(pts)).astype(np.float32)
+    for mode in (0, 1):
+        gexp = oracle.compute_pdf_pt_grads(g.sorted_points, pairs, ranges, inv_bw, nbh.inv_radii,
+                                           up, mode)
+        got = ops.compute_pdf_pt_grads(dev(g.sorted_points), dev(pairs), dev(ranges), dev(inv_bw),
+                                       dev(nbh.inv_radii), dev(up), mode)
+        assert_normwise(got.cpu().numpy(), gexp)
+
+
 # ------------------------------------------------------------- basis_proj ----
 
 @pytest.mark.parametrize("c,k", [(1, 8), (3, 16), (5, 32), (8, 8), (16, 16), (32, 32),
