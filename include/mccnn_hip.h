@@ -100,6 +100,9 @@ int mccnn_grid_setup(mccnn_stream_t stream, int64_t num_pts, int num_dims,
  *                 pylib/pc/Neighborhood.py:246-250
  *   pdf per pair  out[m] = pdf[neighbors[m,0]]   pylib/pc/Neighborhood.py:287
  *                 (_column: of either column, for the transposed pair table)
+ *   swapped pairs out[i] = (neighbors[order[i],1], neighbors[order[i],0]): the rows of
+ *                 the transposed pair table from the order mccnn_transpose_neighbors
+ *                 returns (no counterpart: the reference searches again, Neighborhood.py:318-329)
  *   int32 gather  out[i] = src[indices[i]]       pylib/pc/sampling.py:142-146
  *   row gather    out[i,:] = src[indices[i],:]   (tf.gather of feature rows, e.g.
  *                 pylib/pc/layers/utils.py:47; num_cols a multiple of 4, rows 16-byte aligned) */
@@ -110,6 +113,9 @@ int mccnn_original_neighbor_ids(mccnn_stream_t stream, int64_t num_neighbors,
 int mccnn_gather_pdf(mccnn_stream_t stream, int64_t num_neighbors,
                      const int32_t *neighbors, const float *pdf,
                      float *pdf_per_pair_out);
+int mccnn_swapped_pairs(mccnn_stream_t stream, int64_t num_neighbors,
+                        const int32_t *neighbors, const int32_t *pair_order,
+                        int32_t *swapped_out);
 int mccnn_gather_pdf_column(mccnn_stream_t stream, int64_t num_neighbors,
                             const int32_t *neighbors, int column, const float *pdf,
                             float *pdf_per_pair_out);

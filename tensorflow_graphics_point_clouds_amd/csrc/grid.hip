@@ -62,6 +62,18 @@ __global__ void __launch_bounds__(256) original_ids_kernel(int64_t m,
   }
 }
 
+// Rows of the transposed pair table: out[i] = (centre, point) of pair order[i].
+__global__ void __launch_bounds__(256) swapped_pairs_kernel(int64_t m,
+                                                            const int2 *__restrict__ nbrs,
+                                                            const int *__restrict__ order,
+                                                            int2 *__restrict__ out) {
+  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < m;
+       i += (int64_t)gridDim.x * blockDim.x) {
+    const int2 p = nbrs[order[i]];
+    out[i] = make_int2(p.y, p.x);
+  }
+}
+
 __global__ void __launch_bounds__(256) gather_pdf_kernel(int64_t m, const int2 *__restrict__ nbrs,
                                                          int column, const float *__restrict__ pdf,
                                                          float *__restrict__ out) {
@@ -367,6 +379,19 @@ extern "C" int mccnn_original_neighbor_ids(mccnn_stream_t stream, int64_t num_ne
   hipLaunchKernelGGL(original_ids_kernel, dim3(capped_grid(num_neighbors)), dim3(256), 0,
                      as_stream(stream), num_neighbors, (const int2 *)neighbors, sorted_indices,
                      (int2 *)original_neighbors_out);
+  MCCNN_LAUNCH_CHECK();
+  return MCCNN_OK;
+}
+
+extern "C" int mccnn_swapped_pairs(mccnn_stream_t stream, int64_t num_neighbors,
+                                   const int32_t *neighbors, const int32_t *pair_order,
+                                   int32_t *swapped_out) {
+  MCCNN_REQUIRE(num_neighbors >= 0, "swapped_pairs expects a non-negative size");
+  if (num_neighbors == 0) return MCCNN_OK;
+  MCCNN_REQUIRE(neighbors && pair_order && swapped_out, "swapped_pairs received a null tensor");
+  hipLaunchKernelGGL(swapped_pairs_kernel, dim3(capped_grid(num_neighbors)), dim3(256), 0,
+                     as_stream(stream), num_neighbors, (const int2 *)neighbors, pair_order,
+                     (int2 *)swapped_out);
   MCCNN_LAUNCH_CHECK();
   return MCCNN_OK;
 }

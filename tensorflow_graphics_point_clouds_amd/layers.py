@@ -278,7 +278,7 @@ class _MCConvLayer(torch.autograd.Function):
         k, n, c = l * h, view.ranges.shape[0], feats.shape[1]
         g = final_weights.shape[2]
         f = g * l
-        if view.centre_order is not None:
+        if view.centre_rows is not None:
             dout = _gather_rows(dout, view.centre_rows)
         else:
             dout = dout.contiguous()
@@ -607,7 +607,7 @@ class _PointConvLayer(torch.autograd.Function):
         n, c, m = view.ranges.shape[0], feats.shape[1], view.table.shape[0]
         dense = final_weights[0]                                      # [C*K, F]
         f = dense.shape[1]
-        if view.centre_order is not None:
+        if view.centre_rows is not None:
             dout = _gather_rows(dout, view.centre_rows)
         else:
             dout = dout.contiguous()
@@ -899,7 +899,7 @@ class _KPConvRigidLayer(torch.autograd.Function):
         dense, feats, features, inv_radii, kernel_points = ctx.saved_tensors
         view = ctx.neighborhood.sorted_view()
         k, c, f = ctx.k, feats.shape[1], dense.shape[1]
-        if view.centre_order is not None and not ctx.rows_in_view_order:
+        if view.centre_rows is not None and not ctx.rows_in_view_order:
             dout = _gather_rows(dout, view.centre_rows)
         else:
             dout = dout.contiguous()
@@ -963,7 +963,7 @@ class _KPConvDeformLayer(torch.autograd.Function):
         kp, dims = kernel_points.shape
         k, c, f = 16, feats.shape[1], dense.shape[1]
         n_out = view.ranges.shape[0]
-        if view.centre_order is not None:
+        if view.centre_rows is not None:
             dout = _gather_rows(dout, view.centre_rows)
         else:
             dout = dout.contiguous()

@@ -343,23 +343,21 @@ class _SortedView:
         grid, samples = nbh._grid, nbh._point_cloud_sampled
         self.points_in = grid._sorted_points
         self.point_rows = grid._sorted_indices           # int32, for kernels
-        self.point_order = grid._sorted_indices.long()
+        self._point_order = self._centre_order = None    # their int64 forms, on first use
         n_out = samples._points.shape[0]
         if nbh._equal_samples:
-            self.centre_order = self.centre_rows = None
+            self.centre_rows = None
             self.points_out = grid._sorted_points
             self.table, self.ranges = nbh._neighbors, nbh._samples_neigh_ranges
         elif nbh._self_neighborhood is not None:     # same cloud: the shared sorted search
             own = nbh._self_neighborhood
             self.centre_rows = grid._sorted_indices
-            self.centre_order = grid._sorted_indices.long()
             self.points_out = grid._sorted_points
             self.table, self.ranges = own._neighbors, own._samples_neigh_ranges
         else:
             order = nbh.compute_centre_order()
-            self.points_out = samples._points[order.long()].contiguous()
             self.centre_rows = order
-            self.centre_order = order.long()
+            self.points_out = samples._points[self.centre_order].contiguous()
             L = _lib.lib()
             L.mccnn_reorder_neighbors_workspace_bytes.restype = _lib.csize
             dev = nbh._neighbors.device
@@ -379,10 +377,24 @@ class _SortedView:
         else:
             self.ranges_t, pair_order = tfg_custom_ops.transpose_neighbors(
                 self.table, self.points_in.shape[0])
-            sel = pair_order.long()
-            self.table_t = torch.stack((self.table[sel, 1], self.table[sel, 0]),
-                                       dim=1).contiguous()
+            self.table_t = torch.empty_like(self.table)
+            _lib.call("swapped_pairs", stream(), i64(self.table.shape[0]), ptr(self.table, _I32),
+                      ptr(pair_order, _I32), ptr(self.table_t))
         self._pdf_key, self.pdf, self.pdf_t = None, None, None
+
+    @property
+    def point_order(self):
+        """position -> original point id as int64 (for torch indexing)."""
+        if self._point_order is None:
+            self._point_order = self.point_rows.long()
+        return self._point_order
+
+    @property
+    def centre_order(self):
+        """slot -> original centre id as int64, None if the centres are the sorted points."""
+        if self._centre_order is None and self.centre_rows is not None:
+            self._centre_order = self.centre_rows.long()
+        return self._centre_order
 
     def pair_pdf(self, nbh):
         """Per-pair densities of `table` and `table_t` (the neighbour point's)."""
