@@ -436,20 +436,28 @@ extern "C" int mccnn_final_product(mccnn_stream_t stream, int64_t num_rows, int 
   if (num_rows == 0) return MCCNN_OK;
   MCCNN_REQUIRE(x && w && out, "final_product received a null tensor");
   hipStream_t s = as_stream(stream);
-  unsigned blocks = 1;
-  int rc = layer_grid(num_rows, &blocks);
-  if (rc != MCCNN_OK) return rc;
+  int device = 0, cus = 0, rc = MCCNN_OK;
+  MCCNN_HIP_CHECK(hipGetDevice(&device));
+  MCCNN_HIP_CHECK(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device));
   const int R = num_cols_in, F = num_cols_out;
+  const int64_t tiles = (num_rows + kLayerWaves - 1) / kLayerWaves;
   // weights beyond a block's registers: the tiled product, once its 128- or 256-row tiles give
   // every compute unit a block (below that a launch is a few blocks walking the whole
   // reduction alone: 170 us for 400 rows x 4096 x 256 against 20 us for the blocked
   // register-resident product, whose tiles are 16 rows)
   if ((int64_t)R * F > 65536 && tile_product_supported(R, F) &&
       (num_rows + tile_product_rows(F) - 1) / tile_product_rows(F) *
-              (F / (F % 128 == 0 ? 128 : 64)) >= (int64_t)blocks)
+              (F / (F % 128 == 0 ? 128 : 64)) >= cus)
     return launch_tile_product(s, num_rows, R, x, F, w, false, out_rows, out);
   int rb = 0, fb = 0;
   product_blocks(R, F, &rb, &fb);
+  // A small input leaves compute units idle: narrower column blocks with longer reduction
+  // blocks then give more blocks of threads, each walking fewer blocks of the reduction
+  // (1500 rows x 4096 x 256: 8 visits of 512 rows of w per block of threads become 4 of 1024)
+  while (fb > 16 && rb < 1024 && R % (2 * rb) == 0 && tiles * (F / (fb / 2)) <= cus) {
+    fb /= 2;
+    rb *= 2;
+  }
   // out[:, f0:f0+fb] = sum over the reduction blocks r0 of x[:, r0:r0+rb] W[r0:r0+rb, f0:f0+fb]:
   // one launch, column block f0 = blockIdx.y * fb, every block walking the reduction blocks
   // in order for its own tiles
@@ -460,17 +468,11 @@ extern "C" int mccnn_final_product(mccnn_stream_t stream, int64_t num_rows, int 
   ld.r_total = R;
   ld.f_block = fb;
   const int col_blocks = F / fb;
-  {
-    // one block per compute unit in all (the register-resident weights and the LDS tile
-    // fill it), shared among the column blocks; never more blocks than tiles
-    int device = 0, cus = 0;
-    MCCNN_HIP_CHECK(hipGetDevice(&device));
-    MCCNN_HIP_CHECK(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device));
-    const int64_t tiles = (num_rows + kLayerWaves - 1) / kLayerWaves;
-    int64_t per = cus / col_blocks < 1 ? 1 : cus / col_blocks;
-    if (per > tiles) per = tiles;
-    blocks = (unsigned)per;
-  }
+  // one block per compute unit in all (the register-resident weights and the LDS tile
+  // fill it), shared among the column blocks; never more blocks than tiles
+  int64_t per = cus / col_blocks < 1 ? 1 : cus / col_blocks;
+  if (per > tiles) per = tiles;
+  const unsigned blocks = (unsigned)per;
   MCCNN_LAYER_SHAPE_SWITCH(rb / kFusedK, fb,
                            rc = launch_layer(final_product_kernel<CPL, FT>, s,
                                              dim3(blocks, (unsigned)col_blocks),
