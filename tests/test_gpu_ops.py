@@ -514,6 +514,12 @@ def test_gathered_feature_gradient(ops, oracle, c, k):
     expect_order = np.argsort(ids[:, 0], kind="stable")
     assert np.array_equal(t_order.cpu().numpy(), expect_order)
     assert np.array_equal(t_ranges.cpu().numpy(), np.cumsum(np.bincount(ids[:, 0], minlength=n)))
+    # the rows of the transposed table: (centre, point) of the pairs in that order
+    from tensorflow_graphics_point_clouds_amd import _lib
+    from tensorflow_graphics_point_clouds_amd._lib import i64, ptr, stream
+    swapped = torch.empty((len(ids), 2), dtype=torch.int32, device="cuda")
+    _lib.call("swapped_pairs", stream(), i64(len(ids)), ptr(dev(ids)), ptr(t_order), ptr(swapped))
+    assert np.array_equal(swapped.cpu().numpy(), ids[expect_order][:, ::-1])
     basis = rng.random((len(ids), k)).astype(np.float32)
     feat = rng.standard_normal((n, c)).astype(np.float32)
     up = rng.standard_normal((900, c, k)).astype(np.float32)
