@@ -95,6 +95,23 @@ int mccnn_grid_setup(mccnn_stream_t stream, int64_t num_pts, int num_dims,
                      int32_t *num_cells_out, float *scaled_aabb_min_out,
                      float *inv_cell_sizes_out);
 
+/* The whole grid of pylib/pc/Grid.py:32-64 in one call: mccnn_grid_setup,
+ * mccnn_compute_keys, the host copy of the grid shape (one synchronisation of the
+ * stream; num_cells_out_host [D] and *key_bits_out_host are host memory),
+ * mccnn_sort_keys_descending with that key width, mccnn_gather_points.  Same outputs
+ * as the five calls; for small clouds, whose cost is the calls and launches
+ * themselves.  Workspace: mccnn_build_grid_workspace_bytes(num_pts). */
+size_t mccnn_build_grid_workspace_bytes(int64_t num_pts);
+int mccnn_build_grid(mccnn_stream_t stream, int64_t num_pts, int num_dims,
+                     const float *points, const int32_t *batch_ids, int batch_size,
+                     const float *cell_sizes, float *aabb_min_out, float *aabb_max_out,
+                     int32_t *num_cells_out, float *scaled_aabb_min_out,
+                     float *inv_cell_sizes_out, int64_t *keys_out,
+                     int64_t *sorted_keys_out, int32_t *sorted_indices_out,
+                     float *sorted_points_out, int32_t *sorted_batch_ids_out,
+                     void *workspace, size_t workspace_bytes,
+                     int32_t *num_cells_out_host, int *key_bits_out_host);
+
 /* Small gathers of the caller glue:
  *   original ids  out[m] = (sorted_indices[neighbors[m,0]], neighbors[m,1])
  *                 pylib/pc/Neighborhood.py:246-250

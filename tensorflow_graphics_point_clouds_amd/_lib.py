@@ -43,7 +43,8 @@ def lib():
                 "`make -C %s` or __graft_entry__.build()" % (LIB_PATH, CSRC_DIR))
         handle = ctypes.CDLL(LIB_PATH)
         handle.mccnn_last_error.restype = ctypes.c_char_p
-        for name in ("mccnn_find_neighbors_workspace_bytes",
+        for name in ("mccnn_build_grid_workspace_bytes",
+                     "mccnn_find_neighbors_workspace_bytes",
                      "mccnn_mc_basis_grads_workspace_bytes",
                      "mccnn_mc_conv_project_grads_workspace_bytes",
                      "mccnn_pointconv_density_grads_workspace_bytes",

@@ -441,3 +441,49 @@ extern "C" int mccnn_gather_i32(mccnn_stream_t stream, int64_t count, const int3
   MCCNN_LAUNCH_CHECK();
   return MCCNN_OK;
 }
+
+// The grid of pylib/pc/Grid.py:32-64 in one call: bounding boxes and grid shape, keys, the
+// host copy of the grid shape (the one synchronisation: it sizes the key width of the sort
+// and, for the caller, the grid table), stable descending sort, gathers.  The same
+// sequence a caller gets from the five entry points above; small clouds are bound by the
+// cost of making calls and launches, and this is one call instead of five.
+extern "C" size_t mccnn_build_grid_workspace_bytes(int64_t num_pts) {
+  return mccnn_sort_keys_workspace_bytes(num_pts);
+}
+
+extern "C" int mccnn_build_grid(mccnn_stream_t stream, int64_t num_pts, int num_dims,
+                                const float *points, const int32_t *batch_ids, int batch_size,
+                                const float *cell_sizes, float *aabb_min_out,
+                                float *aabb_max_out, int32_t *num_cells_out,
+                                float *scaled_aabb_min_out, float *inv_cell_sizes_out,
+                                int64_t *keys_out, int64_t *sorted_keys_out,
+                                int32_t *sorted_indices_out, float *sorted_points_out,
+                                int32_t *sorted_batch_ids_out, void *workspace,
+                                size_t workspace_bytes, int32_t *num_cells_out_host,
+                                int *key_bits_out_host) {
+  MCCNN_REQUIRE(valid_dims(num_dims), "build_grid expects a valid number of dimensions");
+  MCCNN_REQUIRE(num_cells_out_host && key_bits_out_host,
+                "build_grid needs host outputs for the grid shape and the key width");
+  int rc = mccnn_grid_setup(stream, num_pts, num_dims, points, batch_ids, batch_size, cell_sizes,
+                            aabb_min_out, aabb_max_out, num_cells_out, scaled_aabb_min_out,
+                            inv_cell_sizes_out);
+  if (rc != MCCNN_OK) return rc;
+  rc = mccnn_compute_keys(stream, num_pts, num_dims, points, num_pts, batch_ids, batch_size,
+                          num_dims, scaled_aabb_min_out, num_dims, num_cells_out, num_dims,
+                          inv_cell_sizes_out, keys_out);
+  if (rc != MCCNN_OK) return rc;
+  hipStream_t s = as_stream(stream);
+  MCCNN_HIP_CHECK(hipMemcpyAsync(num_cells_out_host, num_cells_out, sizeof(int32_t) * num_dims,
+                                 hipMemcpyDeviceToHost, s));
+  MCCNN_HIP_CHECK(hipStreamSynchronize(s));
+  unsigned long long total = (unsigned long long)(batch_size > 0 ? batch_size : 1);
+  for (int d = 0; d < num_dims; ++d) total *= (unsigned long long)num_cells_out_host[d];
+  int bits = 1;
+  while (bits < 64 && (1ull << bits) < total) ++bits;
+  *key_bits_out_host = bits;
+  rc = mccnn_sort_keys_descending(stream, num_pts, bits, keys_out, sorted_keys_out,
+                                  sorted_indices_out, workspace, workspace_bytes);
+  if (rc != MCCNN_OK) return rc;
+  return mccnn_gather_points(stream, num_pts, num_dims, points, batch_ids, sorted_indices_out,
+                             sorted_points_out, sorted_batch_ids_out);
+}

@@ -6,6 +6,7 @@ grid shape, sort and gathers are kernels of libmccnn_hip.so as well.
 """
 import ctypes
 import enum
+import threading
 import math
 
 import numpy as np
@@ -261,6 +262,10 @@ def _sort_keys(keys, key_bits):
     return sorted_keys, sorted_indices
 
 
+_ONE_CALL_GRID = 16384     # points up to which a grid is built by the single-call entry point
+_pinned_shape = threading.local()
+
+
 class Grid:
     """Regular grid over a point cloud (pylib/pc/Grid.py:32-84): grid shape from
     the per-cloud bounding boxes, cell keys, stable descending sort, gathers."""
@@ -279,6 +284,34 @@ class Grid:
         self._num_cells = torch.empty(d, dtype=_I32, device=dev)
         self._scaled_aabb_min = torch.empty((b, d), dtype=_F32, device=dev)
         self._inv_cell_sizes = torch.empty(d, dtype=_F32, device=dev)
+        self._fast_DS = None
+        self._sorted_positions = None
+        self._self_neighborhoods = {}
+        if 0 < n <= _ONE_CALL_GRID:
+            # small clouds are bound by calls and launches: the same five steps in one call
+            self._cur_keys = torch.empty(n, dtype=_I64, device=dev)
+            self._sorted_keys = torch.empty(n, dtype=_I64, device=dev)
+            self._sorted_indices = torch.empty(n, dtype=_I32, device=dev)
+            self._sorted_points = torch.empty_like(pc._points)
+            self._sorted_batch_ids = torch.empty_like(pc._batch_ids)
+            ws = _lib.workspace(L.mccnn_build_grid_workspace_bytes(i64(n)), dev)
+            # the grid shape comes back through pinned host memory (one allocation, reused)
+            # (per host thread: two threads may build grids at the same time)
+            pinned = getattr(_pinned_shape, "buffer", None)
+            if pinned is None:
+                pinned = _pinned_shape.buffer = torch.empty(16, dtype=_I32, pin_memory=True)
+            cells_host = (ctypes.c_int32 * d).from_address(pinned.data_ptr())
+            bits_host = ctypes.c_int.from_address(pinned.data_ptr() + 32)
+            _lib.call("build_grid", stream(), i64(n), cint(d), ptr(pc._points, _F32),
+                      ptr(pc._batch_ids, _I32), cint(b), ptr(self._cell_sizes),
+                      ptr(self._aabb_min), ptr(self._aabb_max), ptr(self._num_cells),
+                      ptr(self._scaled_aabb_min), ptr(self._inv_cell_sizes), ptr(self._cur_keys),
+                      ptr(self._sorted_keys), ptr(self._sorted_indices), ptr(self._sorted_points),
+                      ptr(self._sorted_batch_ids), ptr(ws), _lib.csize(ws.numel()), cells_host,
+                      ctypes.byref(bits_host))
+            self._num_cells_host = [int(v) for v in cells_host]
+            self._key_bits = int(bits_host.value)
+            return
         _lib.call("grid_setup", stream(), i64(n), cint(d), ptr(pc._points, _F32), ptr(pc._batch_ids, _I32), cint(b),
             ptr(self._cell_sizes), ptr(self._aabb_min), ptr(self._aabb_max),
             ptr(self._num_cells), ptr(self._scaled_aabb_min), ptr(self._inv_cell_sizes))
@@ -296,9 +329,6 @@ class Grid:
         self._sorted_batch_ids = torch.empty_like(pc._batch_ids)
         _lib.call("gather_points", stream(), i64(n), cint(d), ptr(pc._points), ptr(pc._batch_ids),
             ptr(self._sorted_indices), ptr(self._sorted_points), ptr(self._sorted_batch_ids))
-        self._fast_DS = None
-        self._sorted_positions = None
-        self._self_neighborhoods = {}
 
     def sorted_positions(self):
         """Inverse of the sort: position of every original point in the sorted order."""
