@@ -417,21 +417,32 @@ class MCConv(torch.nn.Module):
         result is cut back.  None if the shape is out of reach."""
         d, c, f, l, h = (self._num_dims, self._num_features_in, self._num_features_out,
                          self._num_mlps, self._hidden)
-        if k not in (16, 32, 64) or d not in (2, 3):
+        if d not in (2, 3):
             return None
+        # hidden units per kernel MLP padded with zero columns until the layer has 16, 32 or
+        # 64 basis columns (every activation maps 0 to 0, and the rows of the final weights
+        # that meet the padding are zero too): `MCConv(c, f, 3, 1, [8])` then runs on the
+        # 16-column kernels
+        h_pad = next((v // l for v in (16, 32, 64) if v % l == 0 and v // l >= h), None)
         pad = _layer_padding(c, f, l)
-        if pad is None:
+        if pad is None or h_pad is None:
             return None
         c_pad, g_pad = pad
         g = f // l
+        weights = self.weights
+        if h_pad != h:
+            weights = torch.nn.functional.pad(weights, (0, h_pad - h))
+            biases = torch.nn.functional.pad(biases, (0, h_pad - h))
+            k = l * h_pad
         fuse_final = self.fuse_final and bool(_lib.lib().mccnn_mc_conv_layer_supported(
             cint(d), cint(c_pad), cint(k), cint(g_pad * l)))
         final = self.final_weights
-        if c_pad != c or g_pad != g:
+        if c_pad != c or g_pad != g or h_pad != h:
             final = torch.nn.functional.pad(final.reshape(l, c, h, g),
-                                            (0, g_pad - g, 0, 0, 0, c_pad - c))
-            final = final.reshape(l, c_pad * h, g_pad)
+                                            (0, g_pad - g, 0, h_pad - h, 0, c_pad - c))
+            final = final.reshape(l, c_pad * h_pad, g_pad)
             features = torch.nn.functional.pad(features, (0, c_pad - c))
+            h = h_pad
         inv_radii = pc._reciprocal(radii)
         per = 16 // h if h <= 16 and 16 % h == 0 else 0       # kernel MLPs per 16 basis columns
         if k > 16 and per > 0 and l % per == 0 and (per * g_pad) % 16 == 0:
@@ -440,14 +451,14 @@ class MCConv(torch.nn.Module):
             # slice of the output: the dense products then cost l / per times less than on
             # the block-diagonal [C*K, F] matrix (default constructor, 4 x 8: 16.5 -> 12 ms
             # per step on the scene-scale batch).
-            outs = [_MCConvLayer.apply(self.weights[t:t + per], biases[t:t + per],
-                                       final[t:t + per], features, neighborhood, inv_radii,
-                                       self._act, False)
+            outs = [_MCConvLayer.apply(weights[t:t + per].contiguous(),
+                                       biases[t:t + per].contiguous(), final[t:t + per],
+                                       features, neighborhood, inv_radii, self._act, False)
                     for t in range(0, l, per)]
             out = torch.cat(outs, dim=1)
         else:
-            out = _MCConvLayer.apply(self.weights, biases, final, features, neighborhood,
-                                     inv_radii, self._act, fuse_final)
+            out = _MCConvLayer.apply(weights.contiguous(), biases.contiguous(), final, features,
+                                     neighborhood, inv_radii, self._act, fuse_final)
         if g_pad != g:
             out = out.reshape(-1, l, g_pad)[:, :, :g].reshape(-1, f)
         return out
