@@ -260,9 +260,17 @@ class Neighborhood:
             self.samples, self.sample_batch_ids, grid.sorted_points, grid.sorted_keys,
             grid.get_ds(), grid.num_cells, grid.scaled_aabb_min, grid.inv_cell_sizes,
             self.inv_radii, max_neighbors)
-        self.original_neigh_ids = np.stack(
-            [grid.sorted_indices[self.neighbors[:, 0]], self.neighbors[:, 1]],
-            axis=1).astype(np.int32)
+        self._original = None
+
+    @property
+    def original_neigh_ids(self):
+        """Neighborhood.py:246-250: the pairs with the points' ids before the sort (built
+        on first use: the gather takes seconds at 10^8 pairs)."""
+        if self._original is None:
+            self._original = np.empty_like(self.neighbors)
+            self._original[:, 0] = np.take(self.grid.sorted_indices, self.neighbors[:, 0])
+            self._original[:, 1] = self.neighbors[:, 1]
+        return self._original
 
     def pdf_per_pair(self, bandwidth=0.2, mode=0):
         d = self.grid.points.shape[1]

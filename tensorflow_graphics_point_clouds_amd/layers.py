@@ -434,8 +434,12 @@ class MCConv(torch.nn.Module):
             weights = torch.nn.functional.pad(weights, (0, h_pad - h))
             biases = torch.nn.functional.pad(biases, (0, h_pad - h))
             k = l * h_pad
-        fuse_final = self.fuse_final and bool(_lib.lib().mccnn_mc_conv_layer_supported(
-            cint(d), cint(c_pad), cint(k), cint(g_pad * l)))
+        # the backward runs the same single-kernel layer transposed (output channels as its
+        # input channels), so both directions have to be covered
+        supported = _lib.lib().mccnn_mc_conv_layer_supported
+        fuse_final = (self.fuse_final
+                      and bool(supported(cint(d), cint(c_pad), cint(k), cint(g_pad * l)))
+                      and bool(supported(cint(d), cint(g_pad * l), cint(k), cint(c_pad))))
         final = self.final_weights
         if c_pad != c or g_pad != g or h_pad != h:
             final = torch.nn.functional.pad(final.reshape(l, c, h, g),

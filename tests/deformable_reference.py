@@ -34,6 +34,7 @@ def check_deformable_kpconv(pts, bids, ctr, cb, batch, ids_np, radius, feat, kp,
     entries), takes the layer's values inside it, and is then carried on to the
     features and the offset weights, so that every parameter gradient is compared in
     full."""
+    from oracle import layers_f64 as L
     from tensorflow_graphics_point_clouds_amd import layers, pc
     n, c = len(ctr), feat.shape[1]
     kpn = kp.shape[0]
@@ -46,34 +47,28 @@ def check_deformable_kpconv(pts, bids, ctr, cb, batch, ids_np, radius, feat, kp,
     tkp = torch.tensor(kp.astype(np.float64) * 0.75).cuda()
     centre = ids[:, 1]
 
-    def weight(dist):
-        if kind == "linear":
-            return torch.relu(1 - dist / sigma)
-        return torch.exp(-(dist / (sigma / 3)) ** 2)
-
     tf = torch.tensor(feat.astype(np.float64), device="cuda", requires_grad=True)
     tw = torch.tensor(wts.astype(np.float64), device="cuda", requires_grad=True)
     two = torch.tensor(woff.astype(np.float64), device="cuda", requires_grad=True)
 
-    def project(basis, f):
-        return torch.zeros(n, c, kpn, **f64).index_add(
-            0, centre, f[ids[:, 0]][:, :, None] * basis[:, None, :])
-
-    rigid = weight((delta[:, None, :] - tkp[None]).norm(dim=2))
-    off = (project(rigid, tf).reshape(n, -1) @ two).reshape(n, kpn, 3)
+    # the float64 restatement lives beside the oracle (oracle/layers_f64.py) and is pinned on
+    # the CPU by tests/test_oracle_float.py; here it runs on the device
+    weight = lambda dist: L.kp_weight(dist, sigma, kind)
+    off = L.kp_offsets(delta, ids, n, tf, tkp, two, sigma, kind)
     cut = off.detach().clone().requires_grad_(True)          # the reference, cut at the offsets
-    dist = (delta[:, None, :] - (tkp[None] + cut[centre])).norm(dim=2)
-    deformed = weight(dist)
-    ref_out = project(deformed, tf).reshape(n, -1) @ tw
+    ref_out, dist = L.kp_conv(delta, ids, n, tf, tkp, tw, sigma, kind, cut)
     with torch.no_grad():
-        out_mag = project(deformed, tf.abs()).reshape(n, -1) @ tw.abs()
+        out_mag = L.project(weight(dist), tf.abs(), ids, n).reshape(n, -1) @ tw.abs()
+    # (a centre without pairs contributes 0 to the fitting term in this library; TensorFlow's
+    # segment minimum would contribute the largest float32)
+    fit_sum, rep_sum = L.kp_regularization_loss(dist, ids, n, tkp, cut, sigma, kind,
+                                                empty_value=0.0)
+    ref_loss = fit_sum + rep_sum
     sq = (dist / sigma) ** 2
     expand = centre[:, None].expand(-1, kpn)
     fit = torch.full((n, kpn), float("inf"), **f64).scatter_reduce(0, expand, sq, "amin")
     kpd = tkp[None] + cut
     kd = (kpd[:, None] - kpd[:, :, None] + 1e-300).norm(dim=3)
-    rep = weight(kd) * (1 - torch.eye(kpn, **f64))[None]
-    ref_loss = fit.sum() + rep.sum()
 
     with torch.no_grad():       # (centre, kernel point) entries whose gradient may flip
         unsure_out = torch.zeros((n, kpn), dtype=torch.bool, device="cuda")

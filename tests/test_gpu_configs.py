@@ -391,7 +391,7 @@ def _chunked_dot(a, b, chunk=1 << 27):
     return s, t
 
 
-@pytest.mark.parametrize("radius", [0.04, 0.06])
+@pytest.mark.parametrize("radius", [0.02, 0.04, 0.06])
 def test_config4_basis_proj_beyond_int32_element_offsets(radius):
     """Dense configuration at its real size: 4 x 200k uniform points, C = 128, K = 32.
     The projection holds N*C*K = 3.28e9 elements (offsets pass 2^31 from centre 524 288
@@ -435,7 +435,7 @@ def test_config4_basis_proj_beyond_int32_element_offsets(radius):
         assert_rel_t(dbasis[a:e], torch.einsum("ck,mc->mk", g, f),
                      torch.einsum("ck,mc->mk", g.abs(), f.abs()))
     # the last rows of the basis gradient (beyond element 2^32 at radius 0.06)
-    assert (m - 1) * k > (2 ** 32 if radius == 0.06 else 2 ** 30)
+    assert (m - 1) * k > {0.02: 2 ** 27, 0.04: 2 ** 30, 0.06: 2 ** 32}[radius]
     # feature gradient of sampled points: all pairs whose neighbour is that point
     order = torch.argsort(idl[:, 0], stable=True)
     sorted_pt = idl[order, 0]
@@ -451,6 +451,36 @@ def test_config4_basis_proj_beyond_int32_element_offsets(radius):
     rb, _ = _chunked_dot(dbasis, basis)
     rf, _ = _chunked_dot(dfeat, feat)
     assert abs(lhs - rb) <= REL * scale and abs(lhs - rf) <= REL * scale
+
+
+@pytest.mark.parametrize("radius", [0.02, 0.04, 0.06])
+def test_config4_compute_pdf_sampled_rows_at_full_size(radius):
+    """Density estimate of the 4 x 200k uniform clouds (bandwidth 0.2) at the three radii:
+    rows sampled over the whole cloud (the last point included) are recomputed in float64
+    on the device from the GPU's own pair table with the Gaussian product of
+    compute_pdf_kernels.cu.cc:72-130, and the pair table itself is the one
+    tests/test_gpu_full_size.py compares with the oracle.  1e-5 relative (all terms of the
+    sum are positive, so the sum is its own magnitude)."""
+    from tensorflow_graphics_point_clouds_amd import pc, synthetic
+    cfg = synthetic.config4()
+    cloud = pc.PointCloud(dev(cfg["points"]), dev(cfg["batch_ids"]), cfg["batch_size"])
+    grid = pc.Grid(cloud, radius)
+    nbh = pc.Neighborhood(grid, radius)
+    pdf = nbh.point_pdf(bandwidth=0.2)                 # per sorted point
+    n = grid._sorted_points.shape[0]
+    assert pdf.shape[0] == n
+    rng = np.random.default_rng(int(radius * 1000))
+    picks = np.concatenate([rng.integers(0, n, 400), [0, n - 1]])
+    ends, pairs, pts = nbh._samples_neigh_ranges.long(), nbh._neighbors.long(), grid._sorted_points
+    bw, norm = 1.0 / 0.2, 0.3989422804014327
+    inv_r = 1.0 / float(np.float32(radius))
+    for i in picks.tolist():
+        a = int(ends[i - 1]) if i > 0 else 0
+        e = int(ends[i])
+        assert bool((pairs[a:e, 1] == i).all())
+        u = (pts[pairs[a:e, 0]].double() - pts[i].double()) * bw * inv_r
+        expect = float((bw * norm * torch.exp(-0.5 * u * u)).prod(dim=1).sum())
+        assert abs(float(pdf[i]) - expect) <= REL * expect, (i, float(pdf[i]), expect)
 
 
 @pytest.mark.parametrize("radius", [0.04, 0.06])

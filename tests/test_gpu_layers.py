@@ -59,7 +59,10 @@ _T_ACT = {"relu": torch.relu, "leaky_relu": lambda x: torch.nn.functional.leaky_
                           (32, 32, 8, 4, "leaky_relu"), (16, 64, 8, 8, "relu"),
                           (64, 16, 32, 1, "elu"), (128, 24, 16, 2, "relu"),
                           # 8 basis columns: hidden units padded with zero columns to 16
-                          (16, 16, 8, 1, "elu"), (32, 32, 4, 2, "leaky_relu")])
+                          (16, 16, 8, 1, "elu"), (32, 32, 4, 2, "leaky_relu"),
+                          # 128 output channels: the transposed single-kernel layer of the
+                          # backward is not covered, the layer has to take the two-kernel form
+                          (16, 128, 16, 1, "relu"), (32, 128, 16, 1, "elu")])
 def test_mcconv_forward_backward(oracle, c_in, c_out, hidden, num_mlps, act, fused, gathered,
                                  transposed, fuse_final):
     from tensorflow_graphics_point_clouds_amd import layers, pc, synthetic
@@ -172,16 +175,14 @@ def test_pointconv_forward_backward(oracle, hidden, act, fused):
     t = {k: torch.tensor(v.astype(np.float64), requires_grad=True) for k, v in par.items()}
     tf = torch.tensor(feat.astype(np.float64), requires_grad=True)
     diff = torch.tensor((pts[ids[:, 0]] - ctr[ids[:, 1]]).astype(np.float64))
-    hid = _T_ACT[act](diff @ t["weights"] + t["biases"])
+    # the float64 restatement is oracle/layers_f64.point_conv, pinned on the CPU against the
+    # per-centre loop of point_conv_test.py:75-117 (tests/test_oracle_float.py)
+    from oracle import layers_f64
     tpdf = torch.tensor(pdf.astype(np.float64))
-    mx = torch.zeros(len(ctr), dtype=torch.float64).scatter_reduce(0, ids[:, 1], tpdf, "amax",
-                                                                   include_self=False)
-    rel = (tpdf / mx[ids[:, 1]]).reshape(-1, 1)
-    cur = torch.relu(rel @ t["pw1"] + t["pb1"]) @ t["pw2"] + t["pb2"]
-    basis = hid / cur
-    per_pair = tf[ids[:, 0]][:, :, None] * basis[:, None, :]
-    proj = torch.zeros(len(ctr), c_in, hidden, dtype=torch.float64).index_add(0, ids[:, 1], per_pair)
-    ref = proj.reshape(len(ctr), -1) @ t["final_weights"]
+    ref, basis, cur, rel = layers_f64.point_conv(
+        diff, ids, len(ctr), tf, tpdf, t["weights"], t["biases"], t["final_weights"],
+        t["pw1"], t["pb1"], t["pw2"], t["pb2"], _T_ACT[act])
+    hid = basis * cur
     up = rng.standard_normal(ref.shape).astype(np.float32)
     out.backward(dev(up))
     (ref * torch.tensor(up.astype(np.float64))).sum().backward()

@@ -340,3 +340,208 @@ def test_mc_basis_activations_hand_values(oracle, activation):
         assert got[0, 0] == -0.4 / 2.0 and got[0, 1] == -0.1 / 2.0
     if activation == "elu":
         np.testing.assert_allclose(got[1, 0], (math.exp(-2.0) - 1.0) / 0.5, rtol=1e-14)
+
+
+# ---------------------------------------------------------------------------------------
+# Float64 layer restatements with gradients (oracle/layers_f64.py): deformable KPConv, its
+# regularisation loss, PointConv.  Each is pinned here on the CPU by hand-computed values
+# or by scalar loops, chosen so that a dropped square, a wrong sigma, a minimum over the
+# wrong axis, a kept diagonal or a single-counted pair fails.
+
+def _t(a):
+    return torch.tensor(np.asarray(a, dtype=np.float64))
+
+
+def _cloud(rng, n, batch):
+    pts = rng.random((n, 3)).astype(np.float32)
+    return pts, np.repeat(np.arange(batch), n // batch).astype(np.int32)
+
+
+_REG_KP = [[0.0, 0.0, 0.0], [0.4, 0.0, 0.0], [0.0, 0.3, 0.0]]
+_REG_PAIRS = [[0, 0], [1, 0], [2, 1]]
+_REG_DELTA = [[0.3, 0.0, 0.0], [0.0, 0.3, 0.4], [0.1, 0.0, 0.0]]
+
+
+def _reg_offsets(n_out=2):
+    off = np.zeros((n_out, 3, 3))
+    off[1, 0] = [0.1, 0.0, 0.0]          # centre 1: kernel point 0 moves onto its one pair
+    return off
+
+
+def test_kp_regularization_fit_hand_values():
+    """KPConv.py:404-410.  sigma = 0.5; centre 0 has two pairs, at distances
+    (0.3, 0.1, sqrt 0.18) and (0.5, sqrt 0.41, 0.4) from the three kernel points: the
+    minima per kernel point are 0.3, 0.1, 0.4 -> (d / sigma)^2 = 0.36 + 0.04 + 0.64.
+    Centre 1 has one pair, which the offset puts on kernel point 0: 0 + 0.36 + 0.4.
+    (Without the square the sum would be 1.6 + ..., with the minimum taken per pair
+    instead of per kernel point centre 0 would give 0.04 + 0.64.)"""
+    import torch
+    from oracle import layers_f64 as L
+    pairs = torch.tensor(_REG_PAIRS)
+    dist = L.kp_distances(_t(_REG_DELTA), pairs, _t(_REG_KP), _t(_reg_offsets()))
+    np.testing.assert_allclose(dist[0].numpy(), [0.3, 0.1, np.sqrt(0.18)], rtol=1e-14)
+    np.testing.assert_allclose(dist[1].numpy(), [0.5, np.sqrt(0.41), 0.4], rtol=1e-14)
+    np.testing.assert_allclose(dist[2].numpy(), [0.0, 0.3, np.sqrt(0.1)], atol=1e-15)
+    fit, _ = L.kp_regularization_loss(dist, pairs, 2, _t(_REG_KP), _t(_reg_offsets()), 0.5,
+                                      "linear")
+    np.testing.assert_allclose(float(fit), (0.36 + 0.04 + 0.64) + (0.0 + 0.36 + 0.4), rtol=1e-13)
+    # another sigma rescales every term by (0.5 / sigma)^2
+    fit2, _ = L.kp_regularization_loss(dist, pairs, 2, _t(_REG_KP), _t(_reg_offsets()), 0.25,
+                                       "gaussian")
+    np.testing.assert_allclose(float(fit2), 4.0 * 1.8, rtol=1e-13)
+    # a centre without pairs: TensorFlow's unsorted_segment_min yields the largest float32
+    fit3, _ = L.kp_regularization_loss(dist, pairs, 3, _t(_REG_KP), _t(_reg_offsets(3)), 0.5,
+                                       "linear")
+    np.testing.assert_allclose(float(fit3), 1.8 + 3 * float(np.finfo(np.float32).max), rtol=1e-13)
+    fit4, _ = L.kp_regularization_loss(dist, pairs, 3, _t(_REG_KP), _t(_reg_offsets(3)), 0.5,
+                                       "linear", empty_value=0.0)
+    np.testing.assert_allclose(float(fit4), 1.8, rtol=1e-13)
+
+
+def test_kp_regularization_repulsion_closed_form():
+    """KPConv.py:412-427.  Centre 0 (no offsets): kernel-point distances 0.4, 0.3, 0.5 at
+    sigma 0.5 -> linear weights 0.2, 0.4, 0; the diagonal is excluded and every unordered
+    pair appears twice in the [K, K] matrix: 2 (0.2 + 0.4).  Centre 1: kernel point 0 is
+    moved to (0.1, 0, 0): distances 0.3, sqrt 0.1, 0.5 -> 2 (0.4 + 1 - sqrt(0.1)/0.5).
+    (With the diagonal kept each centre would gain K = 3.)"""
+    import math
+    import torch
+    from oracle import layers_f64 as L
+    pairs = torch.tensor(_REG_PAIRS)
+    dist = L.kp_distances(_t(_REG_DELTA), pairs, _t(_REG_KP), _t(_reg_offsets()))
+    _, rep = L.kp_regularization_loss(dist, pairs, 2, _t(_REG_KP), _t(_reg_offsets()), 0.5,
+                                      "linear")
+    expect = 2 * (0.2 + 0.4) + 2 * (0.4 + 1.0 - math.sqrt(0.1) / 0.5)
+    np.testing.assert_allclose(float(rep), expect, rtol=1e-13)
+    _, rep_g = L.kp_regularization_loss(dist, pairs, 2, _t(_REG_KP), _t(_reg_offsets()), 0.5,
+                                        "gaussian")
+    s = 0.5 / 3.0
+    g = lambda d: math.exp(-(d / s) ** 2)
+    expect_g = 2 * (g(0.4) + g(0.3) + g(0.5)) + 2 * (g(0.3) + g(math.sqrt(0.1)) + g(0.5))
+    np.testing.assert_allclose(float(rep_g), expect_g, rtol=1e-13)
+
+
+def test_kp_regularization_gradient_by_central_differences():
+    """The offset gradient that autograd takes from the restatement, against central
+    differences of the loss value (random offsets keep every term away from its kinks)."""
+    import torch
+    from oracle import layers_f64 as L
+    rng = np.random.default_rng(5)
+    n_out, k, m = 4, 5, 23
+    pairs = torch.tensor(np.stack([rng.integers(0, 30, m), np.sort(rng.integers(0, n_out, m))], 1))
+    delta = _t(rng.random((m, 3)) * 1.2 - 0.6)
+    kp = _t(rng.random((k, 3)) * 0.8 - 0.4)
+    off = _t(0.05 * rng.standard_normal((n_out, k, 3))).requires_grad_(True)
+
+    def loss(o, kind):
+        fit, rep = L.kp_regularization_loss(L.kp_distances(delta, pairs, kp, o), pairs, n_out,
+                                            kp, o, 0.7, kind)
+        return fit + rep
+    for kind in ("linear", "gaussian"):
+        grad, = torch.autograd.grad(loss(off, kind), off)
+        h = 1e-6
+        for idx in [(0, 0, 0), (1, 3, 2), (3, 4, 1), (2, 2, 0)]:
+            step = torch.zeros_like(off)
+            step[idx] = h
+            fd = (loss(off.detach() + step, kind) - loss(off.detach() - step, kind)) / (2 * h)
+            np.testing.assert_allclose(float(grad[idx]), float(fd), rtol=1e-6, atol=1e-8)
+
+
+@pytest.mark.parametrize("kind", ["linear", "gaussian"])
+def test_kp_conv_f64_matches_pinned_pieces(oracle, kind):
+    """The deformable convolution of layers_f64 equals the composition of the separately
+    pinned oracle pieces: kp_basis (scalar-loop test above) with per-pair offsets
+    off[centre(m)], basis_proj (numpy segment-sum test) and a float64 product; with zero
+    offsets it equals the rigid convolution, and the offsets themselves are the rigid
+    convolution with K*D outputs (KPConv.py:317-392)."""
+    import torch
+    from oracle import layers_f64 as L
+    rng = np.random.default_rng(11)
+    pts, bids = _cloud(rng, 400, 2)
+    g = oracle.Grid(pts, bids, 2, np.float32(0.25))
+    nbh = oracle.Neighborhood(g, np.float32(0.25), pts[:60], bids[:60])
+    ids = nbh.original_neigh_ids
+    n_out, c, k, f = 60, 4, 5, 3
+    sigma = 0.8
+    feat = rng.standard_normal((len(pts), c)).astype(np.float32)
+    kp = (rng.random((k, 3)) * 1.2 - 0.6)
+    w = rng.standard_normal((c * k, f))
+    woff = 0.05 * rng.standard_normal((c * k, k * 3))
+    delta = ((pts[ids[:, 0]] - pts[:60][ids[:, 1]]) / np.float32(0.25)).astype(np.float64)
+    tp = torch.tensor(ids).long()
+
+    off = L.kp_offsets(_t(delta), tp, n_out, _t(feat), _t(kp), _t(woff), sigma, kind).numpy()
+    rigid_basis, _ = oracle.kp_basis(delta, kp, sigma, kind)
+    # (the C oracle's basis_proj takes float32 operands: compare the pieces at that precision)
+    rigid_proj = oracle.basis_proj(rigid_basis.astype(np.float32), feat, ids, nbh.ranges)
+    np.testing.assert_allclose(off.reshape(n_out, -1), rigid_proj.reshape(n_out, -1) @ woff,
+                               rtol=1e-5, atol=1e-6)
+
+    for offsets in (np.zeros((n_out, k, 3)), off):
+        out, dist = L.kp_conv(_t(delta), tp, n_out, _t(feat), _t(kp), _t(w), sigma, kind,
+                              _t(offsets))
+        basis, dist_ref = oracle.kp_basis(delta, kp, sigma, kind, offsets[ids[:, 1]])
+        np.testing.assert_allclose(dist.numpy(), dist_ref, rtol=1e-12, atol=1e-14)
+        proj = oracle.basis_proj(basis.astype(np.float32), feat, ids, nbh.ranges)
+        np.testing.assert_allclose(out.numpy(), proj.reshape(n_out, -1) @ w, rtol=1e-5, atol=1e-5)
+    rigid, _ = L.kp_conv(_t(delta), tp, n_out, _t(feat), _t(kp), _t(w), sigma, kind, None)
+    zero, _ = L.kp_conv(_t(delta), tp, n_out, _t(feat), _t(kp), _t(w), sigma, kind,
+                        _t(np.zeros((n_out, k, 3))))
+    assert torch.equal(rigid, zero)
+
+
+def test_pointconv_density_hand_values():
+    """PointConv.py:176-190.  Centre 0 lists densities 2 and 4 (relative 0.5 and 1), centre
+    1 the density 3 (relative 1).  Hidden layer of three units: 2x - 0.5 (positive for
+    both), -x + 0.75 (cut by the relu at x = 1) and x - 2 (always cut); second layer
+    weights 1, 4, 100 and bias 0.25:
+      x = 0.5: relu(0.5) + 4 relu(0.25) + 0 + 0.25 = 1.75;   x = 1: 1.5 + 0 + 0 + 0.25."""
+    import torch
+    from oracle import layers_f64 as L
+    pairs = torch.tensor([[5, 0], [7, 0], [2, 1]])
+    cur, rel = L.pointconv_density(_t([2.0, 4.0, 3.0]), pairs, 2, _t([[2.0, -1.0, 1.0]]),
+                                   _t([[-0.5, 0.75, -2.0]]), _t([[1.0], [4.0], [100.0]]),
+                                   _t([[0.25]]))
+    np.testing.assert_allclose(rel.numpy().ravel(), [0.5, 1.0, 1.0], rtol=1e-15)
+    np.testing.assert_allclose(cur.numpy().ravel(), [1.75, 1.75, 1.75], rtol=1e-15)
+    cur2, _ = L.pointconv_density(_t([2.0, 4.0, 3.0]), pairs, 2, _t([[2.0, -1.0, 1.0]]),
+                                  _t([[-0.5, 0.75, -2.0]]), _t([[1.0], [2.0], [100.0]]),
+                                  _t([[0.25]]))
+    np.testing.assert_allclose(cur2.numpy().ravel(), [1.25, 1.75, 1.75], rtol=1e-15)
+
+
+def test_point_conv_f64_matches_per_centre_loop(oracle):
+    """The PointConv restatement against the per-centre loop of point_conv_test.py:75-117
+    (differences not divided by the radius, density relative to the neighbourhood maximum,
+    1 -> 16 -> 1 network, sum over each centre's pairs, final product)."""
+    import math
+    import torch
+    from oracle import layers_f64 as L
+    rng = np.random.default_rng(13)
+    pts, bids = _cloud(rng, 300, 2)
+    g = oracle.Grid(pts, bids, 2, np.float32(0.3))
+    nbh = oracle.Neighborhood(g, np.float32(0.3), pts[:25], bids[:25])
+    ids, n_out, c, h, f = nbh.original_neigh_ids, 25, 3, 4, 2
+    pdf = nbh.pdf_per_pair(0.2)
+    feat = rng.standard_normal((len(pts), c))
+    w, b = rng.standard_normal((3, h)), 0.1 * rng.standard_normal((1, h))
+    fw = rng.standard_normal((c * h, f))
+    pw1, pb1 = rng.standard_normal((1, 16)), 0.3 * rng.standard_normal((1, 16))
+    pw2, pb2 = np.abs(rng.standard_normal((16, 1))), np.full((1, 1), 0.5)
+    diff = (pts[ids[:, 0]] - pts[:25][ids[:, 1]]).astype(np.float64)
+    out, basis, cur, rel = L.point_conv(_t(diff), torch.tensor(ids).long(), n_out, _t(feat),
+                                        _t(pdf), _t(w), _t(b), _t(fw), _t(pw1), _t(pb1),
+                                        _t(pw2), _t(pb2), torch.relu)
+    starts = oracle.segment_starts(nbh.ranges)
+    for i in range(n_out):
+        lo, hi = int(starts[i]), int(nbh.ranges[i])
+        top = max([float(pdf[m]) for m in range(lo, hi)], default=1.0)
+        acc = np.zeros((c, h))
+        for m in range(lo, hi):
+            x = float(pdf[m]) / top
+            hid = [max(x * pw1[0, u] + pb1[0, u], 0.0) for u in range(16)]
+            y = math.fsum(hid[u] * pw2[u, 0] for u in range(16)) + pb2[0, 0]
+            assert abs(float(cur[m]) - y) <= 1e-12 * max(1.0, abs(y))
+            lat = [max(float(diff[m] @ w[:, q] + b[0, q]), 0.0) / y for q in range(h)]
+            acc += np.outer(feat[ids[m, 0]], lat)
+        np.testing.assert_allclose(out[i].numpy(), acc.reshape(-1) @ fw, rtol=1e-11, atol=1e-12)
