@@ -665,6 +665,16 @@ int mccnn_weight_grad_product(mccnn_stream_t stream, int64_t num_pts,
                               const float *y, void *workspace,
                               size_t workspace_bytes, float *out);
 
+/* The dense products of the layers (final product, projection gradient, final-weight
+ * gradient) run on the bf16 matrix pipe with float32 accuracy: every float32 operand is
+ * split into three bfloat16 parts and six of the nine part products are accumulated in
+ * float32 (the three left out are below 2^-24 of the term).  mccnn_set_split_products(0)
+ * switches the process back to the float32 matrix instructions (returns the previous
+ * setting); MCCNN_DENSE_FP32=1 in the environment does the same from the start.  No
+ * counterpart in the reference (TensorFlow picks its own GEMM). */
+int mccnn_set_split_products(int enabled);
+int mccnn_split_products_enabled(void);
+
 /* out[n, r] = sum_f x[n, f] * w[r, f]: the gradient of the projection entering a
  * layer's final product (x = output gradient [N, F], w = final weights [R, F],
  * out [N, R]); write-bound, each wavefront keeps its slice of w in registers.

@@ -9,6 +9,7 @@
 #include "common.h"
 #include "fill.h"
 #include "mfma.h"
+#include "split.h"
 
 namespace mccnn {
 
@@ -412,6 +413,8 @@ int tile_product_rows(int F) { return F % 128 == 0 ? 128 : 256; }
 
 int launch_tile_product(hipStream_t s, int64_t n, int R, const float *x, int F, const float *w,
                         bool w_transposed, const int *out_rows, float *out) {
+  if (w_transposed && split_products_enabled())
+    return launch_tile_split(s, n, R, x, F, w, out_rows, out);
   const int bn = F % 128 == 0 ? 128 : 64, bm = tile_product_rows(F);
   const dim3 block(kTileThreads), grid((unsigned)((n + bm - 1) / bm * (F / bn)));
   if (bn == 128) {
@@ -443,7 +446,11 @@ extern "C" int mccnn_weight_grad_product_supported(int num_rows_out, int num_col
 
 extern "C" size_t mccnn_weight_grad_product_workspace_bytes(int num_rows_out, int num_cols_out) {
   if (!tn_supported(num_rows_out, num_cols_out)) return 0;
-  return align256(sizeof(float) * (size_t)tn_slices(num_cols_out) * num_rows_out * num_cols_out);
+  int slices = tn_slices(num_cols_out);          // room for either arrangement of the slices
+  if (tn_split_supported(num_rows_out, num_cols_out) &&
+      tn_split_slices(num_rows_out, num_cols_out) > slices)
+    slices = tn_split_slices(num_rows_out, num_cols_out);
+  return align256(sizeof(float) * (size_t)slices * num_rows_out * num_cols_out);
 }
 
 extern "C" int mccnn_weight_grad_product(mccnn_stream_t stream, int64_t num_pts, int num_rows_out,
@@ -463,11 +470,21 @@ extern "C" int mccnn_weight_grad_product(mccnn_stream_t stream, int64_t num_pts,
   // slices of the point range, each reduced on its own: at least 128 points per slice, so that a
   // small cloud does not pay for summing a thousand empty partials and still fills the device
   const int C = num_rows_out, R = num_cols_out;
-  int slices = tn_slices(R);
+  const bool split = split_products_enabled() && tn_split_supported(C, R);
+  int slices = split ? tn_split_slices(C, R) : tn_slices(R);
   const int64_t by_size = (num_pts + 127) / 128;
   if (slices > by_size) slices = by_size < 1 ? 1 : (int)by_size;
   const dim3 grid((R / 256) * slices), block(256);
   float *partials = (float *)workspace;
+  const int64_t elems = (int64_t)C * R;
+  if (split) {
+    int rc = launch_tn_split(s, num_pts, C, x, R, y, slices, partials);
+    if (rc != MCCNN_OK) return rc;
+    hipLaunchKernelGGL(tn_reduce_kernel, dim3(blocks_for(elems, 256)), dim3(256), 0, s, elems,
+                       slices, partials, out);
+    MCCNN_LAUNCH_CHECK();
+    return MCCNN_OK;
+  }
   // 128 channels: operands staged through LDS (3.80 against 4.14 ms on [825 274, 128]^T x
   // [825 274, 2048]); up to 64 channels the direct kernel is as fast (1.18 / 1.21 ms on
   // [763 063, 64]^T x [763 063, 1024])
@@ -478,7 +495,6 @@ extern "C" int mccnn_weight_grad_product(mccnn_stream_t stream, int64_t num_pts,
     default: hipLaunchKernelGGL(tn_product_kernel<1>, grid, block, 0, s, num_pts, R, x, y, slices, partials); break;
   }
   MCCNN_LAUNCH_CHECK();
-  const int64_t elems = (int64_t)C * R;
   hipLaunchKernelGGL(tn_reduce_kernel, dim3(blocks_for(elems, 256)), dim3(256), 0, s, elems,
                      slices, partials, out);
   MCCNN_LAUNCH_CHECK();
@@ -500,6 +516,8 @@ extern "C" int mccnn_projection_grad_product(mccnn_stream_t stream, int64_t num_
   if (num_pts == 0) return MCCNN_OK;
   MCCNN_REQUIRE(x && w && out, "projection_grad_product received a null tensor");
   hipStream_t s = as_stream(stream);
+  if (split_products_enabled() && nt_split_supported(num_cols_in, num_cols_out))
+    return launch_nt_split(s, num_pts, num_cols_in, x, num_cols_out, w, out);
   const int F = num_cols_in, R = num_cols_out, groups = R / (64 * nt_cols(F));
   // one round of blocks: the kernel keeps 3 blocks of 4 wavefronts resident per compute unit
   // (136 registers), and a grid of exactly that many leaves no partly filled last round

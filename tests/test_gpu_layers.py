@@ -395,34 +395,63 @@ def test_local_and_global_pooling(oracle, c):
         normwise(t.grad.cpu().numpy(), gexp)
 
 
+def _wide_range(shape, gen):
+    """Standard-normal values times 10^U(-3, 3): operands whose magnitudes span six decades,
+    so that an operand split that loses low-order bits of small entries would show."""
+    return torch.randn(shape, device="cuda", generator=gen) * \
+        10.0 ** (6.0 * torch.rand(shape, device="cuda", generator=gen) - 3.0)
+
+
+@pytest.fixture(params=[True, False], ids=["split-bf16", "fp32-mfma"])
+def dense_mode(request):
+    """Runs a test once with the dense products on the bf16 matrix pipe (three-way operand
+    splits, the default) and once with the float32 matrix instructions."""
+    from tensorflow_graphics_point_clouds_amd import _lib
+    before = _lib.lib().mccnn_set_split_products(1 if request.param else 0)
+    yield request.param
+    _lib.lib().mccnn_set_split_products(before)
+
+
 @pytest.mark.parametrize("n,c,r", [(1, 16, 256), (4099, 64, 1024), (20000, 128, 512),
-                                   (777, 32, 2048), (0, 64, 256)])
-def test_weight_grad_product_matches_float64(n, c, r):
-    """x^T y with the long reduction over the points against float64 matmul
-    (tolerance 1e-5 of the largest entry)."""
+                                   (777, 32, 2048), (0, 64, 256), (100003, 64, 1024),
+                                   (50001, 128, 2048), (33, 128, 128), (257, 32, 256)])
+def test_weight_grad_product_matches_float64(n, c, r, dense_mode):
+    """x^T y with the long reduction over the points, elementwise against float64:
+    |got - expect| <= 1e-5 * (|x|^T |y|), on operands whose magnitudes span six decades;
+    equal bits on a second call (the partial sums are added in a fixed order)."""
     from tensorflow_graphics_point_clouds_amd import layers
     gen = torch.Generator(device="cuda").manual_seed(n + c)
-    x = torch.randn((n, c), device="cuda", generator=gen)
-    y = torch.randn((n, r), device="cuda", generator=gen)
-    got = layers._weight_grad_product(x, y).cpu().numpy().astype(np.float64)
-    expect = (x.double().t() @ y.double()).cpu().numpy()
+    x = _wide_range((n, c), gen)
+    y = _wide_range((n, r), gen)
+    got = layers._weight_grad_product(x, y)
     assert got.shape == (c, r)
-    assert np.abs(got - expect).max() <= 1e-5 * max(1.0, np.abs(expect).max())
+    assert torch.equal(got, layers._weight_grad_product(x, y))
+    expect = x.double().t() @ y.double()
+    mag = x.double().abs().t() @ y.double().abs()
+    err = (got.double() - expect).abs()
+    assert bool((err <= 1e-5 * mag).all()), float((err / mag.clamp(min=1e-300)).max())
 
 
 @pytest.mark.parametrize("n,f,r", [(1, 16, 256), (4099, 64, 1024), (20000, 32, 512), (0, 64, 256),
                                    (4099, 128, 1024), (3001, 128, 2048), (1500, 256, 4096),
-                                   (17, 256, 64), (33, 128, 128)])
-def test_projection_grad_product_matches_float64(n, f, r):
+                                   (17, 256, 64), (33, 128, 128), (31, 64, 256), (70001, 64, 1024),
+                                   (5000, 32, 1024), (65, 128, 256)])
+def test_projection_grad_product_matches_float64(n, f, r, dense_mode):
+    """x w^T elementwise against float64: |got - expect| <= 1e-5 * (|x| |w|^T), on operands
+    whose magnitudes span six decades; equal bits on a second call."""
     from tensorflow_graphics_point_clouds_amd import layers
     gen = torch.Generator(device="cuda").manual_seed(n + f)
-    x = torch.randn((n, f), device="cuda", generator=gen)
-    w = torch.randn((r, f), device="cuda", generator=gen)
-    got = layers._projection_grad_product(x, w).cpu().numpy().astype(np.float64)
-    expect = (x.double() @ w.double().t()).cpu().numpy()
+    x = _wide_range((n, f), gen)
+    w = _wide_range((r, f), gen)
+    got = layers._projection_grad_product(x, w)
     assert got.shape == (n, r)
-    if n:
-        assert np.abs(got - expect).max() <= 1e-5 * np.abs(expect).max()
+    assert torch.equal(got, layers._projection_grad_product(x, w))
+    expect = x.double() @ w.double().t()
+    mag = x.double().abs() @ w.double().abs().t()
+    err = (got.double() - expect).abs()
+    assert bool((err <= 1e-5 * mag).all()), float((err / mag).max()) if n else 0.0
+    if n:       # the split path is as accurate as float32 accumulation, far inside the bound
+        assert float((err / mag).max()) <= 2e-6
 
 
 @pytest.mark.parametrize("n,r,f", [(1, 256, 16), (15, 256, 128), (4099, 1024, 64), (20000, 512, 128),
