@@ -682,10 +682,13 @@ def main():
     ap.add_argument("--no-isolated", action="store_true", help="skip the isolated basis_proj case")
     ap.add_argument("--no-sweep", action="store_true",
                     help="skip the other two radii (0.02, 0.06) of the dense case")
+    ap.add_argument("--no-small-configs", action="store_true",
+                    help="skip configurations 1 (2 x 1024 points, forward) and 2 (16 x 1024 "
+                         "points, three-level network, fwd+bwd): they launch the layer's kernels "
+                         "on tiny shapes and blur the per-kernel averages of a profile")
     ap.add_argument("--extra-configs", action="store_true",
-                    help="also time configurations 1 (2 x 1024 points, forward) and 2 (16 x 1024 "
-                         "points, three-level network, fwd+bwd) and PointConv on the scene-scale "
-                         "clouds")
+                    help="also time PointConv on the scene-scale clouds and the atomic-free "
+                         "variant of the basis_proj gradients")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run a 1 GiB device copy three times (reference point for the "
                          "FETCH_SIZE / WRITE_SIZE counters) and exit")
@@ -735,7 +738,8 @@ def main():
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
-    _lib.start_timing()
+    # the timed region: exactly `steps` steps with nothing recorded inside a step (one event
+    # after each step gives the median and the minimum)
     marks = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
     t0 = time.perf_counter()
     marks[0].record()
@@ -744,9 +748,17 @@ def main():
         marks[i + 1].record()
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
-    per_op = {k.replace("_ordered", ""): v for k, v in _lib.collect_timing().items()}
     ms_per_step = dt * 1e3 / args.steps
     step_ms = sorted(marks[i].elapsed_time(marks[i + 1]) for i in range(args.steps))
+    # a second region of the same length with a pair of events around every op call: the
+    # per-op times (about 14 event records per step)
+    _lib.start_timing()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_per_step_instrumented = (time.perf_counter() - t0) * 1e3 / args.steps
+    per_op = {k.replace("_ordered", ""): v for k, v in _lib.collect_timing().items()}
 
     ops = {}
     for name, vals in per_op.items():
@@ -768,7 +780,7 @@ def main():
         if name in ("permute_rows", "gather_rows"):
             ops[name].update(GBps_copy=round(8 * N * C * calls / ms / 1e6, 1))
     kernel_ms = sum(v["ms"] for v in ops.values())
-    ops["host_gaps_and_small_kernels"] = {"ms": round(ms_per_step - kernel_ms, 4)}
+    ops["host_gaps_and_small_kernels"] = {"ms": round(ms_per_step_instrumented - kernel_ms, 4)}
     dominant = max((n for n in ops if "GBps" in ops[n]), key=lambda n: ops[n]["ms"])
     launch_ms = ops[dominant]["ms"] / ops[dominant]["calls_per_step"]
     traffic, traffic_source = (measured_traffic(dominant, "config3_C%d_K%d" % (C, K))
@@ -792,13 +804,24 @@ def main():
                     "matrix peak"}
     if traffic:
         roof["traffic_frac"] = round(traffic / (launch_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
+    # the step as a whole against the fp32 matrix peak: four dense products [N, C*K] x
+    # [C*K, C_out] (forward, feature gradient, projection gradient, final-weight gradient) and
+    # three projection-shaped contractions over the pairs
+    step_flops = 4 * 2.0 * N * C * K * CO + 3 * 2.0 * M * C * K
+    roof["step_flops"] = step_flops
+    roof["step_matrix_TFLOPs"] = round(step_flops / ms_per_step / 1e9, 1)
+    roof["step_matrix_frac"] = round(step_flops / ms_per_step / 1e9 / FP32_MATRIX_PEAK_TFLOPS, 4)
 
     result = {
         "metric": "MCConv layer fwd+bwd points/sec", "value": N / (ms_per_step * 1e-3),
         "unit": "points/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "ms_per_step_median": step_ms[len(step_ms) // 2],
-        "ms_per_step_min": step_ms[0], "higher_is_better": True, "scaling": "weak",
+        "ms_per_step_min": step_ms[0], "ms_per_step_instrumented": ms_per_step_instrumented,
+        "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "dense_products": ("bf16 matrix pipe, three-way operand splits, float32 accumulation "
+                           "(float32-accurate)" if _lib.lib().mccnn_split_products_enabled()
+                           else "float32 matrix instructions"),
         "config": {"workload": "config 3: 8 clustered clouds of 50k-150k points (seed 1003), "
                                "MCConv 64->64, 16-unit kernel MLP, radius 0.15, fp32, fwd+bwd, "
                                "neighbourhood and densities prebuilt",
@@ -824,11 +847,14 @@ def main():
         result["per_op_dense_case"] = per_op_times(torch, pc, layers, synthetic, _lib)
         torch.cuda.empty_cache()
         result["kpconv_config5"] = kpconv_config5(torch, pc, layers, synthetic, _lib)
-    if args.extra_configs:
-        # (not in the default run: these launch the layer's kernels on tiny shapes, which
-        # would blur the per-kernel averages of a profile of the default command)
-        result["config2_network"] = config2_network(torch, pc, layers, synthetic)
+    if not args.no_small_configs and args.scale == 1.0:
+        # the two small configurations, bound by launches and host round trips rather than bytes
+        # (profile commands pass --no-small-configs: the layer's kernels on these tiny shapes
+        # would blur the per-kernel averages)
+        torch.cuda.empty_cache()
         result["config1_forward"] = config1_forward(torch, pc, layers, synthetic)
+        result["config2_network"] = config2_network(torch, pc, layers, synthetic)
+    if args.extra_configs:
         result["pointconv_config3"] = pointconv_config3(torch, pc, layers, synthetic, _lib)
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(synthetic)

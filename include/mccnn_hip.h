@@ -201,10 +201,14 @@ int mccnn_compute_pdf(mccnn_stream_t stream, int64_t num_pts, int num_dims,
                       const float *inv_radii, int mode, float *pdf_out);
 
 /* ComputePdfPtGrads: compute_pdf/cc/ops/compute_pdf_ops.cpp:163-259.
- * pt_grads_out [num_pts, D] = d(sum_i pdf_grads_i * pdf_i) / d(points).  Valid for any
- * pair table; where the reverse of a pair is in the table too (always, in an
- * untruncated self-neighbourhood) its term is gathered instead of scattered, so
- * atomics are used only for pairs without a reverse. */
+ * pt_grads_out [num_pts, D] = d(sum_i pdf_grads_i * pdf_i) / d(points).  The table must be
+ * a self-neighbourhood (centre c is point c: num_samples == num_pts, as the op requires,
+ * compute_pdf_ops.cpp:205-207) in which no pair occurs twice -- what find_neighbors writes,
+ * truncated by max_neighs or not, in any order inside a centre.  Where the reverse of a
+ * pair is in the table too (always, in an untruncated self-neighbourhood) its term is
+ * gathered instead of scattered, so atomics are used only for pairs without a reverse.
+ * (A repeated pair would be gathered once per occurrence of its reverse; the reference's
+ * atomics weight every occurrence.) */
 int mccnn_compute_pdf_pt_grads(mccnn_stream_t stream, int64_t num_pts,
                                int num_dims, const float *points,
                                int64_t num_neighbors, int neighbors_rank,
@@ -664,6 +668,26 @@ int mccnn_weight_grad_product(mccnn_stream_t stream, int64_t num_pts,
                               int num_rows_out, const float *x, int num_cols_out,
                               const float *y, void *workspace,
                               size_t workspace_bytes, float *out);
+
+/* One layer of a kernel MLP per neighbour pair: y[m, :] = act(x[m, :] * weights + biases)
+ * for x [num_rows, num_cols_in], weights [num_cols_in, num_cols_out] (both widths 1..64),
+ * biases [num_cols_out] or NULL; activation -1 (none) or MCCNN_ACT_*.  The reference
+ * evaluates its kernel MLPs with tf.matmul on [M, .] tensors (MCConv.py:163-168,
+ * PointConv.py:168-190); these are the same layers as memory-bound kernels, used for kernel
+ * MLPs of several layers and where the kernel input stays differentiable.
+ * _grads: from the layer's output y and the upstream gradient dy, dx [num_rows,
+ * num_cols_in] (NULL to skip), dweights and dbiases (NULL to skip); partial sums per slice
+ * of the rows in the workspace, added in a fixed order. */
+int mccnn_pair_dense(mccnn_stream_t stream, int64_t num_rows, int num_cols_in,
+                     const float *x, int num_cols_out, const float *weights,
+                     const float *biases, int activation, float *y);
+size_t mccnn_pair_dense_grads_workspace_bytes(int64_t num_rows, int num_cols_in,
+                                              int num_cols_out);
+int mccnn_pair_dense_grads(mccnn_stream_t stream, int64_t num_rows, int num_cols_in,
+                           const float *x, int num_cols_out, const float *weights,
+                           const float *y, const float *dy, int activation,
+                           void *workspace, size_t workspace_bytes, float *dx,
+                           float *dweights, float *dbiases);
 
 /* The dense products of the layers (final product, projection gradient, final-weight
  * gradient) run on the bf16 matrix pipe with float32 accuracy: every float32 operand is

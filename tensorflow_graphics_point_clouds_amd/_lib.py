@@ -47,6 +47,7 @@ def lib():
                      "mccnn_find_neighbors_workspace_bytes",
                      "mccnn_mc_basis_grads_workspace_bytes",
                      "mccnn_mc_conv_project_grads_workspace_bytes",
+                     "mccnn_pair_dense_grads_workspace_bytes",
                      "mccnn_pointconv_density_grads_workspace_bytes",
                      "mccnn_reorder_neighbors_workspace_bytes",
                      "mccnn_sampling_workspace_bytes",

@@ -189,7 +189,7 @@ __global__ void __launch_bounds__(kNbrThreads) nbr_visit_kernel(
   int found = 0;                                   // kFill: slots used so far
   int64_t start = 0;
   if (kFill) start = c > 0 ? ends[c - 1] : 0;
-  // the slices of the centre, 16 at a time: lane `sub` fetches one, the group then
+  // the slices of the centre, kGroup at a time: lane `sub` fetches one, the group then
   // takes them in turn (one round trip to memory instead of one per slice)
   for (int r0 = 0; r0 < R; r0 += kGroup) {
     const int2 mine = r0 + sub < R ? ranges[c * R + r0 + sub] : make_int2(0, 0);

@@ -86,7 +86,9 @@ __global__ void __launch_bounds__(kPdfThreads) compute_pdf_kernel(
 // not (a list cut by max_neighs, a hand-made table), c sends the term to grad[j] with
 // an atomic.  Lists written by find_neighbors ascend by point index, so the look-up is a
 // binary search; a miss is confirmed by a linear scan, which keeps tables in any order
-// correct.  Every centre adds its register sum once (grads are zero-filled first).  An
+// correct.  Preconditions: centre c is point c (the op requires num_samples == num_pts)
+// and no pair occurs twice in the table.  Every centre adds its register sum once (grads
+// are zero-filled first).  An
 // untruncated self-neighbourhood takes no scatter at all: 41.8 M pairs in 1.06 ms where
 // scattering every pair's term with atomics takes 3.4 ms.
 template <int D>

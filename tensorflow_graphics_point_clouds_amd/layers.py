@@ -3,7 +3,9 @@ signatures of the reference's layers (pylib/pc/layers/MCConv.py, KPConv.py,
 Pooling.py).  Per-pair basis evaluation, basis projection, pooling and all
 their gradients are kernels of libmccnn_hip.so, and so are the dense
 [N, C*K] x [C*K, C_out] product and its two gradient products for channel
-counts that are multiples of 16 (others fall back to torch.matmul)."""
+counts that are multiples of 16 (other shapes of the dense products fall back to
+torch.matmul inside `_final_product`, `_weight_grad_product` and
+`_projection_grad_product`, nowhere else)."""
 import math
 
 import numpy as np
@@ -220,6 +222,76 @@ def _final_product(x, w):
 _TILED_ABOVE = 65536      # weights that fit the registers of a block of wavefronts
 
 
+class _DenseProduct(torch.autograd.Function):
+    """x w for x [N, R], w [R, F] on the library's dense kernels, differentiable in both:
+    dx = dout w^T (projection-gradient product), dw = x^T dout (final-weight-gradient
+    product); shapes the kernels do not cover fall back to torch inside the three helpers."""
+
+    @staticmethod
+    def forward(ctx, x, w):
+        ctx.save_for_backward(x, w)
+        return _final_product(x.contiguous(), w)
+
+    @staticmethod
+    def backward(ctx, dout):
+        x, w = ctx.saved_tensors
+        dout = dout.contiguous()
+        dx = _projection_grad_product(dout, w.contiguous()) if ctx.needs_input_grad[0] else None
+        # x^T dout with the reduction over the rows: the kernel takes the narrow operand first
+        dw = None
+        if ctx.needs_input_grad[1]:
+            if _lib.lib().mccnn_weight_grad_product_supported(cint(dout.shape[1]), cint(x.shape[1])):
+                dw = _weight_grad_product(dout, x.contiguous()).t()
+            else:
+                dw = _weight_grad_product(x.contiguous(), dout)
+        return dx, dw
+
+
+def _dense_product(x, w):
+    return _DenseProduct.apply(x, w)
+
+
+class _PairDense(torch.autograd.Function):
+    """One layer of a kernel MLP per neighbour pair, y = act(x w + b) for x [M, I] with
+    I, O <= 64 (MCConv.py:163-168, PointConv.py:168-190), forward and all gradients on the
+    library's memory-bound kernels (mccnn_pair_dense, mccnn_pair_dense_grads)."""
+
+    @staticmethod
+    def forward(ctx, x, w, b, act):
+        x, w = x.contiguous(), w.contiguous()
+        ctx.bias_shape = None if b is None else tuple(b.shape)
+        b = None if b is None else b.reshape(-1).contiguous()
+        y = torch.empty((x.shape[0], w.shape[1]), dtype=_F32, device=x.device)
+        _lib.call("pair_dense", stream(), i64(x.shape[0]), cint(w.shape[0]), ptr(x, _F32),
+                  cint(w.shape[1]), ptr(w, _F32), ptr(b, _F32), cint(act), ptr(y))
+        ctx.save_for_backward(x, w, y)
+        ctx.act = act
+        return y
+
+    @staticmethod
+    def backward(ctx, dy):
+        x, w, y = ctx.saved_tensors
+        rows, i, o = x.shape[0], w.shape[0], w.shape[1]
+        L = _lib.lib()
+        ws = _lib.workspace(L.mccnn_pair_dense_grads_workspace_bytes(i64(rows), cint(i), cint(o)),
+                            x.device)
+        dx = torch.empty_like(x) if ctx.needs_input_grad[0] else None
+        dw = torch.empty_like(w)
+        db = torch.empty(o, dtype=_F32, device=x.device) if ctx.bias_shape is not None else None
+        _lib.call("pair_dense_grads", stream(), i64(rows), cint(i), ptr(x, _F32), cint(o),
+                  ptr(w, _F32), ptr(y, _F32), ptr(dy.contiguous(), _F32), cint(ctx.act), ptr(ws),
+                  _lib.csize(ws.numel()), ptr(dx), ptr(dw), ptr(db))
+        return dx, dw, None if db is None else db.reshape(ctx.bias_shape), None
+
+
+def _pair_dense(x, w, b, act):
+    """act(x w + b) per pair; `act` -1 for none.  Widths beyond 64 take torch."""
+    if w.shape[0] > 64 or w.shape[1] > 64:
+        z = x @ w if b is None else x @ w + b.reshape(1, -1)
+        return z if act < 0 else _activate(z, act)
+    return _PairDense.apply(x, w, b, act)
+
+
 def _dense_final_weights(final_weights, c):
     """[L, C*H, G] per-MLP blocks -> dense [C*(L*H), L*G] with zero off-diagonal blocks."""
     l, ch, g = final_weights.shape
@@ -397,19 +469,25 @@ class MCConv(torch.nn.Module):
         ids = neighborhood._original_neigh_ids.long()
         l, c, h = self._num_mlps, self._num_features_in, self._hidden
         diff = (point_cloud_in._points[ids[:, 0]] - point_cloud_out._points[ids[:, 1]]) / radii
-        cur = diff.unsqueeze(0).expand(l, -1, -1)
         layers_w = [self.weights] + list(self.deep_weights)
         layers_b = [self.biases] + list(self.deep_biases)
-        for w, b in zip(layers_w, layers_b):
-            cur = _activate(torch.bmm(cur, w) + b, self._act)
+        columns = []
+        for mlp in range(l):             # every kernel MLP is a chain of per-pair layers
+            cur = diff
+            for w, b in zip(layers_w, layers_b):
+                cur = _pair_dense(cur, w[mlp], b[mlp], self._act)
+            columns.append(cur)
         pdf = neighborhood.get_pdf() if pdf is None else pdf
-        basis = cur.permute(1, 0, 2).reshape(ids.shape[0], l * h) / pdf.reshape(-1, 1)
+        basis = (columns[0] if l == 1 else torch.cat(columns, dim=1)) / pdf.reshape(-1, 1)
         proj = tfg_custom_ops.basis_proj(basis.contiguous(), features.contiguous(),
                                          neighborhood._original_neigh_ids,
                                          neighborhood._samples_neigh_ranges)
         n = proj.shape[0]
+        if l == 1:
+            return _dense_product(proj.reshape(n, c * h), self.final_weights[0])
         p = proj.reshape(n, c, l, h).permute(2, 0, 1, 3).reshape(l, n, c * h)
-        return torch.bmm(p, self.final_weights).permute(1, 0, 2).reshape(n, -1)
+        return torch.cat([_dense_product(p[mlp].contiguous(), self.final_weights[mlp])
+                          for mlp in range(l)], dim=1)
 
     def _convolve_on_view(self, features, neighborhood, radii, biases, k):
         """The fused path on the grid-ordered view; channel counts it does not cover
@@ -511,9 +589,10 @@ class MCConv(torch.nn.Module):
                                              neighborhood._centre_order, transposed)
         n, c, l, h = proj.shape[0], self._num_features_in, self._num_mlps, self._hidden
         if l == 1:
-            return proj.reshape(n, c * h) @ self.final_weights[0]
+            return _dense_product(proj.reshape(n, c * h), self.final_weights[0])
         p = proj.reshape(n, c, l, h).permute(2, 0, 1, 3).reshape(l, n, c * h)
-        return torch.bmm(p, self.final_weights).permute(1, 0, 2).reshape(n, -1)
+        return torch.cat([_dense_product(p[mlp].contiguous(), self.final_weights[mlp])
+                          for mlp in range(l)], dim=1)
 
 
 def _differentiable_pdf(neighborhood, bandwidth):
@@ -750,7 +829,7 @@ class PointConv(torch.nn.Module):
             pdf = _differentiable_pdf(neighborhood, bandwidth)
             diff = point_cloud_in._points[ids[:, 0].long()] - \
                 point_cloud_out._points[ids[:, 1].long()]
-            hidden = _activate(diff @ self.weights + self.biases, self._act)
+            hidden = _pair_dense(diff, self.weights, self.biases, self._act)
         else:
             out = self._convolve_on_view(features, neighborhood, bandwidth)
             if out is not None:
@@ -768,11 +847,11 @@ class PointConv(torch.nn.Module):
         max_pdf = torch.zeros(n_out, dtype=_F32, device=dev).scatter_reduce(
             0, centre, pdf, "amax", include_self=False)
         rel = (pdf / max_pdf[centre]).reshape(-1, 1)
-        cur = torch.relu(rel @ self.pdf_weights_1 + self.pdf_biases_1)
-        cur = cur @ self.pdf_weights_2 + self.pdf_biases_2
+        cur = _pair_dense(rel, self.pdf_weights_1, self.pdf_biases_1, 0)
+        cur = _pair_dense(cur, self.pdf_weights_2, self.pdf_biases_2, -1)
         basis = hidden / cur
         proj = tfg_custom_ops.basis_proj(basis, features.contiguous(), ids, ranges)
-        return proj.reshape(n_out, -1) @ self.final_weights
+        return _dense_product(proj.reshape(n_out, -1), self.final_weights)
 
 
 def _padded_basis_count(num_kernel_points):
@@ -1113,12 +1192,12 @@ class KPConv(torch.nn.Module):
                                                   self._kind, sigma, False)[:, :cols]
             else:
                 rigid = _KPBasis.apply(None, *geometry, k, self._kind, sigma)
-                offsets = project(rigid).reshape(-1, c * k) @ w_off
+                offsets = _dense_product(project(rigid).reshape(-1, c * k), w_off)
             offsets = offsets.reshape(-1, kp, d).contiguous()
         self._last = (offsets, geometry, sigma)
         self.last_offsets = offsets
         basis = _KPBasis.apply(offsets, *geometry, k, self._kind, sigma)
-        return project(basis).reshape(-1, c * k) @ self._padded(self.weights)
+        return _dense_product(project(basis).reshape(-1, c * k), self._padded(self.weights))
 
     def _convolve_deformed_on_view(self, features, neighborhood, radii, sigma):
         """KPConv.py:317-392 on the grid-ordered view: a rigid convolution predicts the
@@ -1177,7 +1256,7 @@ class KPConv(torch.nn.Module):
 
         offsets = None
         if self.deformable:
-            offsets = (project(correlation(None)) @ self._padded(self.offset_weights))
+            offsets = _dense_product(project(correlation(None)), self._padded(self.offset_weights))
             offsets = offsets.reshape(-1, kp, d)
         self._last = None
         self.last_offsets = offsets
@@ -1185,7 +1264,7 @@ class KPConv(torch.nn.Module):
             geometry = (point_cloud_in._points.detach(), point_cloud_out._points.detach(), ids,
                         ranges, pc._reciprocal(radii), self._kernel_points)
             self._last = (offsets, geometry, sigma)
-        return project(correlation(offsets)) @ self._padded(self.weights)
+        return _dense_product(project(correlation(offsets)), self._padded(self.weights))
 
     def regularization_loss(self):
         """Fitting + repulsive loss of the last deformable call (KPConv.py:394-429)."""

@@ -27,8 +27,17 @@ class KDEMode(enum.Enum):
     no_pdf = 2
 
 
-_vector_cache = {}
-_vector_values = {}
+_vector_cache = {}       # (bytes of the host values, dims, device) -> shared device vector
+_shared = {}             # id of a shared vector -> (the vector itself, its host values)
+_derived_cache = {}      # (operation, id of a shared vector) -> shared result
+
+
+def _share(t, values):
+    """Registers a small read-only device vector under its own identity.  The entry keeps
+    the tensor alive, so the id (and the memory behind it) cannot be handed to another
+    tensor while the entry exists."""
+    _shared[id(t)] = (t, values)
+    return t
 
 
 def _as_vector(value, dims, device):
@@ -50,26 +59,21 @@ def _as_vector(value, dims, device):
             t = t.repeat(dims)
         t = t.to(device).contiguous()
         if len(_vector_cache) < 4096:
-            _vector_cache[key] = t
-            _vector_values[t.data_ptr()] = tuple(float(v) for v in t.tolist())
+            _vector_cache[key] = _share(t, tuple(float(v) for v in t.tolist()))
     return t
-
-
-_derived_cache = {}      # (operation, address of a shared vector) -> shared result
-_shared_vectors = set()  # addresses of the derived vectors themselves
 
 
 def _derived(op, fn, t):
     """fn(t) for a small device vector; the vectors `_as_vector` keeps (shared,
     read-only) and what was derived from them get the result once instead of one
-    kernel launch per use."""
-    key = t.data_ptr()
-    if key not in _vector_values and key not in _shared_vectors:
+    kernel launch per use.  Shared vectors are recognised by object identity, never by
+    address: a caller's own tensor always takes fn(t)."""
+    entry = _shared.get(id(t))
+    if entry is None or entry[0] is not t:
         return fn(t)
-    r = _derived_cache.get((op, key))
+    r = _derived_cache.get((op, id(t)))
     if r is None:
-        r = _derived_cache[(op, key)] = fn(t)
-        _shared_vectors.add(r.data_ptr())
+        r = _derived_cache[(op, id(t))] = _share(fn(t), None)
     return r
 
 
@@ -84,9 +88,11 @@ def _negative(t):
 def _host_values(t):
     """The entries of a small device vector as a tuple of floats; no device round
     trip for the vectors `_as_vector` keeps."""
-    known = _vector_values.get(t.data_ptr())
-    return known if known is not None and len(known) == t.numel() else \
-        tuple(float(v) for v in t.tolist())
+    entry = _shared.get(id(t))
+    if entry is not None and entry[0] is t and entry[1] is not None and \
+            len(entry[1]) == t.numel():
+        return entry[1]
+    return tuple(float(v) for v in t.tolist())
 
 
 class AABB:

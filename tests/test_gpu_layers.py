@@ -832,11 +832,62 @@ def test_mcconv_step_replays_from_a_captured_graph():
             p.grad = g
 
 
-@pytest.mark.parametrize("mlp_size,num_mlps,act", [([8, 16], 1, "relu"), ([4, 8, 8], 2, "elu")])
+def _slope(act, z):
+    if act == "relu":
+        return (z > 0).double()
+    if act == "leaky_relu":
+        return torch.where(z > 0, 1.0, 0.2)
+    if act == "elu":
+        return torch.where(z > 0, torch.ones_like(z), torch.exp(z))
+    return torch.ones_like(z)
+
+
+@pytest.mark.parametrize("rows,i,o,act", [(1, 3, 8, "relu"), (70001, 3, 16, "leaky_relu"),
+                                          (5000, 8, 16, "elu"), (333, 16, 64, "relu"),
+                                          (40000, 64, 64, "elu"), (129, 1, 16, "relu"),
+                                          (2049, 16, 1, None), (0, 3, 8, "relu"),
+                                          (10000, 5, 49, "leaky_relu")])
+def test_pair_dense_layer_matches_float64(rows, i, o, act):
+    """One per-pair layer of a kernel MLP, y = act(x w + b), and its three gradients against
+    float64 autograd, elementwise: |got - expect| <= 1e-5 * mag with mag the same sum over
+    the absolute values of its terms; the weight and bias gradients (sums over all rows,
+    added in a fixed order) come out bit-equal on a second call."""
+    from tensorflow_graphics_point_clouds_amd import layers
+    gen = torch.Generator(device="cuda").manual_seed(rows + i + o)
+    x = torch.randn((rows, i), device="cuda", generator=gen).requires_grad_(True)
+    w = (torch.randn((i, o), device="cuda", generator=gen) / max(i, 1) ** 0.5).requires_grad_(True)
+    b = (0.3 * torch.randn((1, o), device="cuda", generator=gen)).requires_grad_(True)
+    up = torch.randn((rows, o), device="cuda", generator=gen)
+    code = {None: -1, "relu": 0, "leaky_relu": 1, "elu": 2}[act]
+    y = layers._pair_dense(x, w, b, code)
+    grads = torch.autograd.grad((y * up).sum(), [x, w, b])
+    again = torch.autograd.grad((layers._pair_dense(x, w, b, code) * up).sum(), [x, w, b])
+    for a, c in zip(grads, again):
+        assert torch.equal(a, c)
+    xd, wd, bd = (t.detach().double().requires_grad_(True) for t in (x, w, b))
+    z = xd @ wd + bd
+    ref = z if act is None else _T_ACT[act](z)
+    mag_z = xd.detach().abs() @ wd.detach().abs() + bd.detach().abs()
+    slope = _slope(act, z.detach())
+    assert bool(((y.double() - ref).abs() <= 1e-5 * (slope * mag_z + ref.detach().abs()) + 1e-30).all())
+    want = torch.autograd.grad((ref * up.double()).sum(), [xd, wd, bd])
+    dz = (up.double() * slope).abs()
+    mags = (dz @ wd.detach().abs().t(), xd.detach().abs().t() @ dz, dz.sum(0, keepdim=True))
+    for got, expect, mag, what in zip(grads, want, mags, ("dx", "dw", "db")):
+        err = (got.double() - expect).abs()
+        assert bool((err <= 1e-5 * mag + 1e-30).all()), what
+
+
+@pytest.mark.parametrize("mlp_size,num_mlps,act", [([8, 16], 1, "relu"), ([4, 8, 8], 2, "elu"),
+                                                   ([16, 32], 1, "leaky_relu")])
 def test_mcconv_with_deeper_kernel_mlp(oracle, mlp_size, num_mlps, act):
     """Kernel MLPs of several layers (MCConv.py:163-171): forward and all gradients
     against float64 autograd of the same expressions on the oracle's pairs and
-    densities."""
+    densities.  Elementwise: |got - expect| <= 1e-5 * mag, where mag comes from a second
+    chain built on the absolute values of every operand -- through an activation a
+    magnitude m of the pre-activation becomes slope * m + |act(z)| (the slope carries the
+    error of z, the second term the rounding of the activation itself) -- and, for the
+    gradients, from autograd of that chain with the upstream |up|."""
     from tensorflow_graphics_point_clouds_amd import layers, pc
     rng = np.random.default_rng(len(mlp_size))
     batch, radius, c_in, c_out = 2, 0.2, 8, 12
@@ -858,23 +909,37 @@ def test_mcconv_with_deeper_kernel_mlp(oracle, mlp_size, num_mlps, act):
     params = [conv.weights] + list(conv.deep_weights) + [conv.biases] + list(conv.deep_biases) + \
         [conv.final_weights]
     ref = [p.detach().cpu().double().requires_grad_(True) for p in params]
+    mref = [p.detach().cpu().double().abs().requires_grad_(True) for p in params]
     depth = len(mlp_size)
     tf = torch.tensor(feat.astype(np.float64), requires_grad=True)
-    cur = torch.tensor(((pts[ids[:, 0]] - ctr[ids[:, 1]]) / np.float32(radius)).astype(np.float64))
-    cur = cur.unsqueeze(0).expand(num_mlps, -1, -1)
-    for w, b in zip(ref[:depth], ref[depth:2 * depth]):
-        cur = _T_ACT[act](torch.bmm(cur, w) + b)
+    mf = torch.tensor(np.abs(feat).astype(np.float64), requires_grad=True)
+    diff = torch.tensor(((pts[ids[:, 0]] - ctr[ids[:, 1]]) / np.float32(radius)).astype(np.float64))
+    cur = diff.unsqueeze(0).expand(num_mlps, -1, -1)
+    mag = cur.abs()
+    for w, b, mw, mb in zip(ref[:depth], ref[depth:2 * depth], mref[:depth], mref[depth:2 * depth]):
+        z = torch.bmm(cur, w) + b
+        cur = _T_ACT[act](z)
+        mag = _slope(act, z.detach()) * (torch.bmm(mag, mw) + mb) + cur.detach().abs()
     h = mlp_size[-1]
-    bas = cur.permute(1, 0, 2).reshape(len(ids), -1) / torch.tensor(pdf.astype(np.float64)).reshape(-1, 1)
-    per_pair = tf[ids[:, 0]][:, :, None] * bas[:, None, :]
-    pj = torch.zeros(len(ctr), c_in, num_mlps * h, dtype=torch.float64).index_add(0, ids[:, 1], per_pair)
-    pj = pj.reshape(-1, c_in, num_mlps, h).permute(2, 0, 1, 3).reshape(num_mlps, -1, c_in * h)
-    expect = torch.bmm(pj, ref[-1]).permute(1, 0, 2).reshape(len(ctr), -1)
-    normwise(out.detach().cpu().numpy(), expect.detach().numpy(), tol=1e-5)
-    (expect * torch.tensor(up.astype(np.float64))).sum().backward()
-    normwise(tfeat.grad.cpu().numpy(), tf.grad.numpy(), tol=1e-5)
-    for p, r in zip(params, ref):
-        normwise(p.grad.cpu().numpy(), r.grad.numpy(), tol=1e-5)
+    tpdf = torch.tensor(pdf.astype(np.float64)).reshape(-1, 1)
+
+    def rest(hidden, f, final):
+        bas = hidden.permute(1, 0, 2).reshape(len(ids), -1) / tpdf
+        per_pair = f[ids[:, 0]][:, :, None] * bas[:, None, :]
+        pj = torch.zeros(len(ctr), c_in, num_mlps * h, dtype=torch.float64).index_add(
+            0, ids[:, 1], per_pair)
+        pj = pj.reshape(-1, c_in, num_mlps, h).permute(2, 0, 1, 3).reshape(num_mlps, -1, c_in * h)
+        return torch.bmm(pj, final).permute(1, 0, 2).reshape(len(ctr), -1)
+
+    expect = rest(cur, tf, ref[-1])
+    bound = rest(mag, mf, mref[-1])
+    elementwise(out.detach().cpu().numpy(), expect.detach().numpy(), bound.detach().numpy())
+    tup = torch.tensor(up.astype(np.float64))
+    want = torch.autograd.grad((expect * tup).sum(), [tf] + ref)
+    mags = torch.autograd.grad((bound * tup.abs()).sum(), [mf] + mref)
+    got = [tfeat.grad] + [p.grad for p in params]
+    for g, e, m in zip(got, want, mags):
+        elementwise(g.cpu().numpy(), e.numpy(), m.numpy())
 
 
 def test_mcconv_gradient_with_respect_to_points(oracle):
