@@ -621,8 +621,9 @@ def isolated_basis_proj(torch, pc, synthetic, tfg, _lib, radius=0.04, steps=5, g
             # over kernel time; with the pairs in the caller's order those rows do come from
             # HBM (counter traffic 0.99x this figure), in grid order L2 serves most of them
             entry["operand_frac_hbm_peak"] = round(by / ms / 1e6 / HBM_PEAK_GBS, 4)
-            traffic, source = measured_traffic(name, "dense_C%d_K%d%s" % (C, K, tag)) \
-                if radius == 0.04 else (None, "no counter run at this radius")
+            # (the workload tag of the counter summary: r = 0.04 carries no radius suffix)
+            workload = "dense_C%d_K%d%s%s" % (C, K, tag, "" if radius == 0.04 else "_r%.2f" % radius)
+            traffic, source = measured_traffic(name, workload)
             entry["traffic"], entry["traffic_source"] = traffic, source
             if traffic:
                 entry["traffic_frac"] = round(traffic / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
@@ -689,6 +690,9 @@ def main():
     ap.add_argument("--extra-configs", action="store_true",
                     help="also time PointConv on the scene-scale clouds and the atomic-free "
                          "variant of the basis_proj gradients")
+    ap.add_argument("--only-dense-radius", type=float, default=None,
+                    help="only run the isolated basis_proj case at this radius and exit (counter "
+                         "runs for the radii of the sweep)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run a 1 GiB device copy three times (reference point for the "
                          "FETCH_SIZE / WRITE_SIZE counters) and exit")
@@ -713,6 +717,10 @@ def main():
     from tensorflow_graphics_point_clouds_amd import _lib, layers, pc, synthetic, tfg_custom_ops
     _lib.lib()
     torch.backends.cuda.matmul.allow_tf32 = False
+    if args.only_dense_radius is not None:
+        print(json.dumps(isolated_basis_proj(torch, pc, synthetic, tfg_custom_ops, _lib,
+                                             radius=args.only_dense_radius, steps=2)))
+        return
 
     cfg, cloud = build_scene(torch, pc, synthetic, args.scale)
     radius = cfg["radius"]

@@ -125,6 +125,9 @@ __device__ __forceinline__ void project_run_body(
         asm volatile("" : "+v"(tile[j][kt]));
         acc[j][kt] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
       }
+#ifdef MCCNN_PROBE_NO_TILE_STORES
+    if (row == -7)          // measurement probe (no output): the kernel without its write-out
+#endif
 #pragma unroll
     for (int j = 0; j < kCPL; ++j)
 #pragma unroll
@@ -165,9 +168,17 @@ __device__ __forceinline__ void project_run_body(
         const float4 gn = stage->geo[n];
         // one 32-bit lane offset on the wavefront's (scalar) base address
         const unsigned rn = stage->row[n];
+#ifdef MCCNN_PROBE_NO_FEATURE_LOADS
+        // measurement probe (wrong results): the B operands come from registers, so the run
+        // time is that of the kernel with every feature row already on chip -- the bound of
+        // any scheme that stages the rows in LDS
+#pragma unroll
+        for (int j = 0; j < kCPL; ++j) f[u].v[j] = gn.y + __uint_as_float(rn);
+#else
 #pragma unroll
         for (int j = 0; j < kCPL; ++j)
           f[u].v[j] = *reinterpret_cast<const float *>(feat_base + (size_t)(rn + lane_off) + j * 64);
+#endif
         int aux = 0;
         if constexpr (Basis::kUsesAux) aux = stage->aux[n];
 #pragma unroll
