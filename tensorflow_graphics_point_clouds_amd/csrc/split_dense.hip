@@ -114,7 +114,10 @@ __global__ void __launch_bounds__(256, 2) nt_split_kernel(int64_t n, int R,
   }
 }
 
-static int nt_split_ct(int F) { return F == 128 ? 1 : F == 64 ? 2 : F == 32 ? 4 : 0; }
+// (F = 128 stays on the float32 kernel: with 32 output columns per wavefront the split of
+// the 128-wide rows of x costs more vector instructions than the six matrix instructions
+// save -- 4.5 against 2.1 ms on [825 274, 128] x [2048, 128]^T)
+static int nt_split_ct(int F) { return F == 64 ? 2 : F == 32 ? 4 : 0; }
 
 bool nt_split_supported(int F, int R) {
   const int ct = nt_split_ct(F);
@@ -135,7 +138,6 @@ int launch_nt_split(hipStream_t s, int64_t n, int F, const float *x, int R, cons
   if (slices > tiles) slices = (int)tiles;
   const dim3 grid(groups * slices), block(256);
   switch (F) {
-    case 128: hipLaunchKernelGGL((nt_split_kernel<128, 1>), grid, block, 0, s, n, R, x, w, slices, out); break;
     case 64: hipLaunchKernelGGL((nt_split_kernel<64, 2>), grid, block, 0, s, n, R, x, w, slices, out); break;
     default: hipLaunchKernelGGL((nt_split_kernel<32, 4>), grid, block, 0, s, n, R, x, w, slices, out); break;
   }
