@@ -176,6 +176,23 @@ int mccnn_find_neighbors_count(
     const float *inv_cell_sizes, int inv_radii_len, const float *inv_radii,
     int max_neighs, void *workspace, size_t workspace_bytes,
     int32_t *ranges_out, int64_t *num_neighbors_out_host);
+/* _count with two facts about the table it sizes, read back in the same synchronisation:
+ * facts_out_host[0] = 1 if some centre lost pairs to max_neighs, [1] = 1 if the centres are
+ * the searched points themselves (same address and count).  With [0] == 0 and [1] == 1 the
+ * table is symmetric (j in N(c) <=> c in N(j)) and mccnn_compute_pdf_pt_grads_symmetric
+ * applies.  No counterpart in the reference. */
+int mccnn_find_neighbors_count_facts(
+    mccnn_stream_t stream, int64_t num_samples, int num_dims,
+    const float *samples, int64_t sample_batch_ids_len,
+    const int32_t *sample_batch_ids, int64_t num_pts, int pts_dims,
+    const float *points, int64_t point_keys_len, const int64_t *point_keys,
+    int ds_rank, int ds_batch, int ds_nx, int ds_ny, int ds_last,
+    const int32_t *grid_ds, int num_cells_len, const int32_t *num_cells,
+    int aabb_dims, const float *scaled_aabb_min, int inv_cell_sizes_len,
+    const float *inv_cell_sizes, int inv_radii_len, const float *inv_radii,
+    int max_neighs, void *workspace, size_t workspace_bytes,
+    int32_t *ranges_out, int64_t *num_neighbors_out_host,
+    int64_t *facts_out_host);
 int mccnn_find_neighbors_fill(
     mccnn_stream_t stream, int64_t num_samples, int num_dims,
     const float *samples, const int32_t *sample_batch_ids, int64_t num_pts,

@@ -101,7 +101,8 @@ def host_count():
     import torch
     t = getattr(_host_counts, "tensor", None)
     if t is None:
-        t = torch.zeros(1, dtype=torch.int64, pin_memory=True)
+        # [0] the count; [1], [2] the two facts mccnn_find_neighbors_count_facts reports
+        t = torch.zeros(4, dtype=torch.int64, pin_memory=True)
         _host_counts.tensor = t
     return t, vptr(t.data_ptr())
 

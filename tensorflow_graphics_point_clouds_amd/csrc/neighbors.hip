@@ -171,7 +171,8 @@ template <int D, bool kFill>
 __global__ void __launch_bounds__(kNbrThreads) nbr_visit_kernel(
     int64_t ns, const float *__restrict__ samples, const float *__restrict__ pts,
     const int2 *__restrict__ ranges, const float *__restrict__ inv_radii, int max_neighs,
-    int *__restrict__ counts, const int *__restrict__ ends, int2 *__restrict__ nbrs) {
+    int *__restrict__ counts, const int *__restrict__ ends, int2 *__restrict__ nbrs,
+    int64_t *__restrict__ truncated = nullptr) {
   constexpr int R = OffsetInfo<D>::count();
   const int sub = threadIdx.x & (kGroup - 1);
   const int lane = lane_id();
@@ -213,7 +214,11 @@ __global__ void __launch_bounds__(kNbrThreads) nbr_visit_kernel(
   if (!kFill) {
 #pragma unroll
     for (int off = kGroup / 2; off > 0; off >>= 1) found += __shfl_xor(found, off, kWave);
-    if (sub == 0) counts[c] = found < limit ? found : limit;
+    if (sub == 0) {
+      counts[c] = found < limit ? found : limit;
+      // some centre lost pairs to max_neighs (every writer stores the same value)
+      if (truncated && found > limit) *truncated = 1;
+    }
   }
 }
 
@@ -279,7 +284,9 @@ extern "C" size_t mccnn_find_neighbors_workspace_bytes(int num_dims, int64_t num
   return carve_nbr_workspace(nullptr, num_dims, num_samples).bytes;
 }
 
-extern "C" int mccnn_find_neighbors_count(
+// `facts_out_host` (optional, two values): [0] 1 if some centre lost pairs to max_neighs,
+// [1] 1 if the centres are the searched points themselves (same address, same count).
+static int find_neighbors_count_impl(
     mccnn_stream_t stream, int64_t num_samples, int num_dims, const float *samples,
     int64_t sample_batch_ids_len, const int32_t *sample_batch_ids, int64_t num_pts, int pts_dims,
     const float *points, int64_t point_keys_len, const int64_t *point_keys, int ds_rank,
@@ -287,7 +294,7 @@ extern "C" int mccnn_find_neighbors_count(
     const int32_t *num_cells, int aabb_dims, const float *scaled_aabb_min, int inv_cell_sizes_len,
     const float *inv_cell_sizes, int inv_radii_len, const float *inv_radii, int max_neighs,
     void *workspace, size_t workspace_bytes, int32_t *ranges_out,
-    int64_t *num_neighbors_out_host) {
+    int64_t *num_neighbors_out_host, int64_t *facts_out_host) {
   MCCNN_REQUIRE(valid_dims(num_dims), "FindNeighbors expects a valid number of dimensions");
   MCCNN_REQUIRE(num_cells_len == num_dims,
                 "FindNeighbors expects a number of dimensions in num_cells equal to the number of "
@@ -318,6 +325,10 @@ extern "C" int mccnn_find_neighbors_count(
                 "FindNeighbors expects sizes in [0, 2^31)");
   MCCNN_REQUIRE(num_neighbors_out_host, "FindNeighbors received a null output");
   *num_neighbors_out_host = 0;
+  if (facts_out_host) {
+    facts_out_host[0] = 0;
+    facts_out_host[1] = samples == points && num_samples == num_pts ? 1 : 0;
+  }
   if (num_samples == 0) return MCCNN_OK;
   MCCNN_REQUIRE(samples && sample_batch_ids && grid_ds && num_cells && scaled_aabb_min &&
                     inv_cell_sizes && inv_radii && ranges_out && workspace,
@@ -336,16 +347,25 @@ extern "C" int mccnn_find_neighbors_count(
                                       w.ranges));
   MCCNN_LAUNCH_CHECK();
   const unsigned grid = blocks_for(num_samples, kCentresPerBlock);
+  // truncation can only happen with max_neighs > 0: only then is the flag cleared and read
+  int64_t *truncated = facts_out_host && max_neighs > 0 ? w.total + 1 : nullptr;
+  if (truncated) {
+    int rc0 = fill_zero(s, truncated, sizeof(int64_t));
+    if (rc0 != MCCNN_OK) return rc0;
+  }
   MCCNN_DIM_SWITCH(num_dims, hipLaunchKernelGGL((nbr_visit_kernel<D, false>), dim3(grid),
                                                 dim3(kNbrThreads), 0, s, num_samples, samples,
                                                 points, (const int2 *)w.ranges, inv_radii,
                                                 max_neighs, ranges_out, (const int *)nullptr,
-                                                (int2 *)nullptr));
+                                                (int2 *)nullptr, truncated));
   MCCNN_LAUNCH_CHECK();
   int rc = inclusive_scan_i32(s, num_samples, ranges_out, w.scan_scratch, w.total);
   if (rc != MCCNN_OK) return rc;
   MCCNN_HIP_CHECK(hipMemcpyAsync(num_neighbors_out_host, w.total, sizeof(int64_t),
                                  hipMemcpyDeviceToHost, s));
+  if (truncated)
+    MCCNN_HIP_CHECK(hipMemcpyAsync(facts_out_host, truncated, sizeof(int64_t),
+                                   hipMemcpyDeviceToHost, s));
   MCCNN_HIP_CHECK(hipStreamSynchronize(s));
   // the scan saturates partial sums at 2^31 - 1, so a total from there on is a lower bound
   MCCNN_REQUIRE(*num_neighbors_out_host < (((int64_t)1 << 31) - 1),
@@ -353,6 +373,41 @@ extern "C" int mccnn_find_neighbors_count(
                 "hold fewer than 2^31 - 1",
                 (long long)*num_neighbors_out_host);
   return MCCNN_OK;
+}
+
+extern "C" int mccnn_find_neighbors_count(
+    mccnn_stream_t stream, int64_t num_samples, int num_dims, const float *samples,
+    int64_t sample_batch_ids_len, const int32_t *sample_batch_ids, int64_t num_pts, int pts_dims,
+    const float *points, int64_t point_keys_len, const int64_t *point_keys, int ds_rank,
+    int ds_batch, int ds_nx, int ds_ny, int ds_last, const int32_t *grid_ds, int num_cells_len,
+    const int32_t *num_cells, int aabb_dims, const float *scaled_aabb_min, int inv_cell_sizes_len,
+    const float *inv_cell_sizes, int inv_radii_len, const float *inv_radii, int max_neighs,
+    void *workspace, size_t workspace_bytes, int32_t *ranges_out,
+    int64_t *num_neighbors_out_host) {
+  return find_neighbors_count_impl(
+      stream, num_samples, num_dims, samples, sample_batch_ids_len, sample_batch_ids, num_pts,
+      pts_dims, points, point_keys_len, point_keys, ds_rank, ds_batch, ds_nx, ds_ny, ds_last,
+      grid_ds, num_cells_len, num_cells, aabb_dims, scaled_aabb_min, inv_cell_sizes_len,
+      inv_cell_sizes, inv_radii_len, inv_radii, max_neighs, workspace, workspace_bytes, ranges_out,
+      num_neighbors_out_host, nullptr);
+}
+
+extern "C" int mccnn_find_neighbors_count_facts(
+    mccnn_stream_t stream, int64_t num_samples, int num_dims, const float *samples,
+    int64_t sample_batch_ids_len, const int32_t *sample_batch_ids, int64_t num_pts, int pts_dims,
+    const float *points, int64_t point_keys_len, const int64_t *point_keys, int ds_rank,
+    int ds_batch, int ds_nx, int ds_ny, int ds_last, const int32_t *grid_ds, int num_cells_len,
+    const int32_t *num_cells, int aabb_dims, const float *scaled_aabb_min, int inv_cell_sizes_len,
+    const float *inv_cell_sizes, int inv_radii_len, const float *inv_radii, int max_neighs,
+    void *workspace, size_t workspace_bytes, int32_t *ranges_out,
+    int64_t *num_neighbors_out_host, int64_t *facts_out_host) {
+  MCCNN_REQUIRE(facts_out_host, "FindNeighbors received a null output");
+  return find_neighbors_count_impl(
+      stream, num_samples, num_dims, samples, sample_batch_ids_len, sample_batch_ids, num_pts,
+      pts_dims, points, point_keys_len, point_keys, ds_rank, ds_batch, ds_nx, ds_ny, ds_last,
+      grid_ds, num_cells_len, num_cells, aabb_dims, scaled_aabb_min, inv_cell_sizes_len,
+      inv_cell_sizes, inv_radii_len, inv_radii, max_neighs, workspace, workspace_bytes, ranges_out,
+      num_neighbors_out_host, facts_out_host);
 }
 
 extern "C" int mccnn_find_neighbors_fill(

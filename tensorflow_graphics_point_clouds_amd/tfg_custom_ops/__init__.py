@@ -65,7 +65,7 @@ def find_neighbors(samples, samples_batch_ids, points, point_keys, grid_acc_ds, 
     ranges = torch.empty(ns, dtype=_I32, device=dev)
     total, total_ptr = _lib.host_count()
     dsr = grid_acc_ds.dim()
-    _lib.call("find_neighbors_count", stream(), i64(ns), cint(nd), ptr(samples, _F32), i64(samples_batch_ids.shape[0]),
+    _lib.call("find_neighbors_count_facts", stream(), i64(ns), cint(nd), ptr(samples, _F32), i64(samples_batch_ids.shape[0]),
         ptr(samples_batch_ids, _I32), i64(points.shape[0]), cint(_dim(points, 1)),
         ptr(points, _F32), i64(point_keys.shape[0]), ptr(point_keys, _I64), cint(dsr),
         cint(_dim(grid_acc_ds, 0)), cint(_dim(grid_acc_ds, 1)), cint(_dim(grid_acc_ds, 2)),
@@ -73,9 +73,12 @@ def find_neighbors(samples, samples_batch_ids, points, point_keys, grid_acc_ds, 
         ptr(num_cells, _I32), cint(_dim(scaled_aabb_min, 1)), ptr(scaled_aabb_min, _F32),
         cint(inv_cell_sizes.shape[0]), ptr(inv_cell_sizes, _F32), cint(inv_radii.shape[0]),
         ptr(inv_radii, _F32), cint(max_neighs), ptr(ws), _lib.csize(ws.numel()), ptr(ranges),
-        total_ptr)
+        total_ptr, _lib.vptr(total.data_ptr() + 8), timed_as="find_neighbors_count")
     m = int(total[0])
+    symmetric = int(total[1]) == 0 and int(total[2]) == 1
     neighbors = torch.empty((m, 2), dtype=_I32, device=dev)
+    if symmetric:
+        _remember_symmetric(neighbors)
     _lib.call("find_neighbors_fill", stream(), i64(ns), cint(nd), ptr(samples, _F32), ptr(samples_batch_ids, _I32),
         i64(points.shape[0]), ptr(points, _F32), ptr(point_keys, _I64), ptr(grid_acc_ds, _I32),
         ptr(num_cells, _I32), ptr(scaled_aabb_min, _F32), ptr(inv_cell_sizes, _F32),
@@ -119,11 +122,32 @@ def _compute_pdf_raw(points, neighbors, ranges, inv_bandwidth, inv_radii, mode):
     return pdf
 
 
+# Pair tables that find_neighbors reported as untruncated self-neighbourhoods (symmetric:
+# j in N(c) <=> c in N(j)), by the identity of the tensor it returned; the entry dies with it.
+_symmetric_tables = {}
+
+
+def _remember_symmetric(neighbors):
+    import weakref
+    key = id(neighbors)
+    _symmetric_tables[key] = weakref.ref(neighbors, lambda _, k=key: _symmetric_tables.pop(k, None))
+
+
+def is_symmetric_table(neighbors):
+    """True for a pair table that `find_neighbors` returned for the points as their own
+    centres without cutting any neighbourhood at max_neighs."""
+    ref = _symmetric_tables.get(id(neighbors))
+    return ref is not None and ref() is neighbors
+
+
 def compute_pdf_pt_grads(points, neighbors, sample_neigh_indices, inv_bandwidth, inv_radii,
                          pdf_grads, mode, symmetric=False):
     """ComputePdfPtGrads (compute_pdf_ops.cpp:58-74): [N, D] gradient of
     sum(pdf_grads * pdf) with respect to the points.  `symmetric=True` (the caller
-    vouches that j in N(c) <=> c in N(j)) selects the atomic-free gather."""
+    vouches that j in N(c) <=> c in N(j)) selects the atomic-free gather; a table that
+    `find_neighbors` itself reported as an untruncated self-neighbourhood takes it
+    without being told."""
+    symmetric = symmetric or is_symmetric_table(neighbors)
     out = torch.empty_like(points)
     _lib.call("compute_pdf_pt_grads_symmetric" if symmetric else "compute_pdf_pt_grads", stream(), i64(points.shape[0]), cint(_dim(points, 1)), ptr(points, _F32),
         i64(neighbors.shape[0]), cint(neighbors.dim()), cint(_dim(neighbors, 1)),

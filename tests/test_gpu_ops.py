@@ -210,6 +210,35 @@ def test_pdf_and_point_grads(ops, oracle, d, mode):
     assert_normwise(sym.cpu().numpy(), gexp)
 
 
+def test_find_neighbors_reports_symmetric_tables(ops, oracle):
+    """find_neighbors marks the table it returns as symmetric exactly when the centres are the
+    searched points themselves and no neighbourhood was cut at max_neighs; compute_pdf_pt_grads
+    then takes the atomic-free form by itself and must still give the oracle's gradient."""
+    rng = np.random.default_rng(91)
+    pts, bids = _cloud(rng, 2, 3000, 3)
+    g = oracle.Grid(pts, bids, 2, 0.15)
+    sp, sb = dev(g.sorted_points), dev(g.sorted_batch_ids)
+    args = (dev(g.sorted_keys), dev(g.get_ds()), dev(g.num_cells), dev(g.scaled_aabb_min),
+            dev(g.inv_cell_sizes), dev(np.full(3, 1 / np.float32(0.15), np.float32)))
+    largest = int(np.diff(np.concatenate([[0], oracle.Neighborhood(g, 0.15).ranges])).max())
+    inv_bw = np.full(3, 1 / np.float32(0.2), np.float32)
+    up = rng.standard_normal(len(pts)).astype(np.float32)
+    for limit, same, expect in ((0, True, True), (largest, True, True), (largest - 1, True, False),
+                                (6, True, False), (0, False, False)):
+        centres = sp if same else sp.clone()
+        ranges, nbrs = ops.find_neighbors(centres, sb, sp, *args, limit)
+        assert ops.is_symmetric_table(nbrs) == expect, (limit, same)
+        assert not ops.is_symmetric_table(nbrs.clone())
+        nbh = oracle.Neighborhood(g, 0.15, max_neighbors=limit)
+        assert np.array_equal(nbrs.cpu().numpy(), nbh.neighbors)
+        for mode in (0, 1):
+            gexp = oracle.compute_pdf_pt_grads(g.sorted_points, nbh.neighbors, nbh.ranges, inv_bw,
+                                               nbh.inv_radii, up, mode)
+            got = ops.compute_pdf_pt_grads(sp, nbrs, ranges, dev(inv_bw), dev(nbh.inv_radii),
+                                           dev(up), mode)
+            assert_normwise(got.cpu().numpy(), gexp)
+
+
 @pytest.mark.parametrize("variant", ["truncated", "shuffled", "truncated+shuffled"])
 def test_pdf_point_grads_on_asymmetric_and_unordered_tables(ops, oracle, variant):
     """compute_pdf_pt_grads looks the reverse of every pair up in the neighbour's list: lists
