@@ -122,6 +122,16 @@ __device__ __forceinline__ void wave_lds_sync() {
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
+// Barrier of the block that orders its LDS traffic only: what any thread wrote to LDS
+// before the call is what every thread reads after it.  Unlike __syncthreads() it does not
+// wait for the wavefront's outstanding global loads and stores (a prefetch in flight,
+// streamed stores whose acknowledgement takes microseconds).  Every thread must reach it.
+__device__ __forceinline__ void block_lds_sync() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
 // Inclusive prefix sum across the 64 lanes of a wave.
 __device__ __forceinline__ int wave_inclusive_scan(int v) {
   const int lane = lane_id();

@@ -435,7 +435,8 @@ def test_weight_grad_product_matches_float64(n, c, r, dense_mode):
 @pytest.mark.parametrize("n,f,r", [(1, 16, 256), (4099, 64, 1024), (20000, 32, 512), (0, 64, 256),
                                    (4099, 128, 1024), (3001, 128, 2048), (1500, 256, 4096),
                                    (17, 256, 64), (33, 128, 128), (31, 64, 256), (70001, 64, 1024),
-                                   (5000, 32, 1024), (65, 128, 256)])
+                                   (5000, 32, 1024), (65, 128, 256), (70001, 128, 2048),
+                                   (2081, 128, 384)])
 def test_projection_grad_product_matches_float64(n, f, r, dense_mode):
     """x w^T elementwise against float64: |got - expect| <= 1e-5 * (|x| |w|^T), on operands
     whose magnitudes span six decades; equal bits on a second call."""
