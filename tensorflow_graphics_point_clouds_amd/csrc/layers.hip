@@ -267,6 +267,95 @@ __global__ void __launch_bounds__(256) kp_regularization_kernel(
   rep[t] = r;
 }
 
+// The same terms for up to 16 kernel points in 2 or 3 dimensions: the 16 lanes of a quarter of a wavefront take
+// one centre, lane k kernel point k.  The quarter fetches 16 pairs of its centre at a time --
+// lane j pair m0 + j: index, coordinates, scaled offset to the centre -- and parks them in
+// LDS; every lane then runs over the parked offsets with one broadcast LDS read per pair,
+// instead of one index load and D coordinate loads per pair in each of the KP threads of a
+// centre (1.34 -> 0.54 ms on 825 274 centres, 32.3 M pairs, 15 kernel points).  Same
+// operations in the same order per (centre, kernel point): same bits.
+template <int D>
+__global__ void __launch_bounds__(256) kp_regularization16_kernel(
+    int64_t n_out, int KP, int kind, float sigma, const float *__restrict__ pin,
+    const float *__restrict__ pout, const int2 *__restrict__ nbrs, const int *__restrict__ ranges,
+    const float *__restrict__ inv_radii, const float *__restrict__ kpts,
+    const float *__restrict__ offsets, float *__restrict__ fit, int *__restrict__ argmin,
+    float *__restrict__ rep) {
+  static_assert(D <= 3, "a parked offset is three floats");
+  __shared__ float4 stage[256];
+  float ir[D];
+#pragma unroll
+  for (int d = 0; d < D; ++d) ir[d] = inv_radii[d];
+  const int k = threadIdx.x & 15;
+  float4 *mine = stage + (threadIdx.x & ~15);       // the 16 slots of this quarter
+  const int64_t c = (blockIdx.x * (int64_t)blockDim.x + threadIdx.x) >> 4;
+  const bool centre = c < n_out, live = centre && k < KP;
+  const int64_t t = c * KP + k;
+  float kp[3] = {0.0f, 0.0f, 0.0f}, ctr[3] = {0.0f, 0.0f, 0.0f};
+#pragma unroll
+  for (int d = 0; d < D; ++d) {
+    if (live) kp[d] = kpts[k * D + d] + offsets[t * D + d];
+    if (centre) ctr[d] = pout[c * D + d];
+  }
+  const int a = centre ? (c > 0 ? ranges[c - 1] : 0) : 0, b = centre ? ranges[c] : 0;
+  float best = 0.0f;
+  int best_m = -1;
+  for (int m0 = a; __any(m0 < b); m0 += 16) {        // every lane of the wavefront stays in step
+    const int cnt = b - m0 < 16 ? b - m0 : 16;       // <= 0 for a quarter that has finished
+    if (k < cnt) {
+      const int idx = nbrs[m0 + k].x;
+      float dl[3] = {0.0f, 0.0f, 0.0f};
+#pragma unroll
+      for (int d = 0; d < D; ++d) dl[d] = (pin[(int64_t)idx * D + d] - ctr[d]) * ir[d];
+      mine[k] = make_float4(dl[0], dl[1], dl[2], 0.0f);
+    }
+    wave_lds_sync();
+    for (int j = 0; j < cnt; ++j) {
+      const float4 g = mine[j];
+      const float dl[3] = {g.x, g.y, g.z};
+      float sq = 0.0f;
+#pragma unroll
+      for (int d = 0; d < D; ++d) {
+        const float diff = dl[d] - kp[d];
+        sq += diff * diff;
+      }
+      if (best_m < 0 || sq < best) {
+        best = sq;
+        best_m = m0 + j;
+      }
+    }
+    wave_lds_sync();
+  }
+  // repulsion of this kernel point against the others of the same centre
+  mine[k] = make_float4(kp[0], kp[1], kp[2], 0.0f);
+  wave_lds_sync();
+  float r = 0.0f;
+  for (int k2 = 0; k2 < KP; ++k2) {
+    if (k2 == k) continue;
+    const float4 o = mine[k2];
+    const float other[3] = {o.x, o.y, o.z};
+    float sq = 0.0f;
+#pragma unroll
+    for (int d = 0; d < D; ++d) {
+      const float diff = kp[d] - other[d];
+      sq += diff * diff;
+    }
+    const float dist = sqrtf(sq);
+    if (kind == 0) {
+      const float v = 1.0f - dist / sigma;
+      r += v > 0.0f ? v : 0.0f;
+    } else {
+      const float q = dist / (sigma / 3.0f);
+      r += expf(-(q * q));
+    }
+  }
+  if (live) {
+    fit[t] = best / (sigma * sigma);
+    argmin[t] = best_m;
+    rep[t] = r;
+  }
+}
+
 // d(scale * (sum fit + sum rep)) / d(offsets).
 template <int D>
 __global__ void __launch_bounds__(256) kp_regularization_grads_kernel(
@@ -549,6 +638,21 @@ extern "C" int mccnn_kp_regularization(mccnn_stream_t stream, int64_t num_neighb
   MCCNN_REQUIRE(points_out && ranges && inv_radii && kernel_points && offsets && fit_out &&
                     argmin_out && repulsion_out && (num_neighbors == 0 || (points_in && neighbors)),
                 "kp_regularization received a null tensor");
+  if (num_kernel_points <= 16 && num_dims <= 3) {
+    const dim3 grid(blocks_for(num_samples * 16, 256)), block(256);
+    if (num_dims == 2)
+      hipLaunchKernelGGL(kp_regularization16_kernel<2>, grid, block, 0, as_stream(stream),
+                         num_samples, num_kernel_points, kind, sigma, points_in, points_out,
+                         (const int2 *)neighbors, ranges, inv_radii, kernel_points, offsets,
+                         fit_out, argmin_out, repulsion_out);
+    else
+      hipLaunchKernelGGL(kp_regularization16_kernel<3>, grid, block, 0, as_stream(stream),
+                         num_samples, num_kernel_points, kind, sigma, points_in, points_out,
+                         (const int2 *)neighbors, ranges, inv_radii, kernel_points, offsets,
+                         fit_out, argmin_out, repulsion_out);
+    MCCNN_LAUNCH_CHECK();
+    return MCCNN_OK;
+  }
   const int64_t work = num_samples * num_kernel_points;
   MCCNN_DIM_SWITCH(num_dims,
                    hipLaunchKernelGGL(kp_regularization_kernel<D>, dim3(blocks_for(work, 256)),

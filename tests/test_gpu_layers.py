@@ -348,6 +348,66 @@ def test_deformable_kpconv_and_regularization(oracle, kind, c_in, c_out):
                             wts, woff, 0.5 * radius, kind)
 
 
+@pytest.mark.parametrize("kpn", [5, 15, 16, 20])
+@pytest.mark.parametrize("dims", [2, 3])
+@pytest.mark.parametrize("kind", [0, 1])
+def test_kp_regularization_terms(oracle, kpn, dims, kind):
+    """The per-(centre, kernel point) terms of the regularisation loss (KPConv.py:394-429) as
+    the op returns them -- fitting distance, the pair that attains it, repulsion -- against a
+    float64 evaluation on the oracle's pairs; up to 16 kernel points take the kernel with a
+    quarter of a wavefront per centre, more the one with a thread per term.  Centres without
+    pairs report 0 and -1."""
+    from tensorflow_graphics_point_clouds_amd import _lib
+    from tensorflow_graphics_point_clouds_amd._lib import cfloat, cint, i64, ptr, stream
+    rng = np.random.default_rng(100 * kpn + 10 * dims + kind)
+    n, n_out, batch, radius, sigma = 1500, 420, 2, 0.2, 0.45
+    pts = rng.random((n, dims)).astype(np.float32)
+    bids = np.sort(rng.integers(0, batch, n)).astype(np.int32)
+    ctr = (rng.random((n_out, dims)) * 2.0 - 0.5).astype(np.float32)    # some far from every point
+    cb = np.sort(rng.integers(0, batch, n_out)).astype(np.int32)
+    g = oracle.Grid(pts, bids, batch, np.float32(radius))
+    nbh = oracle.Neighborhood(g, np.float32(radius), ctr, cb)
+    ids, ranges = nbh.original_neigh_ids, nbh.ranges
+    counts = np.diff(np.concatenate([[0], ranges]))
+    assert (counts == 0).any() and counts.max() > 16
+    kp = (rng.standard_normal((kpn, dims)) * 0.5).astype(np.float32)
+    off = (rng.standard_normal((n_out, kpn, dims)) * 0.05).astype(np.float32)
+    inv_r = np.full(dims, 1 / np.float32(radius), np.float32)
+    fit = torch.empty((n_out, kpn), dtype=torch.float32, device="cuda")
+    rep = torch.empty_like(fit)
+    argmin = torch.empty((n_out, kpn), dtype=torch.int32, device="cuda")
+    # the device copies stay referenced until the results have been read back
+    t_pts, t_ctr, t_ids, t_ranges = dev(pts), dev(ctr), dev(ids), dev(ranges)
+    t_inv_r, t_kp, t_off = dev(inv_r), dev(kp), dev(off)
+    assert t_ids.dtype == torch.int32 and t_ranges.dtype == torch.int32
+    assert t_ids.shape == (int(ranges[-1]), 2) and int(ids[:, 0].max()) < n
+    _lib.call("kp_regularization", stream(), i64(len(ids)), cint(dims), cint(kpn), cint(kind),
+              cfloat(sigma), ptr(t_pts), ptr(t_ctr), ptr(t_ids), i64(n_out), ptr(t_ranges),
+              ptr(t_inv_r), ptr(t_kp), ptr(t_off), ptr(fit), ptr(argmin), ptr(rep))
+    fit, rep, argmin = fit.cpu().numpy(), rep.cpu().numpy(), argmin.cpu().numpy()
+    del t_pts, t_ctr, t_ids, t_ranges, t_inv_r, t_kp, t_off
+    moved = kp.astype(np.float64)[None] + off.astype(np.float64)            # [n_out, kpn, dims]
+    delta = (pts.astype(np.float64)[ids[:, 0]] - ctr.astype(np.float64)[ids[:, 1]]) * inv_r
+    sq = ((delta[:, None, :] - moved[ids[:, 1]]) ** 2).sum(-1)              # [M, kpn]
+    start = 0
+    for c, end in enumerate(ranges):
+        if end == start:
+            assert (fit[c] == 0).all() and (argmin[c] == -1).all()
+            continue
+        seg = sq[start:end]
+        best = seg.min(0)
+        # differences of coordinates of order 1 are squared: absolute float32 error ~1e-7
+        np.testing.assert_allclose(fit[c], best / sigma ** 2, rtol=1e-5, atol=2e-6)
+        assert ((argmin[c] >= start) & (argmin[c] < end)).all()
+        # the reported pair attains the minimum (ties and near-ties: to float32 accuracy)
+        np.testing.assert_allclose(sq[argmin[c], np.arange(kpn)], best, rtol=1e-5, atol=1e-6)
+        start = end
+    dist = np.sqrt(((moved[:, :, None, :] - moved[:, None, :, :]) ** 2).sum(-1))
+    wgt = np.maximum(1 - dist / sigma, 0) if kind == 0 else np.exp(-(dist / (sigma / 3)) ** 2)
+    wgt[:, np.arange(kpn), np.arange(kpn)] = 0
+    np.testing.assert_allclose(rep, wgt.sum(-1), rtol=1e-5, atol=1e-6)
+
+
 @pytest.mark.parametrize("c", [1, 4, 5, 16, 64, 100, 128, 256])
 def test_local_and_global_pooling(oracle, c):
     from tensorflow_graphics_point_clouds_amd import layers, pc
