@@ -114,18 +114,19 @@ __global__ void __launch_bounds__(256, 2) nt_split_kernel(int64_t n, int R,
   }
 }
 
-// The same product for F = 128, where a wavefront has registers for 32 rows of w only: if
-// every wavefront split the 128-wide rows of x for its 32 output columns, the split would
-// cost more vector instructions than the six matrix instructions save (4.5 ms against 4.2 ms
-// of the float32 kernel on [825 274, 128] x [2048, 128]^T; this kernel 2.5 ms).  Here the
-// four wavefronts of a block (128 output columns) split the tile of 32 points together: a
-// thread fetches two runs of 8 values two tiles ahead, splits them while the current tile is
-// multiplied, and parks the three parts as 16-byte vectors in operand order ([part][matrix step][lane
-// half][point], one slot of padding per 32 points, so that the 16 lanes of a store phase --
-// the 16 runs of one point -- fall into 16 different bank groups); every A operand is one
-// 16-byte LDS read.  The 32 x 128 tile of the output leaves through a block-wide LDS
-// transposition as runs of 512 bytes.
-template <int F>
+// The same product with the split of x shared by the four wavefronts of a block.  Above, a
+// wavefront splits its tile of x for its own 32 kCT output columns; with F = 128 (registers
+// for 32 columns only) that split costs more vector instructions than the six matrix
+// instructions save (4.5 ms against 4.2 ms of the float32 kernel on [825 274, 128] x
+// [2048, 128]^T; this kernel 2.5 ms), and with F = 64 the shared split is still the faster
+// one (0.65 against 0.79 ms on [763 063, 64] x [1024, 64]^T).  Here the block owns 128 kCT columns and splits a tile
+// of 32 points once: a thread fetches its runs of 8 values two tiles ahead, splits them while
+// the current tile is multiplied, and parks the three parts as 16-byte vectors in operand
+// order ([part][matrix step][lane half][point], one slot of padding per 32 points, so that
+// the lanes of a store phase -- the runs of one point -- fall into different bank groups);
+// every A operand is one 16-byte LDS read.  The 32 x 128 kCT tile of the output leaves
+// through a block-wide LDS transposition as runs of 512 kCT bytes.
+template <int F, int kCT>
 __global__ void __launch_bounds__(256, 2) nt_split_shared_kernel(int64_t n, int R,
                                                                  const float *__restrict__ x,
                                                                  const float *__restrict__ w,
@@ -134,26 +135,31 @@ __global__ void __launch_bounds__(256, 2) nt_split_shared_kernel(int64_t n, int 
   constexpr int KS = F / 16;                    // matrix steps per tile
   constexpr int kRuns = F / 8;                  // runs of 8 reduction values per point
   constexpr int kItems = 32 * kRuns / 256;      // (point, run) items per thread
+  constexpr int kCols = 128 * kCT;              // output columns of the block
   constexpr int kLdA = 32 + 1;
-  constexpr int kLdO = 128 + 8;                 // lane halves (4 rows apart) 32 banks apart
+  constexpr int kLdO = kCols + 8;               // lane halves (4 rows apart) 32 banks apart
+  constexpr int kPieces = kCols / 4;            // 16-byte pieces per output row
+  constexpr int kRowsPer = kWave / kPieces;     // rows per store instruction
+  static_assert(kItems >= 1 && kRowsPer >= 1, "tile shape");
   __shared__ v8bf a_lds[2][3 * kRuns * kLdA];
   __shared__ __align__(16) float o_lds[32][kLdO];
   const int lane = lane_id(), wave = threadIdx.x / kWave;
   const int p = lane & 31, h = lane >> 5;
-  const int groups = R / 128;
+  const int groups = R / kCols;
   // the hardware deals consecutive blocks to the eight XCDs in turn: the column groups of a
   // slice share its rows of x, so they are numbered onto one XCD (one L2)
   const int in_xcd = blockIdx.x / 8;
   const int grp = in_xcd % groups, slice = (in_xcd / groups) * 8 + blockIdx.x % 8;
   if (slice >= slices) return;
-  const int col0 = grp * 128 + wave * 32;
-  Split8 b[KS];
-  {
-    const float *wr = w + (int64_t)(col0 + p) * F + (F / 2) * h;
+  const int wcol = wave * 32 * kCT;             // first column of this wavefront in the block
+  Split8 b[kCT][KS];
+#pragma unroll
+  for (int ct = 0; ct < kCT; ++ct) {
+    const float *wr = w + (int64_t)(grp * kCols + wcol + 32 * ct + p) * F + (F / 2) * h;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks)
-      b[ks] = split8(*reinterpret_cast<const v4f *>(wr + 8 * ks),
-                     *reinterpret_cast<const v4f *>(wr + 8 * ks + 4));
+      b[ct][ks] = split8(*reinterpret_cast<const v4f *>(wr + 8 * ks),
+                         *reinterpret_cast<const v4f *>(wr + 8 * ks + 4));
   }
   const int64_t tiles_total = (n + 31) >> 5;
   const int64_t per = (tiles_total + slices - 1) / slices;
@@ -186,31 +192,39 @@ __global__ void __launch_bounds__(256, 2) nt_split_shared_kernel(int64_t n, int 
   // receives the tile after that.
   auto step = [&](int64_t t, int cur, v4f (*parked)[2], v4f (*fetched)[2]) {
     if (t + 2 < t1) fetch(t + 2, fetched);
-    v16f acc;
+    v16f acc[kCT];
 #pragma unroll
-    for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
+    for (int ct = 0; ct < kCT; ++ct)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[ct][i] = 0.0f;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       Split8 a;
 #pragma unroll
       for (int q = 0; q < 3; ++q) a.p[q] = a_lds[cur][((q * KS + ks) * 2 + h) * kLdA + p];
-      acc = mma_split(a, b[ks], acc);
-    }
-    // acc[i]: point 32 t + (i / 4) * 8 + 4 h + i % 4, column col0 + p
 #pragma unroll
-    for (int i = 0; i < 16; ++i) o_lds[(i / 4) * 8 + 4 * h + (i % 4)][32 * wave + p] = acc[i];
+      for (int ct = 0; ct < kCT; ++ct) acc[ct] = mma_split(a, b[ct][ks], acc[ct]);
+    }
+    // acc[ct][i]: point 32 t + (i / 4) * 8 + 4 h + i % 4, column wcol + 32 ct + p of the block
+#pragma unroll
+    for (int ct = 0; ct < kCT; ++ct)
+#pragma unroll
+      for (int i = 0; i < 16; ++i)
+        o_lds[(i / 4) * 8 + 4 * h + (i % 4)][wcol + 32 * ct + p] = acc[ct][i];
     if (t + 1 < t1) park(cur ^ 1, parked);
     block_lds_sync();             // the output tile and the next tile of x are complete
-    v4f rows[4];
+    // wavefront w sends rows 8 w .. 8 w + 7 of the tile
+    const int piece = lane % kPieces, rr = lane / kPieces;
+    v4f rows[8 / kRowsPer];
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
-      rows[j] = *reinterpret_cast<const v4f *>(&o_lds[8 * wave + 2 * j + h][4 * p]);
+    for (int j = 0; j < 8 / kRowsPer; ++j)
+      rows[j] = *reinterpret_cast<const v4f *>(&o_lds[8 * wave + kRowsPer * j + rr][4 * piece]);
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int64_t row = 32 * t + 8 * wave + 2 * j + h;
+    for (int j = 0; j < 8 / kRowsPer; ++j) {
+      const int64_t row = 32 * t + 8 * wave + kRowsPer * j + rr;
       if (row < n)        // streamed: the product is read once, by a later kernel
         __builtin_nontemporal_store(
-            rows[j], reinterpret_cast<v4f *>(out + row * R + grp * 128 + 4 * p));
+            rows[j], reinterpret_cast<v4f *>(out + row * R + grp * kCols + 4 * piece));
     }
     block_lds_sync();             // the output tile has been read
   };
@@ -226,18 +240,17 @@ __global__ void __launch_bounds__(256, 2) nt_split_shared_kernel(int64_t n, int 
   }
 }
 
-static int nt_split_ct(int F) { return F == 64 ? 2 : F == 32 ? 4 : 0; }
+// F = 32: every wavefront splits its own tile (128 columns); F = 64 and 128: shared split.
+static int nt_split_cols(int F) { return F == 128 ? 128 : F == 64 ? 256 : F == 32 ? 512 : 0; }
 
 bool nt_split_supported(int F, int R) {
-  if (F == 128) return R >= 128 && R % 128 == 0;
-  const int ct = nt_split_ct(F);
-  return ct > 0 && R >= 128 * ct && R % (128 * ct) == 0;
+  const int cols = nt_split_cols(F);
+  return cols > 0 && R >= cols && R % cols == 0;
 }
 
 int launch_nt_split(hipStream_t s, int64_t n, int F, const float *x, int R, const float *w,
                     float *out) {
-  const int ct = F == 128 ? 1 : nt_split_ct(F);
-  const int groups = R / (128 * ct);
+  const int groups = R / nt_split_cols(F);
   int device = 0, cus = 0;
   MCCNN_HIP_CHECK(hipGetDevice(&device));
   MCCNN_HIP_CHECK(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device));
@@ -246,11 +259,11 @@ int launch_nt_split(hipStream_t s, int64_t n, int F, const float *x, int R, cons
   if (slices < 1) slices = 1;
   const int64_t tiles = (n + 31) / 32;
   if (slices > tiles) slices = (int)tiles;
-  // (the kernel for F = 128 numbers its blocks per XCD: slices rounded up to eight)
-  const dim3 grid(groups * (F == 128 ? (slices + 7) / 8 * 8 : slices)), block(256);
+  // (the kernels with a shared split number their blocks per XCD: slices rounded up to eight)
+  const dim3 grid(groups * (F >= 64 ? (slices + 7) / 8 * 8 : slices)), block(256);
   switch (F) {
-    case 128: hipLaunchKernelGGL((nt_split_shared_kernel<128>), grid, block, 0, s, n, R, x, w, slices, out); break;
-    case 64: hipLaunchKernelGGL((nt_split_kernel<64, 2>), grid, block, 0, s, n, R, x, w, slices, out); break;
+    case 128: hipLaunchKernelGGL((nt_split_shared_kernel<128, 1>), grid, block, 0, s, n, R, x, w, slices, out); break;
+    case 64: hipLaunchKernelGGL((nt_split_shared_kernel<64, 2>), grid, block, 0, s, n, R, x, w, slices, out); break;
     default: hipLaunchKernelGGL((nt_split_kernel<32, 4>), grid, block, 0, s, n, R, x, w, slices, out); break;
   }
   MCCNN_LAUNCH_CHECK();
