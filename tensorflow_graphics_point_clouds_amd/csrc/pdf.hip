@@ -2,7 +2,7 @@
 // with respect to the point coordinates
 // (custom_ops/tfg_custom_ops/compute_pdf/cc/kernels/compute_pdf_kernels.cu.cc:72-215).
 //
-// 16 lanes share a centre and stride over its pairs; the pair table is read
+// 4, 8 or 16 lanes share a centre and stride over its pairs; the pair table is read
 // coalesced, neighbour coordinates are gathered (they sit close together in the
 // sorted array, so the gathers hit L2).  The product over dimensions of
 // exp(-u_d^2/2) is evaluated as one exponential of the summed exponent.
@@ -11,9 +11,7 @@
 
 namespace mccnn {
 
-constexpr int kPdfGroup = 16;
 constexpr int kPdfThreads = 256;
-constexpr int kPdfCentresPerBlock = kPdfThreads / kPdfGroup;
 constexpr float kInvSqrt2Pi = 0.39894228f;
 
 template <int D>
@@ -37,14 +35,19 @@ __device__ __forceinline__ PdfScale<D> load_pdf_scale(const float *__restrict__ 
   return sc;
 }
 
-template <int D>
+// G lanes share a centre.  The kernel is bound by the chain of dependent loads of a centre
+// (list bounds, pair indices, coordinates) times the centres a compute unit holds in flight,
+// so short lists want few lanes per centre (more centres per wavefront) and long lists many:
+// 4 x 200k points, 7.5 / 52 / 170 pairs per point: 0.027 / 0.134 / 0.486 ms with 4 lanes,
+// 0.041 / 0.115 / 0.355 ms with 8, 0.074 / 0.133 / 0.315 ms with 16.
+template <int D, int G>
 __global__ void __launch_bounds__(kPdfThreads) compute_pdf_kernel(
     int64_t n, const float *__restrict__ pts, const int2 *__restrict__ nbrs,
     const int *__restrict__ ranges, const float *__restrict__ inv_bw,
     const float *__restrict__ inv_r, int mode, float *__restrict__ pdf) {
   const PdfScale<D> sc = load_pdf_scale<D>(inv_bw, inv_r, mode, n);
-  const int sub = threadIdx.x & (kPdfGroup - 1);
-  const int64_t c = (int64_t)blockIdx.x * kPdfCentresPerBlock + threadIdx.x / kPdfGroup;
+  const int sub = threadIdx.x & (G - 1);
+  const int64_t c = (int64_t)blockIdx.x * (kPdfThreads / G) + threadIdx.x / G;
   if (c >= n) return;
   float p[D];
 #pragma unroll
@@ -53,10 +56,10 @@ __global__ void __launch_bounds__(kPdfThreads) compute_pdf_kernel(
   // four pairs per lane and trip: their index loads, then their coordinate gathers, are
   // in flight together (the sums keep the order of a one-pair-per-trip loop)
   float acc = 0.0f;
-  for (int64_t m = a + sub; m < b; m += 4 * kPdfGroup) {
+  for (int64_t m = a + sub; m < b; m += 4 * G) {
     int64_t j[4];
 #pragma unroll
-    for (int q = 0; q < 4; ++q) j[q] = m + q * kPdfGroup < b ? nbrs[m + q * kPdfGroup].x : -1;
+    for (int q = 0; q < 4; ++q) j[q] = m + q * G < b ? nbrs[m + q * G].x : -1;
     float e[4];
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
@@ -72,7 +75,7 @@ __global__ void __launch_bounds__(kPdfThreads) compute_pdf_kernel(
     for (int q = 0; q < 4; ++q) acc += j[q] < 0 ? 0.0f : expf(-0.5f * e[q]);
   }
 #pragma unroll
-  for (int off = kPdfGroup / 2; off > 0; off >>= 1) acc += __shfl_xor(acc, off, kWave);
+  for (int off = G / 2; off > 0; off >>= 1) acc += __shfl_xor(acc, off, kWave);
   if (sub == 0) pdf[c] = acc * sc.norm;
 }
 
@@ -91,15 +94,15 @@ __global__ void __launch_bounds__(kPdfThreads) compute_pdf_kernel(
 // are zero-filled first).  An
 // untruncated self-neighbourhood takes no scatter at all: 41.8 M pairs in 1.06 ms where
 // scattering every pair's term with atomics takes 3.4 ms.
-template <int D>
+template <int D, int G>
 __global__ void __launch_bounds__(kPdfThreads) compute_pdf_grads_lookup_kernel(
     int64_t n, const float *__restrict__ pts, const int2 *__restrict__ nbrs,
     const int *__restrict__ ranges, const float *__restrict__ inv_bw,
     const float *__restrict__ inv_r, const float *__restrict__ pdf_grads, int mode,
     float *__restrict__ grads) {
   const PdfScale<D> sc = load_pdf_scale<D>(inv_bw, inv_r, mode, n);
-  const int sub = threadIdx.x & (kPdfGroup - 1);
-  const int64_t c = (int64_t)blockIdx.x * kPdfCentresPerBlock + threadIdx.x / kPdfGroup;
+  const int sub = threadIdx.x & (G - 1);
+  const int64_t c = (int64_t)blockIdx.x * (kPdfThreads / G) + threadIdx.x / G;
   if (c >= n) return;
   float p[D], own[D];
 #pragma unroll
@@ -109,7 +112,7 @@ __global__ void __launch_bounds__(kPdfThreads) compute_pdf_grads_lookup_kernel(
   }
   const float up = pdf_grads[c];
   const int64_t a = c > 0 ? ranges[c - 1] : 0, b = ranges[c];
-  for (int64_t m = a + sub; m < b; m += kPdfGroup) {
+  for (int64_t m = a + sub; m < b; m += G) {
     const int64_t j = nbrs[m].x;
     if (j == c) continue;                     // zero offset: no gradient either way
     float u[D], e = 0.0f;
@@ -141,7 +144,7 @@ __global__ void __launch_bounds__(kPdfThreads) compute_pdf_grads_lookup_kernel(
   for (int d = 0; d < D; ++d) {
     float v = own[d];
 #pragma unroll
-    for (int off = kPdfGroup / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+    for (int off = G / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
     if (sub == 0) unsafeAtomicAdd(&grads[c * D + d], v);
   }
 }
@@ -152,15 +155,15 @@ __global__ void __launch_bounds__(kPdfThreads) compute_pdf_grads_lookup_kernel(
 // pdf_grad_j * k_cj * u_cj * s, so
 //   grad[c] = sum_{j in N(c)} (pdf_grad_c + pdf_grad_j) * k_cj * u_cj * s
 // is a pure gather: no atomics, no zero fill, fixed summation order.
-template <int D>
+template <int D, int G>
 __global__ void __launch_bounds__(kPdfThreads) compute_pdf_grads_symmetric_kernel(
     int64_t n, const float *__restrict__ pts, const int2 *__restrict__ nbrs,
     const int *__restrict__ ranges, const float *__restrict__ inv_bw,
     const float *__restrict__ inv_r, const float *__restrict__ pdf_grads, int mode,
     float *__restrict__ grads) {
   const PdfScale<D> sc = load_pdf_scale<D>(inv_bw, inv_r, mode, n);
-  const int sub = threadIdx.x & (kPdfGroup - 1);
-  const int64_t c = (int64_t)blockIdx.x * kPdfCentresPerBlock + threadIdx.x / kPdfGroup;
+  const int sub = threadIdx.x & (G - 1);
+  const int64_t c = (int64_t)blockIdx.x * (kPdfThreads / G) + threadIdx.x / G;
   if (c >= n) return;
   float p[D], own[D];
 #pragma unroll
@@ -170,7 +173,7 @@ __global__ void __launch_bounds__(kPdfThreads) compute_pdf_grads_symmetric_kerne
   }
   const float up = pdf_grads[c];
   const int64_t a = c > 0 ? ranges[c - 1] : 0, b = ranges[c];
-  for (int64_t m = a + sub; m < b; m += kPdfGroup) {
+  for (int64_t m = a + sub; m < b; m += G) {
     const int64_t j = nbrs[m].x;
     float u[D], e = 0.0f;
 #pragma unroll
@@ -186,7 +189,7 @@ __global__ void __launch_bounds__(kPdfThreads) compute_pdf_grads_symmetric_kerne
   for (int d = 0; d < D; ++d) {
     float v = own[d];
 #pragma unroll
-    for (int off = kPdfGroup / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+    for (int off = G / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
     if (sub == 0) grads[c * D + d] = v;
   }
 }
@@ -227,11 +230,23 @@ extern "C" int mccnn_compute_pdf(mccnn_stream_t stream, int64_t num_pts, int num
   MCCNN_REQUIRE(points && ranges && inv_bandwidth && inv_radii && pdf_out &&
                     (neighbors || num_neighbors == 0),
                 "ComputePdf received a null tensor");
-  const unsigned grid = blocks_for(num_pts, kPdfCentresPerBlock);
-  MCCNN_DIM_SWITCH(num_dims, hipLaunchKernelGGL(compute_pdf_kernel<D>, dim3(grid),
-                                                dim3(kPdfThreads), 0, as_stream(stream), num_pts,
-                                                points, (const int2 *)neighbors, ranges,
-                                                inv_bandwidth, inv_radii, mode, pdf_out));
+  // lanes per centre by the mean length of a list
+  const int64_t mean = num_neighbors / num_pts;
+#define MCCNN_PDF_LAUNCH(G_)                                                                   \
+  MCCNN_DIM_SWITCH(num_dims,                                                                   \
+                   hipLaunchKernelGGL((compute_pdf_kernel<D, G_>),                             \
+                                      dim3(blocks_for(num_pts, kPdfThreads / G_)),             \
+                                      dim3(kPdfThreads), 0, as_stream(stream), num_pts, points, \
+                                      (const int2 *)neighbors, ranges, inv_bandwidth,          \
+                                      inv_radii, mode, pdf_out))
+  if (mean <= 16) {
+    MCCNN_PDF_LAUNCH(4);
+  } else if (mean <= 96) {
+    MCCNN_PDF_LAUNCH(8);
+  } else {
+    MCCNN_PDF_LAUNCH(16);
+  }
+#undef MCCNN_PDF_LAUNCH
   MCCNN_LAUNCH_CHECK();
   return MCCNN_OK;
 }
@@ -256,22 +271,37 @@ static int pdf_pt_grads_impl(mccnn_stream_t stream, int64_t num_pts, int num_dim
                     (neighbors || num_neighbors == 0),
                 "ComputePdfPtGrads received a null tensor");
   hipStream_t s = as_stream(stream);
-  const unsigned grid = blocks_for(num_pts, kPdfCentresPerBlock);
+  // lanes per centre by the mean length of a list, as in compute_pdf
+  const int64_t mean = num_neighbors / num_pts;
+  const int lanes = mean <= 16 ? 4 : mean <= 96 ? 8 : 16;
+#define MCCNN_PDF_GRADS_LAUNCH(KERNEL_, G_)                                                    \
+  MCCNN_DIM_SWITCH(num_dims,                                                                   \
+                   hipLaunchKernelGGL((KERNEL_<D, G_>),                                        \
+                                      dim3(blocks_for(num_pts, kPdfThreads / G_)),             \
+                                      dim3(kPdfThreads), 0, s, num_pts, points,                \
+                                      (const int2 *)neighbors, ranges, inv_bandwidth,          \
+                                      inv_radii, pdf_grads, mode, pt_grads_out))
   if (symmetric) {
-    MCCNN_DIM_SWITCH(num_dims,
-                     hipLaunchKernelGGL(compute_pdf_grads_symmetric_kernel<D>, dim3(grid),
-                                        dim3(kPdfThreads), 0, s, num_pts, points,
-                                        (const int2 *)neighbors, ranges, inv_bandwidth, inv_radii,
-                                        pdf_grads, mode, pt_grads_out));
+    if (lanes == 4) {
+      MCCNN_PDF_GRADS_LAUNCH(compute_pdf_grads_symmetric_kernel, 4);
+    } else if (lanes == 8) {
+      MCCNN_PDF_GRADS_LAUNCH(compute_pdf_grads_symmetric_kernel, 8);
+    } else {
+      MCCNN_PDF_GRADS_LAUNCH(compute_pdf_grads_symmetric_kernel, 16);
+    }
     MCCNN_LAUNCH_CHECK();
     return MCCNN_OK;
   }
   rc = fill_zero(s, pt_grads_out, sizeof(float) * (size_t)num_pts * num_dims);
   if (rc != MCCNN_OK) return rc;
-  MCCNN_DIM_SWITCH(num_dims, hipLaunchKernelGGL(compute_pdf_grads_lookup_kernel<D>, dim3(grid),
-                                                dim3(kPdfThreads), 0, s, num_pts, points,
-                                                (const int2 *)neighbors, ranges, inv_bandwidth,
-                                                inv_radii, pdf_grads, mode, pt_grads_out));
+  // the look-ups dominate here: 16 lanes stay the better choice for all but short lists
+  // (7.5 / 52 pairs per point: 0.108 / 1.148 ms with 4 / 8 lanes, 0.138 / 1.055 ms with 16)
+  if (lanes == 4) {
+    MCCNN_PDF_GRADS_LAUNCH(compute_pdf_grads_lookup_kernel, 4);
+  } else {
+    MCCNN_PDF_GRADS_LAUNCH(compute_pdf_grads_lookup_kernel, 16);
+  }
+#undef MCCNN_PDF_GRADS_LAUNCH
   MCCNN_LAUNCH_CHECK();
   return MCCNN_OK;
 }
