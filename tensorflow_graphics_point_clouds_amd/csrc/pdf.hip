@@ -79,6 +79,108 @@ __global__ void __launch_bounds__(kPdfThreads) compute_pdf_kernel(
   if (sub == 0) pdf[c] = acc * sc.norm;
 }
 
+#ifdef MCCNN_PROBE_STAGED_PDF
+// Measurement probe (correct results, built by `make probes` only): the same density with the
+// neighbours' coordinates staged in LDS.  A block takes 32 consecutive centres, 8 lanes each.
+// It finds the span of point indices its pairs touch, marks the chunks of 32 consecutive
+// points that occur in a direct-mapped table (index span of up to 65 536 points, no hashing),
+// gives every marked chunk a slot, copies the chunks' coordinates into LDS with coalesced
+// loads, and then evaluates the pairs with the coordinates read from LDS.  Pairs whose chunk
+// found no slot (more than kStageSlots chunks) and blocks whose span exceeds the table read
+// their coordinates from memory as the shipped kernel does.
+constexpr int kStageChunk = 32;
+constexpr int kStageMaxChunks = 2048;
+constexpr int kStageSlots = 48;
+
+template <int D>
+__global__ void __launch_bounds__(kPdfThreads) compute_pdf_staged_kernel(
+    int64_t n, const float *__restrict__ pts, const int2 *__restrict__ nbrs,
+    const int *__restrict__ ranges, const float *__restrict__ inv_bw,
+    const float *__restrict__ inv_r, int mode, float *__restrict__ pdf) {
+  constexpr int G = 8, kCentres = kPdfThreads / G;
+  constexpr unsigned short kUntouched = 0xffff, kTouched = 0xfffe;
+  __shared__ unsigned short slot_of[kStageMaxChunks];
+  __shared__ unsigned short chunk_of[kStageSlots];
+  __shared__ float staged[kStageSlots * kStageChunk * D];
+  __shared__ int s_min, s_max, s_count;
+  const PdfScale<D> sc = load_pdf_scale<D>(inv_bw, inv_r, mode, n);
+  const int sub = threadIdx.x & (G - 1);
+  const int64_t c = (int64_t)blockIdx.x * kCentres + threadIdx.x / G;
+  const bool live = c < n;
+  float p[D];
+#pragma unroll
+  for (int d = 0; d < D; ++d) p[d] = live ? pts[c * D + d] : 0.0f;
+  const int64_t a = live ? (c > 0 ? ranges[c - 1] : 0) : 0, b = live ? ranges[c] : 0;
+  if (threadIdx.x == 0) {
+    s_min = 0x7fffffff;
+    s_max = -1;
+    s_count = 0;
+  }
+  __syncthreads();
+  int lo = 0x7fffffff, hi = -1;
+  for (int64_t m = a + sub; m < b; m += G) {
+    const int j = nbrs[m].x;
+    lo = j < lo ? j : lo;
+    hi = j > hi ? j : hi;
+  }
+  if (hi >= 0) {
+    atomicMin(&s_min, lo);
+    atomicMax(&s_max, hi);
+  }
+  __syncthreads();
+  const int base = s_min;
+  const int chunks = s_max >= 0 ? (s_max - base) / kStageChunk + 1 : 0;
+  const bool table = chunks > 0 && chunks <= kStageMaxChunks;     // the same for the whole block
+  if (table) {
+    for (int i = threadIdx.x; i < chunks; i += kPdfThreads) slot_of[i] = kUntouched;
+    __syncthreads();
+    for (int64_t m = a + sub; m < b; m += G) slot_of[(nbrs[m].x - base) / kStageChunk] = kTouched;
+    __syncthreads();
+    for (int i = threadIdx.x; i < chunks; i += kPdfThreads)
+      if (slot_of[i] == kTouched) {
+        const int slot = atomicAdd(&s_count, 1);
+        if (slot < kStageSlots) {
+          slot_of[i] = (unsigned short)slot;
+          chunk_of[slot] = (unsigned short)i;
+        }
+      }
+    __syncthreads();
+    const int slots = s_count < kStageSlots ? s_count : kStageSlots;
+    for (int i = threadIdx.x; i < slots * kStageChunk * D; i += kPdfThreads) {
+      const int slot = i / (kStageChunk * D), r = i - slot * (kStageChunk * D);
+      const int64_t src = ((int64_t)base + (int64_t)chunk_of[slot] * kStageChunk) * D + r;
+      staged[i] = src < n * D ? pts[src] : 0.0f;
+    }
+    __syncthreads();
+  }
+  float acc = 0.0f;
+  for (int64_t m = a + sub; m < b; m += G) {
+    const int j = nbrs[m].x;
+    float q[D];
+    unsigned slot = kUntouched;
+    if (table) slot = slot_of[(j - base) / kStageChunk];
+    if (slot < (unsigned)kStageSlots) {
+      const float *src = &staged[(slot * kStageChunk + (j - base) % kStageChunk) * D];
+#pragma unroll
+      for (int d = 0; d < D; ++d) q[d] = src[d];
+    } else {
+#pragma unroll
+      for (int d = 0; d < D; ++d) q[d] = pts[(int64_t)j * D + d];
+    }
+    float e = 0.0f;
+#pragma unroll
+    for (int d = 0; d < D; ++d) {
+      const float u = (q[d] - p[d]) * sc.s[d];
+      e += u * u;
+    }
+    acc += expf(-0.5f * e);
+  }
+#pragma unroll
+  for (int off = G / 2; off > 0; off >>= 1) acc += __shfl_xor(acc, off, kWave);
+  if (live && sub == 0) pdf[c] = acc * sc.norm;
+}
+#endif  // MCCNN_PROBE_STAGED_PDF
+
 // grad[i] += g, grad[j] -= g with g_d = pdf_grad_i * pdf_ij * u_d * s_d
 // (compute_pdf_kernels.cu.cc:133-215 scatters both halves with atomics).
 // The gradient for an arbitrary pair table with as few atomics as the table allows.
@@ -230,6 +332,16 @@ extern "C" int mccnn_compute_pdf(mccnn_stream_t stream, int64_t num_pts, int num
   MCCNN_REQUIRE(points && ranges && inv_bandwidth && inv_radii && pdf_out &&
                     (neighbors || num_neighbors == 0),
                 "ComputePdf received a null tensor");
+#ifdef MCCNN_PROBE_STAGED_PDF
+  MCCNN_DIM_SWITCH(num_dims,
+                   hipLaunchKernelGGL(compute_pdf_staged_kernel<D>,
+                                      dim3(blocks_for(num_pts, kPdfThreads / 8)),
+                                      dim3(kPdfThreads), 0, as_stream(stream), num_pts, points,
+                                      (const int2 *)neighbors, ranges, inv_bandwidth, inv_radii,
+                                      mode, pdf_out));
+  MCCNN_LAUNCH_CHECK();
+  return MCCNN_OK;
+#endif
   // lanes per centre by the mean length of a list
   const int64_t mean = num_neighbors / num_pts;
 #define MCCNN_PDF_LAUNCH(G_)                                                                   \
