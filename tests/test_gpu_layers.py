@@ -1027,31 +1027,43 @@ def test_mcconv_gradient_with_respect_to_points(oracle):
 
     p = torch.tensor(pts.astype(np.float64), requires_grad=True)
     order = torch.tensor(g.sorted_indices).long()
-    sp = p[order]
     on = torch.tensor(own.neighbors).long()
-    u = (sp[on[:, 0]] - sp[on[:, 1]]) / (bw * radius)
+    u = (p[order][on[:, 0]] - p[order][on[:, 1]]) / (bw * radius)
+    u.retain_grad()
     kde = torch.prod(torch.exp(-0.5 * u * u) * (0.3989422804014327 / bw), dim=1)
     per_point = torch.zeros(n, dtype=torch.float64).index_add(0, on[:, 1], kde)
     ids = torch.tensor(nbh.original_neigh_ids).long()
     pdf = per_point[torch.tensor(nbh.neighbors[:, 0]).long()]
     w, b = conv.weights.detach().cpu().double()[0], conv.biases.detach().cpu().double()[0]
-    basis = torch.nn.functional.elu(((p[ids[:, 0]] - p[ids[:, 1]]) / radius) @ w + b) / pdf[:, None]
+    diff = (p[ids[:, 0]] - p[ids[:, 1]]) / radius
+    diff.retain_grad()
+    basis = torch.nn.functional.elu(diff @ w + b) / pdf[:, None]
     per_pair = torch.tensor(feat.astype(np.float64))[ids[:, 0]][:, :, None] * basis[:, None, :]
     proj = torch.zeros(n, c_in, hidden, dtype=torch.float64).index_add(0, ids[:, 1], per_pair)
     ref = proj.reshape(n, -1) @ conv.final_weights.detach().cpu().double()[0]
     normwise(out.detach().cpu().numpy(), ref.detach().numpy(), tol=1e-5)
     (ref * torch.tensor(up.astype(np.float64))).sum().backward()
     normwise(tpts.grad.cpu().numpy(), p.grad.numpy(), tol=1e-5)
+    # per coordinate: the gradient of a point is a signed sum of per-pair terms (through the
+    # kernel input of every pair it belongs to, as point or as centre, and through every
+    # density term it enters); the error is held to 1e-5 of the sum of their absolute values
+    mag = _point_gradient_magnitude(n, [(diff.grad / radius, ids[:, 0], ids[:, 1]),
+                                        (u.grad / (bw * radius), order[on[:, 0]], order[on[:, 1]])])
+    elementwise(tpts.grad.cpu().numpy(), p.grad.numpy(), mag.numpy())
 
 
-def _kde_per_point(p, g, own, bw, radius):
-    """float64 Gaussian KDE over the sorted self-neighbourhood, per original point."""
-    order = torch.tensor(g.sorted_indices).long()
-    sp = p[order]
-    on = torch.tensor(own.neighbors).long()
-    u = (sp[on[:, 0]] - sp[on[:, 1]]) / (bw * radius)
-    kde = torch.prod(torch.exp(-0.5 * u * u) * (0.3989422804014327 / bw), dim=1)
-    return torch.zeros(len(p), dtype=torch.float64).index_add(0, on[:, 1], kde)   # by sorted index
+def _point_gradient_magnitude(n, paths, n_centres=None):
+    """Sum of the absolute values of the per-pair terms that a coordinate gradient adds up:
+    every path is (gradient with respect to a per-pair difference `a - b`, index of a, index
+    of b).  Returns the magnitude for the `a` side ([n, D]) and, if the `b` side is another
+    point set of `n_centres` points, for that side too."""
+    first = torch.zeros((n, paths[0][0].shape[1]), dtype=torch.float64)
+    second = first if n_centres is None else torch.zeros((n_centres, first.shape[1]),
+                                                         dtype=torch.float64)
+    for grad, a, b, *same in paths:
+        first.index_add_(0, a, grad.abs())
+        (first if same and same[0] else second).index_add_(0, b, grad.abs())
+    return first if n_centres is None else (first, second)
 
 
 @pytest.mark.parametrize("layer", ["kp_linear", "kp_gaussian_deformable", "pointconv"])
@@ -1079,21 +1091,30 @@ def test_kpconv_and_pointconv_gradient_with_respect_to_points(oracle, layer):
         return torch.zeros(len(ctr), c_in, basis.shape[1], dtype=torch.float64).index_add(
             0, ids[:, 1], per_pair).reshape(len(ctr), -1)
 
+    paths = []      # (per-pair difference a - b, scale of the difference, index of a, index of b)
     if layer == "pointconv":
         conv = layers.PointConv(c_in, c_out, 3, size_hidden=8, non_linearity_type="elu", seed=3)
         with torch.no_grad():
             conv.pdf_biases_2.fill_(0.7)
         out = conv(dev(feat), cin, cout, radius, bandwidth=bw)
         g = oracle.Grid(pts, bids, batch, np.float32(radius))
-        per_sorted = _kde_per_point(p, g, oracle.Neighborhood(g, np.float32(radius)), bw, radius)
+        own = oracle.Neighborhood(g, np.float32(radius))
+        order, on = torch.tensor(g.sorted_indices).long(), torch.tensor(own.neighbors).long()
+        u = (p[order][on[:, 0]] - p[order][on[:, 1]]) / (bw * radius)
+        u.retain_grad()
+        kde = torch.prod(torch.exp(-0.5 * u * u) * (0.3989422804014327 / bw), dim=1)
+        per_sorted = torch.zeros(len(p), dtype=torch.float64).index_add(0, on[:, 1], kde)
         pdf = per_sorted[torch.tensor(nbh.neighbors[:, 0]).long()]
+        paths.append((u, 1.0 / (bw * radius), order[on[:, 0]], order[on[:, 1]], True))
         mx = torch.zeros(len(ctr), dtype=torch.float64).scatter_reduce(0, ids[:, 1], pdf, "amax",
                                                                        include_self=False)
         rel = (pdf / mx[ids[:, 1]]).reshape(-1, 1)
         cur = torch.relu(rel @ f64(conv.pdf_weights_1) + f64(conv.pdf_biases_1))
         cur = cur @ f64(conv.pdf_weights_2) + f64(conv.pdf_biases_2)
-        hid = torch.nn.functional.elu((p[ids[:, 0]] - q[ids[:, 1]]) @ f64(conv.weights) +
-                                      f64(conv.biases))
+        diff = p[ids[:, 0]] - q[ids[:, 1]]
+        diff.retain_grad()
+        paths.append((diff, 1.0, ids[:, 0], ids[:, 1]))
+        hid = torch.nn.functional.elu(diff @ f64(conv.weights) + f64(conv.biases))
         ref = project(hid / cur) @ f64(conv.final_weights)
     else:
         deform = layer.endswith("deformable")
@@ -1107,6 +1128,8 @@ def test_kpconv_and_pointconv_gradient_with_respect_to_points(oracle, layer):
         out = conv(dev(feat), cin, cout, radius, kernel_influence_dist=sigma * radius)
         tkp = torch.tensor(kp.astype(np.float64) * 0.75)
         diff = (p[ids[:, 0]] - q[ids[:, 1]]) / radius
+        diff.retain_grad()
+        paths.append((diff, 1.0 / radius, ids[:, 0], ids[:, 1]))
 
         def correlation(offsets):
             delta = diff[:, None, :] - tkp[None] - (0 if offsets is None else offsets[ids[:, 1]])
@@ -1125,6 +1148,15 @@ def test_kpconv_and_pointconv_gradient_with_respect_to_points(oracle, layer):
     (ref * torch.tensor(up.astype(np.float64))).sum().backward()
     normwise(tpts.grad.cpu().numpy(), p.grad.numpy(), tol=1e-5)
     normwise(tctr.grad.cpu().numpy(), q.grad.numpy(), tol=1e-5)
+    # per coordinate, against the sum of the absolute per-pair terms of its signed sum.  The
+    # kernel-point terms carry a condition number of their own (the unit vector delta / dist of
+    # a pair close to a kernel point amplifies the rounding of delta), which this magnitude
+    # does not contain: 5e-5 there (1.9e-5 and 4.2e-5 measured), 1e-5 for PointConv.
+    mag_p, mag_q = _point_gradient_magnitude(
+        len(pts), [(t.grad * scale, a, b, *same) for t, scale, a, b, *same in paths], len(ctr))
+    tol = 1e-5 if layer == "pointconv" else 5e-5
+    elementwise(tpts.grad.cpu().numpy(), p.grad.numpy(), mag_p.numpy(), tol=tol)
+    elementwise(tctr.grad.cpu().numpy(), q.grad.numpy(), mag_q.numpy(), tol=tol)
 
 
 @pytest.mark.parametrize("layer", ["mcconv", "kpconv", "pointconv", "pool"])
