@@ -32,6 +32,17 @@ def elementwise(got, expect, mag, tol=1e-5):
         (err / np.maximum(mag, 1e-300)).max(), int(bad.sum()), err.size)
 
 
+def _leaky_basis_magnitude(diff, pdf, w, b):
+    """Magnitude of the rounding error of one-layer leaky-ReLU basis values
+    act(diff . w + b) / pdf: the slope carries the error of the pre-activation (sum of the
+    absolute values of its terms), the value itself its own rounding."""
+    z = diff.astype(np.float64) @ np.asarray(w, np.float64)[0] + np.asarray(b, np.float64).reshape(-1)
+    mz = np.abs(diff).astype(np.float64) @ np.abs(np.asarray(w, np.float64)[0]) + \
+        np.abs(np.asarray(b, np.float64).reshape(-1))
+    slope = np.where(z > 0, 1.0, 0.2)
+    return (slope * mz + np.abs(slope * z)) / np.asarray(pdf, np.float64).reshape(-1, 1)
+
+
 def _setup(oracle, rng, n=3000, n_out=800, batch=2, radius=0.15):
     pts = rng.random((n, 3)).astype(np.float32)
     bids = np.sort(rng.integers(0, batch, n)).astype(np.int32)
@@ -643,6 +654,14 @@ def test_three_level_mcconv_network_matches_oracle(oracle):
         out = conv(feat, hier[level], hier[level + 1], float(conv_r), bandwidth=0.2)
         assert np.array_equal(hier[level + 1]._points.cpu().numpy(), nxt_pts)
         normwise(out.detach().cpu().numpy(), expect, tol=1e-5)
+        # elementwise, against the sum of the absolute values of every entry's terms
+        ids = cn.original_neigh_ids
+        diff = (cur_pts[ids[:, 0]] - nxt_pts[ids[:, 1]]) / conv_r
+        bmag = _leaky_basis_magnitude(diff, pdf, w, b)
+        pmag = oracle.basis_proj(bmag.astype(np.float32), np.abs(feat_ref).astype(np.float32), ids,
+                                 cn.ranges)
+        elementwise(out.detach().cpu().numpy(), expect,
+                    pmag.reshape(len(nxt_pts), -1) @ np.abs(wo[0].astype(np.float64)))
         # feed the oracle's (float32-rounded) result to both sides of the next level
         feat_ref = np.maximum(expect, 0.0)
         feat = dev(feat_ref.astype(np.float32))
@@ -687,6 +706,9 @@ def test_projection_runs_with_empty_and_crowded_centres(oracle, d, c, n_out, rad
             dev(pdf), 1)
     out = layers._mc_project(*args)
     normwise(out.cpu().numpy(), expect)
+    bmag = _leaky_basis_magnitude(diff, pdf, w, b)
+    elementwise(out.cpu().numpy(), expect,
+                oracle.basis_proj(bmag.astype(np.float32), np.abs(feat), ids, nbh.ranges))
     assert float(out[dev(far)].abs().max()) == 0.0
     rows = rng.permutation(n_out).astype(np.int32)
     moved = layers._mc_project(*args, out_rows=dev(rows))
