@@ -718,8 +718,9 @@ def test_projection_runs_with_empty_and_crowded_centres(oracle, d, c, n_out, rad
 def test_mcconv_layer_at_full_scene_size():
     """The benchmark configuration at its real size (8 clouds, 763 k points, 28 M
     pairs, 64 -> 64 channels): rows of the output and of the feature gradient at
-    sampled points against float64 numpy on the layer's own pair table and
-    densities (whose integer parity is pinned elsewhere), and two properties over
+    sampled points against float64 on the layer's own pair table and densities (whose
+    integer parity is pinned elsewhere), every entry within 1e-5 of the sum of the
+    absolute values of its terms, and two properties over
     the whole tensors: linearity in the features and <up, conv(x)> == <dfeat, x>."""
     from tensorflow_graphics_point_clouds_amd import layers, pc, synthetic
     cfg = synthetic.config3()
@@ -764,8 +765,11 @@ def test_mcconv_layer_at_full_scene_size():
     for centre, a, e in zip(picks.tolist(), starts.tolist(), ranges[picks].tolist()):
         seg = torch.arange(a, e, device="cuda")
         assert bool((ids[seg, 1] == centre).all())
-        proj = torch.einsum("mc,mk->ck", xs[ids[seg, 0]], basis_of(seg)).reshape(1, -1)
-        normwise(out[centre].detach().cpu().numpy(), (proj @ final).cpu().numpy()[0], tol=1e-5)
+        bas = basis_of(seg)
+        proj = torch.einsum("mc,mk->ck", xs[ids[seg, 0]], bas).reshape(1, -1)
+        pmag = torch.einsum("mc,mk->ck", xs[ids[seg, 0]].abs(), bas.abs()).reshape(1, -1)
+        elementwise(out[centre].detach().cpu().numpy(), (proj @ final).cpu().numpy()[0],
+                    (pmag @ final.abs()).cpu().numpy()[0])
     # the feature gradient of point j collects the pairs (j, i); the pairs of the
     # self-neighbourhood are symmetric, so they are found through j's own segment
     pair_key = ids[:, 0] * n + ids[:, 1]
@@ -778,8 +782,11 @@ def test_mcconv_layer_at_full_scene_size():
         seg = order[pos]
         assert bool((ids[seg, 0] == j).all()) and bool((ids[seg, 1] == centres).all())
         dproj = torch.einsum("mf,ckf->mck", ups[centres], w3)         # [len, C, 16]
-        expect = torch.einsum("mck,mk->c", dproj, basis_of(seg))
-        normwise(dfeat[j].cpu().numpy(), expect.cpu().numpy(), tol=1e-5)
+        bas = basis_of(seg)
+        expect = torch.einsum("mck,mk->c", dproj, bas)
+        mag = torch.einsum("mck,mk->c", torch.einsum("mf,ckf->mck", ups[centres].abs(), w3.abs()),
+                           bas.abs())
+        elementwise(dfeat[j].cpu().numpy(), expect.cpu().numpy(), mag.cpu().numpy())
 
 
 @pytest.mark.parametrize("layer", ["mcconv", "kpconv", "pointconv"])
@@ -856,6 +863,20 @@ def test_fused_layers_in_two_dimensions(layer):
     normwise(tfeat.grad.cpu().numpy(), x.grad.numpy(), tol=1e-5)
     for name, t in ref_params.items():
         normwise(getattr(conv, name).grad.cpu().numpy(), t.grad.numpy(), tol=1e-5)
+    # output, feature gradient and final-weight gradient elementwise: the same sums over the
+    # absolute values of their terms (the basis values enter with their own magnitude)
+    mx = x.detach().abs().requires_grad_(True)
+    mfinal = final.detach().abs().requires_grad_(True)
+    mproj = torch.zeros(n_out, c_in, basis.shape[1], dtype=torch.float64).index_add(
+        0, ids[:, 1], mx[ids[:, 0]][:, :, None] * basis.detach().abs()[:, None, :])
+    mout = mproj.reshape(n_out, -1) @ mfinal.reshape(-1, c_out)
+    elementwise(out.detach().cpu().numpy(), ref.detach().numpy(), mout.detach().numpy())
+    gx, gfinal = torch.autograd.grad((mout * torch.tensor(np.abs(up).astype(np.float64))).sum(),
+                                     [mx, mfinal])
+    elementwise(tfeat.grad.cpu().numpy(), x.grad.numpy(), gx.numpy())
+    fname = "weights" if layer == "kpconv" else "final_weights"
+    elementwise(getattr(conv, fname).grad.cpu().numpy().reshape(gfinal.shape),
+                ref_params[fname].grad.numpy().reshape(gfinal.shape), gfinal.numpy())
 
 
 def test_mcconv_step_replays_from_a_captured_graph():
