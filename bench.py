@@ -534,7 +534,9 @@ def per_op_times(torch, pc, layers, synthetic, _lib, radius=0.04, reps=5):
         g = torch.ones(N, device="cuda")
         pts = grid._sorted_points
         from tensorflow_graphics_point_clouds_amd import tfg_custom_ops as tfg
-        tfg.compute_pdf_pt_grads(pts, nbh._neighbors, nbh._samples_neigh_ranges,
+        # a table that find_neighbors reported as an untruncated self-neighbourhood takes the
+        # symmetric kernel by itself: the general one is timed on a view of the same table
+        tfg.compute_pdf_pt_grads(pts, nbh._neighbors.view(-1, 2), nbh._samples_neigh_ranges,
                                  torch.full((3,), 5.0, device="cuda"), nbh._inv_radii, g, 0)
         tfg.compute_pdf_pt_grads(pts, nbh._neighbors, nbh._samples_neigh_ranges,
                                  torch.full((3,), 5.0, device="cuda"), nbh._inv_radii, g, 0,

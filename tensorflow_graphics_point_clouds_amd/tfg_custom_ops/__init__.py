@@ -77,13 +77,13 @@ def find_neighbors(samples, samples_batch_ids, points, point_keys, grid_acc_ds, 
     m = int(total[0])
     symmetric = int(total[1]) == 0 and int(total[2]) == 1
     neighbors = torch.empty((m, 2), dtype=_I32, device=dev)
-    if symmetric:
-        _remember_symmetric(neighbors)
     _lib.call("find_neighbors_fill", stream(), i64(ns), cint(nd), ptr(samples, _F32), ptr(samples_batch_ids, _I32),
         i64(points.shape[0]), ptr(points, _F32), ptr(point_keys, _I64), ptr(grid_acc_ds, _I32),
         ptr(num_cells, _I32), ptr(scaled_aabb_min, _F32), ptr(inv_cell_sizes, _F32),
         ptr(inv_radii, _F32), cint(max_neighs), ptr(ws), _lib.csize(ws.numel()), ptr(ranges),
         i64(m), ptr(neighbors))
+    if symmetric:
+        _remember_symmetric(neighbors)
     return ranges, neighbors
 
 
@@ -128,16 +128,20 @@ _symmetric_tables = {}
 
 
 def _remember_symmetric(neighbors):
+    """To be called once the table has been filled: its version counter then only moves if
+    somebody writes to the tensor in place, which voids the record."""
     import weakref
     key = id(neighbors)
-    _symmetric_tables[key] = weakref.ref(neighbors, lambda _, k=key: _symmetric_tables.pop(k, None))
+    _symmetric_tables[key] = (weakref.ref(neighbors, lambda _, k=key: _symmetric_tables.pop(k, None)),
+                              neighbors._version)
 
 
 def is_symmetric_table(neighbors):
     """True for a pair table that `find_neighbors` returned for the points as their own
-    centres without cutting any neighbourhood at max_neighs."""
-    ref = _symmetric_tables.get(id(neighbors))
-    return ref is not None and ref() is neighbors
+    centres without cutting any neighbourhood at max_neighs, and that has not been written
+    to since."""
+    entry = _symmetric_tables.get(id(neighbors))
+    return entry is not None and entry[0]() is neighbors and entry[1] == neighbors._version
 
 
 def compute_pdf_pt_grads(points, neighbors, sample_neigh_indices, inv_bandwidth, inv_radii,

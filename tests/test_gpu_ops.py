@@ -229,6 +229,12 @@ def test_find_neighbors_reports_symmetric_tables(ops, oracle):
         ranges, nbrs = ops.find_neighbors(centres, sb, sp, *args, limit)
         assert ops.is_symmetric_table(nbrs) == expect, (limit, same)
         assert not ops.is_symmetric_table(nbrs.clone())
+        if expect:          # an in-place write voids the record
+            other = nbrs.clone()
+            ranges2, edited = ops.find_neighbors(centres, sb, sp, *args, limit)
+            assert ops.is_symmetric_table(edited)
+            edited[0, 0] = edited[0, 0]
+            assert not ops.is_symmetric_table(edited) and torch.equal(edited, other)
         nbh = oracle.Neighborhood(g, 0.15, max_neighbors=limit)
         assert np.array_equal(nbrs.cpu().numpy(), nbh.neighbors)
         for mode in (0, 1):
