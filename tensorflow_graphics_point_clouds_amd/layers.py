@@ -205,9 +205,15 @@ def _final_product(x, w):
     # Weights beyond the registers of a block of wavefronts (R * F > 65536) take the tiled
     # product, which reads both operands along the reduction: w is handed over transposed
     # (a copy of at most a few MB).  Only when its 128-row tiles give every compute unit
-    # one; smaller inputs take the register-resident product in blocks of w.
-    if r * f > _TILED_ABOVE and L.mccnn_final_product_wt_supported(cint(r), cint(f)) and \
-            _tiles(x.shape[0], f) >= _compute_units(x.device):
+    # one; smaller inputs take the register-resident product in blocks of w.  With the dense
+    # products on the bf16 pipe the tiled kernel is also the faster one for smaller weights
+    # once there are one and a half tiles per compute unit ([763 063, 1024] x [1024, 64]:
+    # 0.82 against 0.93 ms inside the layer step; [30 000, 1024] x [1024, 64]: 0.087 against
+    # 0.049 ms, which is why the register-resident float32 kernel keeps the small inputs).
+    tiles, units = _tiles(x.shape[0], f), _compute_units(x.device)
+    if L.mccnn_final_product_wt_supported(cint(r), cint(f)) and (
+            (r * f > _TILED_ABOVE and tiles >= units) or
+            (L.mccnn_split_products_enabled() and 2 * tiles >= 3 * units)):
         _lib.call("final_product_wt", stream(), i64(x.shape[0]), cint(r), ptr(x, _F32), cint(f),
                   ptr(w.t().contiguous(), _F32), ptr(None), ptr(out), timed_as="final_product")
         return out
