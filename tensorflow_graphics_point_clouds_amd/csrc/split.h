@@ -23,18 +23,37 @@ struct Split8 {
   v8bf p[3];
 };
 
+// Two values at a time: one packed conversion per part (v_cvt_pk_bf16_f32, round to nearest
+// even) and the float value of each half of the packed word from a shift or a mask --
+// 5.5 vector instructions per value, against 7.5 when every value is converted on its own.
+typedef float v2f __attribute__((ext_vector_type(2)));
+typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ v2f widen2(v2bf packed) {
+  const unsigned u = __builtin_bit_cast(unsigned, packed);
+  return v2f{__uint_as_float(u << 16), __uint_as_float(u & 0xffff0000u)};
+}
+
 __device__ __forceinline__ Split8 split8(const v4f &lo, const v4f &hi) {
   Split8 s;
+  unsigned w[3][4];
 #pragma unroll
-  for (int e = 0; e < 8; ++e) {
-    const float x = e < 4 ? lo[e & 3] : hi[e & 3];
-    const __bf16 a = (__bf16)x;
-    const float r1 = x - (float)a;
-    const __bf16 b = (__bf16)r1;
-    const float r2 = r1 - (float)b;
-    s.p[0][e] = a;
-    s.p[1][e] = b;
-    s.p[2][e] = (__bf16)r2;
+  for (int e = 0; e < 4; ++e) {
+    const v2f x = e < 2 ? v2f{lo[2 * e], lo[2 * e + 1]} : v2f{hi[2 * e - 4], hi[2 * e - 3]};
+    const v2bf a = __builtin_convertvector(x, v2bf);
+    const v2f r1 = x - widen2(a);
+    const v2bf b = __builtin_convertvector(r1, v2bf);
+    const v2f r2 = r1 - widen2(b);
+    const v2bf c = __builtin_convertvector(r2, v2bf);
+    w[0][e] = __builtin_bit_cast(unsigned, a);
+    w[1][e] = __builtin_bit_cast(unsigned, b);
+    w[2][e] = __builtin_bit_cast(unsigned, c);
+  }
+#pragma unroll
+  for (int q = 0; q < 3; ++q) {
+    typedef unsigned v4u __attribute__((ext_vector_type(4)));
+    const v4u packed = {w[q][0], w[q][1], w[q][2], w[q][3]};
+    s.p[q] = __builtin_bit_cast(v8bf, packed);
   }
   return s;
 }
