@@ -821,6 +821,20 @@ def main():
     roof["step_flops"] = step_flops
     roof["step_matrix_TFLOPs"] = round(step_flops / ms_per_step / 1e9, 1)
     roof["step_matrix_frac"] = round(step_flops / ms_per_step / 1e9 / FP32_MATRIX_PEAK_TFLOPS, 4)
+    # what this box's HBM delivers to a plain device-to-device copy of 1 GiB (2^30 bytes read and
+    # 2^30 written per copy): a measured ceiling beside the published 8 TB/s that `peak` uses
+    src = torch.ones(1 << 28, dtype=torch.float32, device="cuda")
+    dst = torch.empty_like(src)
+    for _ in range(2):
+        dst.copy_(src)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(5):
+        dst.copy_(src)
+    e1.record()
+    torch.cuda.synchronize()
+    roof["measured_copy_GBps"] = round(5 * 2.0 * (1 << 30) / (e0.elapsed_time(e1) * 1e-3) / 1e9, 1)
+    del src, dst
 
     result = {
         "metric": "MCConv layer fwd+bwd points/sec", "value": N / (ms_per_step * 1e-3),
