@@ -193,6 +193,23 @@ int mccnn_find_neighbors_count_facts(
     int max_neighs, void *workspace, size_t workspace_bytes,
     int32_t *ranges_out, int64_t *num_neighbors_out_host,
     int64_t *facts_out_host);
+/* The search without a host round trip, for callers that enqueue a whole step (or record it
+ * in a HIP graph): count, scan and fill in one call on the stream.  The pair table has room
+ * for `capacity` rows; pairs beyond it are dropped, ranges_out holds the true end offsets,
+ * count_out_device[0] the true number of pairs and count_out_device[1] 1 if it exceeds the
+ * capacity (the caller checks that flag when it next reads from the device, e.g. once per
+ * step).  Rows [0, min(count, capacity)) equal those of the _count / _fill pair; the rest of
+ * the table is not written.  Same workspace as _count.  No counterpart in the reference,
+ * whose op returns a tensor of the exact size (find_neighbors_ops.cpp:217-259). */
+int mccnn_find_neighbors_bounded(
+    mccnn_stream_t stream, int64_t num_samples, int num_dims,
+    const float *samples, const int32_t *sample_batch_ids, int64_t num_pts,
+    const float *points, const int64_t *point_keys, int ds_batch, int ds_nx,
+    int ds_ny, const int32_t *grid_ds, const int32_t *num_cells,
+    const float *scaled_aabb_min, const float *inv_cell_sizes,
+    const float *inv_radii, int max_neighs, void *workspace,
+    size_t workspace_bytes, int64_t capacity, int32_t *ranges_out,
+    int32_t *neighbors_out, int64_t *count_out_device);
 int mccnn_find_neighbors_fill(
     mccnn_stream_t stream, int64_t num_samples, int num_dims,
     const float *samples, const int32_t *sample_batch_ids, int64_t num_pts,

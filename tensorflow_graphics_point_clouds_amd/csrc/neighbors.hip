@@ -172,7 +172,7 @@ __global__ void __launch_bounds__(kNbrThreads) nbr_visit_kernel(
     int64_t ns, const float *__restrict__ samples, const float *__restrict__ pts,
     const int2 *__restrict__ ranges, const float *__restrict__ inv_radii, int max_neighs,
     int *__restrict__ counts, const int *__restrict__ ends, int2 *__restrict__ nbrs,
-    int64_t *__restrict__ truncated = nullptr) {
+    int64_t *__restrict__ truncated = nullptr, int64_t capacity = ((int64_t)1 << 62)) {
   constexpr int R = OffsetInfo<D>::count();
   const int sub = threadIdx.x & (kGroup - 1);
   const int lane = lane_id();
@@ -203,7 +203,8 @@ __global__ void __launch_bounds__(kNbrThreads) nbr_visit_kernel(
         if (kFill) {
           const uint64_t hits = __ballot(hit) & group_mask;
           const int slot = found + __popcll(hits & below_mask);
-          if (hit && slot < limit) nbrs[start + slot] = make_int2(j, (int)c);
+          if (hit && slot < limit && start + slot < capacity)
+            nbrs[start + slot] = make_int2(j, (int)c);
           found += __popcll(hits);
         } else {
           found += hit ? 1 : 0;
@@ -294,7 +295,9 @@ static int find_neighbors_count_impl(
     const int32_t *num_cells, int aabb_dims, const float *scaled_aabb_min, int inv_cell_sizes_len,
     const float *inv_cell_sizes, int inv_radii_len, const float *inv_radii, int max_neighs,
     void *workspace, size_t workspace_bytes, int32_t *ranges_out,
-    int64_t *num_neighbors_out_host, int64_t *facts_out_host) {
+    int64_t *num_neighbors_out_host, int64_t *facts_out_host, bool to_host = true) {
+  int64_t unused_total = 0;
+  if (!to_host) num_neighbors_out_host = &unused_total;   // the total stays in the workspace
   MCCNN_REQUIRE(valid_dims(num_dims), "FindNeighbors expects a valid number of dimensions");
   MCCNN_REQUIRE(num_cells_len == num_dims,
                 "FindNeighbors expects a number of dimensions in num_cells equal to the number of "
@@ -361,6 +364,7 @@ static int find_neighbors_count_impl(
   MCCNN_LAUNCH_CHECK();
   int rc = inclusive_scan_i32(s, num_samples, ranges_out, w.scan_scratch, w.total);
   if (rc != MCCNN_OK) return rc;
+  if (!to_host) return MCCNN_OK;
   MCCNN_HIP_CHECK(hipMemcpyAsync(num_neighbors_out_host, w.total, sizeof(int64_t),
                                  hipMemcpyDeviceToHost, s));
   if (truncated)
@@ -433,6 +437,50 @@ extern "C" int mccnn_find_neighbors_fill(
                                                 num_samples, samples, points,
                                                 (const int2 *)w.ranges, inv_radii, max_neighs,
                                                 (int *)nullptr, ranges, (int2 *)neighbors_out));
+  MCCNN_LAUNCH_CHECK();
+  return MCCNN_OK;
+}
+
+// count_out[0] = pairs found, count_out[1] = 1 if they do not fit the capacity
+__global__ void publish_neighbor_count_kernel(const int64_t *__restrict__ total, int64_t capacity,
+                                              int64_t *__restrict__ count_out) {
+  if (threadIdx.x == 0 && blockIdx.x == 0) {
+    count_out[0] = *total;
+    count_out[1] = *total > capacity ? 1 : 0;
+  }
+}
+
+extern "C" int mccnn_find_neighbors_bounded(
+    mccnn_stream_t stream, int64_t num_samples, int num_dims, const float *samples,
+    const int32_t *sample_batch_ids, int64_t num_pts, const float *points,
+    const int64_t *point_keys, int ds_batch, int ds_nx, int ds_ny, const int32_t *grid_ds,
+    const int32_t *num_cells, const float *scaled_aabb_min, const float *inv_cell_sizes,
+    const float *inv_radii, int max_neighs, void *workspace, size_t workspace_bytes,
+    int64_t capacity, int32_t *ranges_out, int32_t *neighbors_out, int64_t *count_out_device) {
+  MCCNN_REQUIRE(capacity >= 0 && capacity < ((int64_t)1 << 31),
+                "find_neighbors_bounded expects a capacity in [0, 2^31)");
+  MCCNN_REQUIRE(count_out_device && (capacity == 0 || neighbors_out),
+                "find_neighbors_bounded received a null output");
+  int rc = find_neighbors_count_impl(
+      stream, num_samples, num_dims, samples, num_samples, sample_batch_ids, num_pts, num_dims,
+      points, num_pts, point_keys, 4, ds_batch, ds_nx, ds_ny, 2, grid_ds, num_dims, num_cells,
+      num_dims, scaled_aabb_min, num_dims, inv_cell_sizes, num_dims, inv_radii, max_neighs,
+      workspace, workspace_bytes, ranges_out, nullptr, nullptr, false);
+  if (rc != MCCNN_OK) return rc;
+  hipStream_t s = as_stream(stream);
+  if (num_samples == 0) return fill_zero(s, count_out_device, 2 * sizeof(int64_t));
+  const NbrWorkspace w = carve_nbr_workspace(workspace, num_dims, num_samples);
+  hipLaunchKernelGGL(publish_neighbor_count_kernel, dim3(1), dim3(64), 0, s, w.total, capacity,
+                     count_out_device);
+  MCCNN_LAUNCH_CHECK();
+  if (capacity == 0) return MCCNN_OK;
+  const unsigned grid = blocks_for(num_samples, kCentresPerBlock);
+  MCCNN_DIM_SWITCH(num_dims, hipLaunchKernelGGL((nbr_visit_kernel<D, true>), dim3(grid),
+                                                dim3(kNbrThreads), 0, s, num_samples, samples,
+                                                points, (const int2 *)w.ranges, inv_radii,
+                                                max_neighs, (int *)nullptr, ranges_out,
+                                                (int2 *)neighbors_out, (int64_t *)nullptr,
+                                                capacity));
   MCCNN_LAUNCH_CHECK();
   return MCCNN_OK;
 }

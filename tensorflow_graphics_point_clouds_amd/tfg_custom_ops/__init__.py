@@ -87,6 +87,34 @@ def find_neighbors(samples, samples_batch_ids, points, point_keys, grid_acc_ds, 
     return ranges, neighbors
 
 
+def find_neighbors_bounded(samples, samples_batch_ids, points, point_keys, grid_acc_ds, num_cells,
+                           scaled_aabb_min, inv_cell_sizes, inv_radii, max_neighs, capacity,
+                           out=None):
+    """find_neighbors without a host round trip: (ranges [N_out], neighbors [capacity, 2],
+    count [2] = (pairs found, 1 if they exceed the capacity), all on the device).  Rows of the
+    table past the count are not written.  `out` = (ranges, neighbors, count) reuses tensors
+    of a previous call, so that the call allocates nothing and can be recorded in a HIP
+    graph."""
+    ns, nd = samples.shape[0], _dim(samples, 1)
+    dev = samples.device
+    L = _lib.lib()
+    if out is None:
+        out = (torch.empty(ns, dtype=_I32, device=dev),
+               torch.empty((capacity, 2), dtype=_I32, device=dev),
+               torch.zeros(2, dtype=_I64, device=dev),
+               torch.empty(max(int(L.mccnn_find_neighbors_workspace_bytes(cint(nd), i64(ns))), 1),
+                           dtype=torch.uint8, device=dev))
+    ranges, neighbors, count, ws = out
+    _lib.call("find_neighbors_bounded", stream(), i64(ns), cint(nd), ptr(samples, _F32),
+              ptr(samples_batch_ids, _I32), i64(points.shape[0]), ptr(points, _F32),
+              ptr(point_keys, _I64), cint(_dim(grid_acc_ds, 0)), cint(_dim(grid_acc_ds, 1)),
+              cint(_dim(grid_acc_ds, 2)), ptr(grid_acc_ds, _I32), ptr(num_cells, _I32),
+              ptr(scaled_aabb_min, _F32), ptr(inv_cell_sizes, _F32), ptr(inv_radii, _F32),
+              cint(max_neighs), ptr(ws), _lib.csize(ws.numel()), i64(neighbors.shape[0]),
+              ptr(ranges), ptr(neighbors), ptr(count))
+    return out
+
+
 def sampling(points, batch_ids, point_keys, num_cells, neighbors, sample_neigh_indices, mode):
     """Sampling (sampling_ops.cpp:33-53): mode 0 Poisson disk, mode 1 cell average.
     -> (sample_pts [S, D], sample_batch_ids [S], sample_indices [S])."""

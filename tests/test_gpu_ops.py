@@ -182,6 +182,61 @@ def test_neighbors_clustered_cloud(ops, oracle):
     assert np.array_equal(nbrs.cpu().numpy(), nbh.neighbors)
 
 
+def test_find_neighbors_bounded_matches_two_phase_and_replays_from_a_graph(ops, oracle):
+    """The search without a host round trip (count, scan and fill enqueued in one call, the pair
+    count left on the device): the first min(count, capacity) rows and the end offsets equal the
+    two-phase op bit for bit, an insufficient capacity raises the flag, and the call -- which
+    allocates nothing when given its outputs -- replays from a captured HIP graph on changed
+    centres with eager calls in between, every replay equal to the two-phase result."""
+    rng = np.random.default_rng(123)
+    pts, bids = _cloud(rng, 3, 5000, 3)
+    g = oracle.Grid(pts, bids, 3, 0.1)
+    grid_args = (dev(g.sorted_points), dev(g.sorted_keys), dev(g.get_ds()), dev(g.num_cells),
+                 dev(g.scaled_aabb_min), dev(g.inv_cell_sizes),
+                 dev(np.full(3, 1 / np.float32(0.1), np.float32)))
+
+    def centres(seed):
+        r = np.random.default_rng(seed)
+        c, cb = _cloud(r, 3, 1200, 3, scale=1.1)
+        return (c - 0.05).astype(np.float32), cb
+
+    ctr, cb = centres(1)
+    t_ctr, t_cb = dev(ctr), dev(cb)
+    for limit in (0, 5):
+        ranges, nbrs = ops.find_neighbors(t_ctr, t_cb, *grid_args, limit)
+        m = nbrs.shape[0]
+        nbh = oracle.Neighborhood(g, 0.1, ctr, cb, max_neighbors=limit)
+        assert np.array_equal(nbrs.cpu().numpy(), nbh.neighbors)
+        for capacity in (m + 1000, m, m - 7, 0):
+            r2, n2, count, _ = ops.find_neighbors_bounded(t_ctr, t_cb, *grid_args, limit, capacity)
+            assert count.tolist() == [m, int(m > capacity)]
+            assert torch.equal(r2, ranges)
+            keep = min(m, capacity)
+            assert torch.equal(n2[:keep], nbrs[:keep])
+    # graph: outputs allocated once, centres rewritten in place between replays
+    capacity = m + 4000
+    out = ops.find_neighbors_bounded(t_ctr, t_cb, *grid_args, 0, capacity)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        ops.find_neighbors_bounded(t_ctr, t_cb, *grid_args, 0, capacity, out=out)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        ops.find_neighbors_bounded(t_ctr, t_cb, *grid_args, 0, capacity, out=out)
+    for seed in (2, 3, 4):
+        ctr2, cb2 = centres(seed)
+        t_ctr.copy_(dev(ctr2))
+        t_cb.copy_(dev(cb2))
+        graph.replay()
+        torch.cuda.synchronize()
+        ranges, nbrs = ops.find_neighbors(t_ctr, t_cb, *grid_args, 0)     # eager work in between
+        count = out[2].tolist()
+        assert count == [nbrs.shape[0], 0]
+        assert torch.equal(out[0], ranges) and torch.equal(out[1][:count[0]], nbrs)
+
+
 # -------------------------------------------------------------------- pdf ----
 
 @pytest.mark.parametrize("d", [2, 3, 4])
