@@ -32,7 +32,7 @@ def log(*a):
 
 def op_bytes(name, M, N_in, N_out, C, K, D):
     """Operand bytes of one launch of each op (fp32, int32 pair table): every per-pair
-    gather counted at full width, as the survey's formulas do.  On grid-ordered inputs
+    gather counted at full width (a feature row per pair).  On grid-ordered inputs
     most of the gathers are served by L2, so this figure can exceed what HBM moves; it is
     reported as `operand_GBps`, never as a roofline fraction."""
     if name == "basis_proj":
