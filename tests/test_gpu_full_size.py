@@ -64,6 +64,19 @@ def _check_grid_and_self_neighbourhood(oracle, points, batch_ids, batch_size, ra
     want[:, 0] = dev(g.sorted_indices)[want[:, 0].long()]
     assert torch.equal(got._original_neigh_ids, want), "pair table with original ids"
     del want
+    # the search without a host round trip: same end offsets and rows, count on the device
+    from tensorflow_graphics_point_clouds_amd import tfg_custom_ops as ops
+    m = len(nbh.neighbors)
+    for capacity in (m + 3, m - 1):
+        ranges, table, count, _ = ops.find_neighbors_bounded(
+            grid._sorted_points, grid._sorted_batch_ids, grid._sorted_points, grid._sorted_keys,
+            grid.get_DS(), grid._num_cells, grid._scaled_aabb_min, grid._inv_cell_sizes,
+            got._inv_radii, 0, capacity)
+        assert count.tolist() == [m, int(m > capacity)]
+        assert torch.equal(ranges, got._samples_neigh_ranges), "bounded search: ranges"
+        keep = min(m, capacity)
+        assert torch.equal(table[:keep], got._neighbors[:keep]), "bounded search: pair table"
+        del ranges, table
     if poisson:
         pts, bids, sel = oracle.sampling(g.sorted_points, g.sorted_batch_ids, g.sorted_keys,
                                          g.num_cells, nbh.neighbors, nbh.ranges, 0)
