@@ -272,8 +272,8 @@ int launch_nt_split(hipStream_t s, int64_t n, int F, const float *x, int R, cons
 
 // out[out_rows[n] or n, :] = x[n, :] * w for x [N, R] and the weights given transposed,
 // wt [F, R]: the tiled product on the bf16 pipe.  A block of four wavefronts owns a BM x BN
-// tile of the output (128 x 128 or 256 x 64), every wavefront 64 x 64 of it as 2 x 2
-// accumulator tiles of 32 x 32, and walks the reduction in chunks of 32.  The chunk of x and
+// tile of the output (128 x 128, 256 x 128 or 256 x 64), every wavefront 64 x 64 or 128 x 64
+// of it as accumulator tiles of 32 x 32, and walks the reduction in chunks of 32.  The chunk of x and
 // of wt for the next step is fetched into registers while the current one is multiplied;
 // the thread that fetched eight consecutive values splits them once and parks the three
 // bfloat16 parts as 16-byte vectors in operand order ([part][group of 8 along the
@@ -282,12 +282,12 @@ int launch_nt_split(hipStream_t s, int64_t n, int F, const float *x, int R, cons
 // matrix operand is one 16-byte LDS read.  x is read once per column block; wt comes from L2.
 constexpr int kSplitK = 32, kSplitGroups = kSplitK / 8, kSplitThreads = 256;
 
-template <int BN>
+template <int BN, int BM = 16384 / BN>
 __global__ void __launch_bounds__(kSplitThreads) tile_split_kernel(
     int64_t n, int R, int F, const float *__restrict__ x, const float *__restrict__ wt,
     const int *__restrict__ out_rows, float *__restrict__ out) {
-  constexpr int BM = 16384 / BN;
-  constexpr int kWN = BN / 64;
+  constexpr int kWN = BN / 64, kWM = 4 / kWN;      // wavefronts across / down the tile
+  constexpr int kRT = BM / kWM / 32;               // 32-row accumulator tiles per wavefront
   constexpr int kLdA = BM + 4, kLdB = BN + 4;                   // vectors per group
   constexpr int kAItems = BM * kSplitGroups / kSplitThreads;    // (row, group) items per thread
   constexpr int kBItems = BN * kSplitGroups / kSplitThreads;
@@ -300,9 +300,9 @@ __global__ void __launch_bounds__(kSplitThreads) tile_split_kernel(
   const int64_t row0 = (int64_t)(blockIdx.x / col_blocks) * BM;
   const int col0 = (blockIdx.x % col_blocks) * BN;
 
-  v16f acc[2][2];
+  v16f acc[kRT][2];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < kRT; ++i)
 #pragma unroll
     for (int j = 0; j < 2; ++j)
 #pragma unroll
@@ -352,26 +352,28 @@ __global__ void __launch_bounds__(kSplitThreads) tile_split_kernel(
     if (k0 + kSplitK < R) fetch(k0 + kSplitK);
 #pragma unroll
     for (int ks = 0; ks < kSplitK / 16; ++ks) {
-      Split8 a[2], b[2];
+      Split8 a[kRT], b[2];
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
+      for (int q = 0; q < 3; ++q) {
 #pragma unroll
-        for (int q = 0; q < 3; ++q) {
-          a[i].p[q] = a_lds[(q * kSplitGroups + 2 * ks + h) * kLdA + wm * 64 + 32 * i + p];
-          b[i].p[q] = b_lds[(q * kSplitGroups + 2 * ks + h) * kLdB + wn * 64 + 32 * i + p];
-        }
+        for (int i = 0; i < kRT; ++i)
+          a[i].p[q] = a_lds[(q * kSplitGroups + 2 * ks + h) * kLdA + wm * (32 * kRT) + 32 * i + p];
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
+        for (int j = 0; j < 2; ++j)
+          b[j].p[q] = b_lds[(q * kSplitGroups + 2 * ks + h) * kLdB + wn * 64 + 32 * j + p];
+      }
+#pragma unroll
+      for (int i = 0; i < kRT; ++i)
 #pragma unroll
         for (int j = 0; j < 2; ++j) acc[i][j] = mma_split(a[i], b[j], acc[i][j]);
     }
   }
-  // acc[i][j][e]: row row0 + 64 wm + 32 i + (e / 4) * 8 + 4 h + e % 4, column col0 + 64 wn + 32 j + p
+  // acc[i][j][e]: row row0 + 32 kRT wm + 32 i + (e / 4) * 8 + 4 h + e % 4, column col0 + 64 wn + 32 j + p
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < kRT; ++i)
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
-      const int64_t row = row0 + wm * 64 + 32 * i + (e / 4) * 8 + 4 * h + (e % 4);
+      const int64_t row = row0 + wm * (32 * kRT) + 32 * i + (e / 4) * 8 + 4 * h + (e % 4);
       if (row < n) {
         const int64_t orow = out_rows ? out_rows[row] : row;
         float *o = out + orow * F + col0 + wn * 64 + p;
@@ -383,9 +385,19 @@ __global__ void __launch_bounds__(kSplitThreads) tile_split_kernel(
 
 int launch_tile_split(hipStream_t s, int64_t n, int R, const float *x, int F, const float *wt,
                       const int *out_rows, float *out) {
-  const int bn = F % 128 == 0 ? 128 : 64, bm = 16384 / bn;
+  const int bn = F % 128 == 0 ? 128 : 64;
+  // 128 columns: tiles of 256 rows (every wavefront 128 x 64) while they still fill the device
+  // twice over -- the weights' chunk is split once per 256 instead of once per 128 rows
+  // (825 k x 2048 by 2048 x 128: 2.31 against 2.40 ms) --, tiles of 128 rows below that
+  int device = 0, cus = 0;
+  MCCNN_HIP_CHECK(hipGetDevice(&device));
+  MCCNN_HIP_CHECK(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device));
+  const bool tall = bn == 128 && (n + 255) / 256 * (F / 128) >= 2 * (int64_t)cus;
+  const int bm = tall ? 256 : 16384 / bn;
   const dim3 block(kSplitThreads), grid((unsigned)((n + bm - 1) / bm * (F / bn)));
-  if (bn == 128)
+  if (tall)
+    hipLaunchKernelGGL((tile_split_kernel<128, 256>), grid, block, 0, s, n, R, F, x, wt, out_rows, out);
+  else if (bn == 128)
     hipLaunchKernelGGL((tile_split_kernel<128>), grid, block, 0, s, n, R, F, x, wt, out_rows, out);
   else
     hipLaunchKernelGGL((tile_split_kernel<64>), grid, block, 0, s, n, R, F, x, wt, out_rows, out);

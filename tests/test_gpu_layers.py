@@ -564,9 +564,11 @@ def test_final_product_matches_float64(n, r, f):
 
 
 @pytest.mark.parametrize("n,r,f", [(40001, 2048, 128), (70000, 1024, 64), (33000, 512, 192),
-                                   (129, 64, 64), (1, 32, 128), (0, 2048, 128)])
+                                   (129, 64, 64), (1, 32, 128), (0, 2048, 128),
+                                   (131101, 512, 128), (66003, 256, 256)])
 def test_final_product_with_transposed_weights_matches_float64(n, r, f):
-    """The tiled product on wt [F, R] (128 x 128 and 256 x 64 tiles, partial last tiles, row
+    """The tiled product on wt [F, R] (128 x 128 and 256 x 64 tiles, 256 x 128 once those fill
+    the device twice over -- the last two shapes --, partial last tiles, row
     permutation), elementwise against float64 with the magnitude sum |x| |w| (1e-5); equal
     bits on a second call; and the layer-level product, which picks the tiles for the large
     shapes, against the same reference."""
