@@ -99,6 +99,8 @@ def find_neighbors(samples, sample_batch_ids, points, point_keys, grid_ds, num_c
             _ptr(keys), _ptr(ds), _ptr(nc), _ptr(smin), _ptr(ic), _ptr(ir),
             _int(max_neighs))
     m = lib().orc_find_neighbors_count(*args, _ptr(ranges))
+    if m >= 2 ** 31 - 1:        # the int32 end offsets of the op contract have wrapped
+        raise ValueError("find_neighbors: %d pairs do not fit the int32 offsets" % m)
     nbrs = np.empty((m, 2), dtype=np.int32)
     lib().orc_find_neighbors_fill(*args, _ptr(ranges), _ptr(nbrs))
     return ranges, nbrs
