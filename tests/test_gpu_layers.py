@@ -336,15 +336,18 @@ def test_kpconv_forward_backward(oracle, kind, influence, c_in, c_out, transpose
                 pmag.T @ np.abs(up64), tol=tol)
 
 
-@pytest.mark.parametrize("c_in,c_out", [(16, 8), (8, 16), (32, 32)])
+@pytest.mark.parametrize("c_in,c_out", [(16, 8), (8, 16), (32, 32), (16, 16), (8, 32), (8, 8),
+                                        (32, 64), (64, 16), (64, 64)])
 @pytest.mark.parametrize("kind", ["linear", "gaussian"])
 def test_deformable_kpconv_and_regularization(oracle, kind, c_in, c_out):
     """Deformable kernel points (offsets predicted by a rigid convolution) and the
     regularisation loss, forward and backward, against float64 autograd of the
     expressions of KPConv.py:165-232, 317-429 on the oracle's neighbour pairs; foreign
     centres; 16 and 32 input channels take the kernels with the weights in registers, 8
-    the materialising ops.  Normwise 2e-5 for the gradients (non-smooth points of the
-    correlation and of the fitting minimum are handled as the helper describes)."""
+    the materialising ops.  Offsets and output elementwise at 1e-5 of the sum of the
+    absolute values of their terms, the reference evaluated at the layer's own offsets;
+    normwise 1e-5 for the gradients (non-smooth points of the correlation and of the
+    fitting minimum are handled as the helper describes)."""
     from tensorflow_graphics_point_clouds_amd import synthetic
     from tests.deformable_reference import check_deformable_kpconv
     rng = np.random.default_rng(17)
